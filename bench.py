@@ -1,0 +1,156 @@
+"""Benchmark of the ragged paged attention forward on one MI355X.
+
+``python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME]`` runs W untimed and K
+timed forward passes of one synthetic batch (already resident in HBM) and prints ONE JSON line.
+A "step" is one pass of the op over the whole ragged batch.  The default workload is the
+Llama-3-8B-shape decode batch (256 sequences x 1 token, kv 512..8192, 32 q / 8 kv heads,
+head_dim 128, page 16, 160k-page pool); the metric is query tokens per second, with the achieved
+fraction of the HBM roofline of the attention kernel and, beside it, the CPU restatement of the
+reference's XLA path timed on this host on a bounded sample of the same batch.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="decode_llama3_8b")
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
+    ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-parity", action="store_true")
+    return ap.parse_args()
+
+
+def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs):
+    """Runs the CPU oracle on a sample of the batch's sequences: times it and checks the device rows."""
+    import numpy as np
+    import torch
+    from threadpoolctl import threadpool_info
+
+    from ejkernel_amd.workloads import compact_for_host
+    from tests.helpers import err_stats, run_exact, run_strict, to_np
+
+    S = len(batch.q_lens)
+    rng = np.random.default_rng(0)
+    cand = [int(s) for s in rng.permutation(S) if batch.q_lens[s] > 0]
+    if n_seqs <= 0:
+        # about 2e9 key-row-head products per second for the NumPy port; aim at ~10 s
+        budget, n_seqs, acc = 2.0e10, 0, 0.0
+        Hq, D = batch.queries.shape[1], batch.queries.shape[2]
+        for s in cand:
+            rows8 = -(-int(batch.q_lens[s]) // 8) * 8
+            acc += rows8 * float(batch.kv_lens[s]) * Hq * D
+            n_seqs += 1
+            if acc > budget:
+                break
+    ids = sorted(cand[:max(1, n_seqs)])
+    sub = compact_for_host(batch, ids)
+    t0 = time.perf_counter()
+    ref = run_strict(sub)
+    dt = time.perf_counter() - t0
+    rows = sub.total_valid_tokens
+    res = {}
+    if want_parity:
+        got = to_np(out[sub.meta["rows"].to(out.device)])
+        bad = np.isnan(ref[:rows]).any(axis=(1, 2))
+        if bad.any():  # strict oracle NaN rows (window defect of the reference): compare with the float64 form
+            ref = ref.copy()
+            ref[:rows][bad] = run_exact(sub)[:rows][bad]
+        mx, mean = err_stats(got, ref, rows)
+        res["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": rows, "oracle_nan_rows": int(bad.sum()),
+                         "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
+    if want_baseline:
+        threads = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
+        res["cpu_baseline"] = {
+            "value": rows / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
+            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens), "
+                      f"NumPy restatement of the XLA path, {dt:.2f} s",
+        }
+    return res
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build measures one GPU only (the op shards without exchange by sequence or by "
+              "kv head); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    import torch
+
+    from ejkernel_amd import _native
+    from ejkernel_amd.modules import ragged_page_attention
+    from ejkernel_amd.roofline import HBM_PEAK_GBPS, MFMA_BF16_PEAK_TFLOPS, algorithmic_counts
+    from ejkernel_amd.workloads import WORKLOADS, make_workload
+
+    _native.load()  # fail loudly before any timing if the HIP library is missing
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = "cuda:0"
+    batch = make_workload(args.workload, device=dev, scale=args.scale)
+    m = batch.meta
+    counts = algorithmic_counts(batch.q_lens, batch.kv_lens, num_q_heads=m["num_q_heads"],
+                                num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m["page_size"],
+                                sliding_window=batch.sliding_window)
+
+    def step():
+        return ragged_page_attention(*batch.args(), **batch.kwargs())
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()  # the op launches on torch's current stream, the one these events are recorded on
+        out = step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    kernel_ms = sum(ev_ms) / len(ev_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    tokens = counts["tokens"]
+
+    gbps = counts["bytes"] / (kernel_ms * 1e-3) / 1e9
+    tflops = counts["flops"] / (kernel_ms * 1e-3) / 1e12
+    hbm_time = counts["bytes"] / (HBM_PEAK_GBPS * 1e9)
+    mfma_time = counts["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)
+    if hbm_time >= mfma_time:
+        roof = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS}
+    else:
+        roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
+    roof.update({"traffic": None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
+                 "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
+                 "algorithmic_flops": counts["flops"], "tflops": tflops, "gbps": gbps})
+
+    line = {
+        "metric": "ragged paged-attn tokens/s", "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "description": WORKLOADS[args.workload], "scale": args.scale,
+                   "query_tokens": tokens, "num_seqs": len(batch.q_lens), "kv_tokens": int(batch.kv_lens.sum())},
+        "roofline": roof,
+    }
+    if not (args.no_cpu_baseline and args.no_parity):
+        line.update(cpu_sample_and_parity(batch, out, not args.no_cpu_baseline, not args.no_parity, args.cpu_seqs))
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,107 @@
+"""ctypes binding of ``librpa_mi355x.so`` (declared in ``include/rpa_mi355x.h``).
+
+There is no fallback: if the shared library is missing or does not load, importing the
+op fails with an error that says how to build it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from pathlib import Path
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so"
+
+RPA_ABI_VERSION = 1
+RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
+RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
+RPA_FLAG_FORCE_GENERIC = 1
+
+EXPORTED_SYMBOLS = (
+    "rpa_abi_version",
+    "rpa_last_error",
+    "rpa_workspace_bytes",
+    "rpa_workspace_init",
+    "rpa_fwd_launch",
+)
+
+
+class RpaParams(ctypes.Structure):
+    """Field-for-field image of ``struct RpaParams``."""
+
+    _fields_ = [
+        ("queries", ctypes.c_void_p),
+        ("kv_pages", ctypes.c_void_p),
+        ("context_lens", ctypes.c_void_p),
+        ("block_tables", ctypes.c_void_p),
+        ("query_start_loc", ctypes.c_void_p),
+        ("num_seqs", ctypes.c_void_p),
+        ("sinks", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("total_tokens", ctypes.c_int32),
+        ("num_q_heads", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("page_size", ctypes.c_int32),
+        ("num_pages", ctypes.c_int32),
+        ("max_num_seqs", ctypes.c_int32),
+        ("pages_per_seq", ctypes.c_int32),
+        ("num_sinks", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float),
+        ("logits_soft_cap", ctypes.c_float),
+        ("sliding_window", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("compute", ctypes.c_int32),
+        ("num_queries_per_block", ctypes.c_int32),
+        ("num_kv_pages_per_block", ctypes.c_int32),
+        ("num_warps", ctypes.c_int32),
+        ("num_stages", ctypes.c_int32),
+        ("flags", ctypes.c_uint32),
+    ]
+
+
+class NativeLibraryError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the shared library once and declare the prototypes."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not LIB_PATH.exists():
+        raise NativeLibraryError(
+            f"{LIB_PATH} is missing: build it with `python -m ejkernel_amd.build` "
+            "(hipcc, --offload-arch=gfx950). There is no CPU or eager fallback."
+        )
+    try:
+        lib = ctypes.CDLL(str(LIB_PATH))
+    except OSError as e:  # pragma: no cover - depends on the host
+        raise NativeLibraryError(f"cannot load {LIB_PATH}: {e}") from e
+    for name in EXPORTED_SYMBOLS:
+        if not hasattr(lib, name):
+            raise NativeLibraryError(f"{LIB_PATH} does not export {name}")
+    lib.rpa_abi_version.restype = ctypes.c_int
+    lib.rpa_abi_version.argtypes = []
+    lib.rpa_last_error.restype = ctypes.c_char_p
+    lib.rpa_last_error.argtypes = []
+    lib.rpa_workspace_bytes.restype = ctypes.c_uint64
+    lib.rpa_workspace_bytes.argtypes = [ctypes.POINTER(RpaParams)]
+    lib.rpa_workspace_init.restype = ctypes.c_int
+    lib.rpa_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.rpa_fwd_launch.restype = ctypes.c_int
+    lib.rpa_fwd_launch.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
+    if lib.rpa_abi_version() != RPA_ABI_VERSION:
+        raise NativeLibraryError(
+            f"{LIB_PATH} has ABI version {lib.rpa_abi_version()}, this package expects {RPA_ABI_VERSION}: rebuild it"
+        )
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().rpa_last_error().decode("utf-8", "replace")

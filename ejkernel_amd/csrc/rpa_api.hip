@@ -1,0 +1,75 @@
+// C ABI of librpa_mi355x.so: argument validation and kernel selection.
+//
+// Validation mirrors what the reference enforces before its kernels run:
+// ejkernel/kernels/_pallas/tpu/ragged_page_attention/_pallas_impl_fwd.py:177-230
+// (static_validate_inputs) and the named-dimension checks of
+// ejkernel/kernels/_xla/ragged_page_attention/_interface.py:26-47.
+#include <cstdarg>
+#include <cstdio>
+
+#include "rpa_host.h"
+
+namespace rpa {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+static int validate(const RpaParams& p, bool need_pointers) {
+  if (p.total_tokens < 0 || p.num_q_heads <= 0 || p.num_kv_heads <= 0 || p.head_dim <= 0 || p.page_size <= 0 ||
+      p.num_pages <= 0 || p.max_num_seqs <= 0 || p.pages_per_seq <= 0 || p.num_sinks < 0)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "non-positive dimension in RpaParams");
+  if (p.num_q_heads % p.num_kv_heads != 0)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "num_q_heads=%d must be divisible by num_kv_heads=%d", p.num_q_heads,
+                p.num_kv_heads);
+  if (p.sliding_window < 0) return fail(RPA_ERR_INVALID_ARGUMENT, "sliding_window=%d must be positive", p.sliding_window);
+  if (p.dtype != RPA_DTYPE_BF16 && p.dtype != RPA_DTYPE_F32) return fail(RPA_ERR_INVALID_ARGUMENT, "unknown dtype %d", p.dtype);
+  if (p.compute != RPA_COMPUTE_BF16 && p.compute != RPA_COMPUTE_F32)
+    return fail(RPA_ERR_INVALID_ARGUMENT, "unknown compute mode %d", p.compute);
+  if (!(p.softmax_scale == p.softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "softmax_scale is NaN");
+  if (!(p.logits_soft_cap == p.logits_soft_cap)) return fail(RPA_ERR_INVALID_ARGUMENT, "logits_soft_cap is NaN");
+  if (need_pointers) {
+    if (!p.queries || !p.kv_pages || !p.context_lens || !p.block_tables || !p.query_start_loc || !p.num_seqs || !p.out)
+      return fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaParams");
+    if (p.num_sinks > 0 && !p.sinks) return fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d but sinks is null", p.num_sinks);
+  }
+  return RPA_OK;
+}
+
+}  // namespace rpa
+
+extern "C" {
+
+int rpa_abi_version(void) { return RPA_ABI_VERSION; }
+
+const char* rpa_last_error(void) { return rpa::g_err; }
+
+uint64_t rpa_workspace_bytes(const RpaParams* dims) {
+  if (dims == nullptr || rpa::validate(*dims, false) != RPA_OK) return 0;
+  return 256;
+}
+
+int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stream) {
+  (void)workspace; (void)workspace_bytes; (void)hip_stream;
+  return RPA_OK;
+}
+
+int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {
+  if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
+  const RpaParams& p = *params;
+  int rc = rpa::validate(p, true);
+  if (rc != RPA_OK) return rc;
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  rc = rpa::launch_generic(p, stream);
+  if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
+  if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return RPA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+// Scalar fp32 ragged paged attention: one wavefront per (query row, kv head).
+//
+// This is the exactness kernel: any head_dim, page_size and dtype, no MFMA, fp32
+// accumulation throughout.  It proves the page-table walk, the K/V de-interleave, the
+// GQA mapping and the causal / window / kv_len masks, and it is the fallback for shapes
+// the tiled kernels do not cover.  Semantics follow the reference's XLA implementation,
+// ejkernel/kernels/_xla/ragged_page_attention/_xla_impl_fwd.py:39-201 (mask :128-136,
+// soft cap :125-126, sinks :161-172, denominator clamp :174), except that key blocks
+// lying entirely outside a sliding window are skipped instead of producing NaN.
+#include "rpa_device.h"
+#include "rpa_host.h"
+
+namespace rpa {
+
+constexpr int kMaxElemsPerLane = 8;  // head_dim <= 512
+
+template <typename T, bool kBf16Compute>
+__global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
+  extern __shared__ float q_lds[];  // [head_dim] scaled query row of the current head
+  const int row = blockIdx.x;
+  const int j = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int D = p.head_dim;
+  const int G = p.num_q_heads / p.num_kv_heads;
+  const T* __restrict__ q = static_cast<const T*>(p.queries);
+  const T* __restrict__ kv = static_cast<const T*>(p.kv_pages);
+  T* __restrict__ out = static_cast<T*>(p.out);
+
+  int nseq = p.num_seqs[0];
+  nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
+  const int total = p.query_start_loc[nseq];
+  const size_t row_base = (static_cast<size_t>(row) * p.num_q_heads + static_cast<size_t>(j) * G) * D;
+  if (row >= total) {  // rows past the ragged batch are defined as zero
+    for (int i = lane; i < G * D; i += kWave) Elem<T>::store(out + row_base + i, 0.f);
+    return;
+  }
+  const int s = find_seq(p.query_start_loc, nseq, row);
+  const int q_len = p.query_start_loc[s + 1] - p.query_start_loc[s];
+  const int kv_len = p.context_lens[s];
+  const int pos = kv_len - q_len + (row - p.query_start_loc[s]);
+  const int hi = min(pos + 1, kv_len);
+  const int lo = p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0;
+
+  const bool t_is_bf16 = sizeof(T) == 2;
+  const float scale = t_is_bf16 ? round_bf16(p.softmax_scale) : p.softmax_scale;
+  const float cap = p.logits_soft_cap;
+  const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;
+  const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
+
+  for (int g = 0; g < G; ++g) {
+    const int h = j * G + g;
+    __syncthreads();
+    for (int d = lane; d < D; d += kWave) {
+      float v = Elem<T>::load(q + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d) * scale;
+      if (t_is_bf16 || kBf16Compute) v = round_bf16(v);
+      q_lds[d] = v;
+    }
+    __syncthreads();
+
+    float m = -INFINITY, l = 0.f;
+    float acc[kMaxElemsPerLane];
+#pragma unroll
+    for (int e = 0; e < kMaxElemsPerLane; ++e) acc[e] = 0.f;
+
+    for (int t0 = lo; t0 < hi; t0 += kWave) {
+      const int t = t0 + lane;
+      const bool valid = t < hi;
+      const int tc = valid ? t : hi - 1;
+      const int page = bt[tc / p.page_size];
+      const size_t tok = static_cast<size_t>(page) * p.page_size + (tc % p.page_size);
+      const size_t k_off = tok * tok_stride + static_cast<size_t>(2 * j) * D;
+      const T* __restrict__ kp = kv + k_off;
+      float sc = 0.f;
+      for (int d = 0; d < D; ++d) {
+        float kvv = Elem<T>::load(kp + d);
+        if (kBf16Compute && !t_is_bf16) kvv = round_bf16(kvv);
+        sc = fmaf(q_lds[d], kvv, sc);
+      }
+      if (kBf16Compute) sc = round_bf16(sc);
+      if (cap != 0.f) {
+        if (kBf16Compute) {
+          sc = round_bf16(round_bf16(tanhf(round_bf16(sc / cap))) * cap);
+        } else {
+          sc = cap * tanhf(sc / cap);
+        }
+      }
+      if (!valid) sc = -INFINITY;
+      const float m_new = fmaxf(m, wave_max(sc));
+      float pr;
+      if (kBf16Compute) {
+        pr = valid ? round_bf16(expf(round_bf16(sc - m_new))) : 0.f;
+      } else {
+        pr = valid ? expf(sc - m_new) : 0.f;
+      }
+      const float alpha = expf(m - m_new);  // m == -inf on the first tile -> 0
+      l = l * alpha + wave_sum(pr);
+      m = m_new;
+#pragma unroll
+      for (int e = 0; e < kMaxElemsPerLane; ++e) acc[e] *= alpha;
+      const int n_in_tile = min(kWave, hi - t0);
+      const uint32_t off_lo = static_cast<uint32_t>(k_off), off_hi = static_cast<uint32_t>(k_off >> 32);
+      for (int tt = 0; tt < n_in_tile; ++tt) {
+        const float p_tt = __shfl(pr, tt, kWave);
+        const size_t o = (static_cast<size_t>(__shfl(off_hi, tt, kWave)) << 32) | __shfl(off_lo, tt, kWave);
+        const T* __restrict__ vp = kv + o + D;  // V row follows the K row of the same kv head
+#pragma unroll
+        for (int e = 0; e < kMaxElemsPerLane; ++e) {
+          const int d = lane + e * kWave;
+          if (d < D) {
+            float vv = Elem<T>::load(vp + d);
+            if (kBf16Compute && !t_is_bf16) vv = round_bf16(vv);
+            acc[e] = fmaf(p_tt, vv, acc[e]);
+          }
+        }
+      }
+    }
+
+    float num_scale = 1.f, denom = l;
+    if (p.sinks != nullptr && p.num_sinks > 0) {
+      const float* __restrict__ sk = p.sinks + static_cast<size_t>(h) * p.num_sinks;
+      float smax = -INFINITY;
+      for (int i = 0; i < p.num_sinks; ++i) smax = fmaxf(smax, sk[i]);
+      const float mt = fmaxf(m, smax);
+      float ssum = 0.f;
+      for (int i = 0; i < p.num_sinks; ++i) ssum += expf(sk[i] - mt);
+      num_scale = (m == -INFINITY) ? 0.f : expf(m - mt);
+      denom = num_scale * l + ssum;
+    }
+    denom = fmaxf(denom, 1e-6f);
+#pragma unroll
+    for (int e = 0; e < kMaxElemsPerLane; ++e) {
+      const int d = lane + e * kWave;
+      if (d < D) Elem<T>::store(out + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d, num_scale * acc[e] / denom);
+    }
+  }
+}
+
+int launch_generic(const RpaParams& p, hipStream_t stream) {
+  if (p.head_dim > kMaxElemsPerLane * kWave) return RPA_ERR_UNSUPPORTED;
+  if (p.total_tokens == 0) return RPA_OK;
+  dim3 grid(p.total_tokens, p.num_kv_heads), block(kWave);
+  const size_t lds = static_cast<size_t>(p.head_dim) * sizeof(float);
+  const bool bf16c = p.compute == RPA_COMPUTE_BF16;
+  if (p.dtype == RPA_DTYPE_BF16) {
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, true>), grid, block, lds, stream, p);
+    else hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, false>), grid, block, lds, stream, p);
+  } else {
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<float, true>), grid, block, lds, stream, p);
+    else hipLaunchKernelGGL((rpa_generic_kernel<float, false>), grid, block, lds, stream, p);
+  }
+  return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
+}
+
+}  // namespace rpa

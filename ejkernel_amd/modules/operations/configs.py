@@ -1,0 +1,47 @@
+"""Configuration dataclasses of the ragged paged attention op.
+
+Field names, order and defaults are those of
+``ejkernel/modules/operations/configs.py:29-34`` (``BaseOperationConfig``) and
+``:242-258`` (``RaggedPageAttentionConfig``), so a config object built for the reference
+can be passed here unchanged.  With a single HIP implementation behind the op the fields
+mean:
+
+``num_queries_per_block``   query tokens per prefill tile (None = library default)
+``num_kv_pages_per_block``  pages per decode split (None = chosen from the batch on device)
+``num_warps``               wavefronts per workgroup (only 4 is built; other values are ignored)
+``num_stages``              accepted, unused
+``platform`` / ``backend``  accepted and validated, never used for dispatch
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Literal
+
+_PLATFORMS = ("triton", "pallas", "cuda", "xla", "auto")
+
+
+@dataclass
+class BaseOperationConfig:
+    """Base configuration for all operations."""
+
+    platform: Literal["triton", "pallas", "cuda", "xla", "auto"] = "auto"
+    backend: str = "any"
+
+
+@dataclass
+class RaggedPageAttentionConfig(BaseOperationConfig):
+    """Configuration for the ragged paged attention operation."""
+
+    num_kv_pages_per_block: int | None = None
+    num_queries_per_block: int | None = None
+    num_warps: int = 4
+    num_stages: int = 1
+
+    def validate(self) -> None:
+        if self.platform not in _PLATFORMS:
+            raise ValueError(f"platform={self.platform!r} must be one of {_PLATFORMS}")
+        if self.num_kv_pages_per_block is not None and self.num_kv_pages_per_block <= 0:
+            raise ValueError(f"num_kv_pages_per_block={self.num_kv_pages_per_block} must be positive.")
+        if self.num_queries_per_block is not None and self.num_queries_per_block <= 0:
+            raise ValueError(f"num_queries_per_block={self.num_queries_per_block} must be positive.")

@@ -1,0 +1,222 @@
+"""Seeded synthetic batches for ragged paged attention.
+
+The layout conventions are those of the reference's own input builder,
+``benchmarks/benchmark_ragged_page_attn.py:40-129`` / ``test/test_ragged_page_attn.py:27-115``:
+K and V pages are drawn separately and interleaved on the head axis
+(``stack([k, v], axis=3).reshape(P, page, 2 * Hkv, D)``), ``context_lens`` counts the
+current query tokens, ``num_seqs`` is an int32 array of shape ``[1]``.
+
+Unlike the reference's builder the block tables are a random permutation of the page
+pool (physically scattered pages), and ``queries`` carries ``>= 8`` zero slack rows after
+the last sequence so that an implementation working in 8-row blocks never has to clamp a
+block against the end of the array.
+
+The five named workloads are the benchmark configurations of this repository.  Small
+integers are drawn on the host with ``numpy.random.Generator(PCG64(seed))``; bulk data is
+drawn on the target device in chunks with a seeded ``torch.Generator``.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+
+import numpy as np
+import torch
+
+
+@dataclass
+class Batch:
+    queries: torch.Tensor
+    kv_pages: torch.Tensor
+    context_lens: torch.Tensor
+    block_tables: torch.Tensor
+    query_start_loc: torch.Tensor
+    num_seqs: torch.Tensor
+    softmax_scale: float
+    sliding_window: int | None = None
+    logits_soft_cap: float | None = None
+    q_lens: np.ndarray | None = None
+    kv_lens: np.ndarray | None = None
+    name: str = ""
+    meta: dict = field(default_factory=dict)
+
+    @property
+    def total_valid_tokens(self) -> int:
+        return int(self.q_lens.sum())
+
+    def args(self):
+        return (self.queries, self.kv_pages, self.context_lens, self.block_tables, self.query_start_loc,
+                self.num_seqs)
+
+    def kwargs(self):
+        return dict(softmax_scale=self.softmax_scale, sliding_window=self.sliding_window,
+                    logits_soft_cap=self.logits_soft_cap)
+
+
+def _randn_chunked(shape, gen, device, dtype, chunk_elems=1 << 27):
+    """N(0,1) in `dtype`, drawn in fp32 chunks so a large pool never needs 2x its size."""
+    out = torch.empty(shape, dtype=dtype, device=device)
+    flat = out.view(-1)
+    n = flat.numel()
+    for i in range(0, n, chunk_elems):
+        m = min(chunk_elems, n - i)
+        flat[i:i + m] = torch.randn(m, generator=gen, device=device, dtype=torch.float32).to(dtype)
+    return out
+
+
+def make_batch(q_lens, kv_lens, *, num_q_heads, num_kv_heads, head_dim, page_size, pages_per_seq, num_pages=None,
+               seed=0, device="cpu", dtype=torch.bfloat16, max_num_seqs=None, sliding_window=None,
+               logits_soft_cap=None, softmax_scale=None, slack_rows=8, permute_pages=True, name="") -> Batch:
+    """Build one ragged batch. ``q_lens[i] <= kv_lens[i]``; pages of different sequences are distinct."""
+    q_lens = np.asarray(q_lens, dtype=np.int64)
+    kv_lens = np.asarray(kv_lens, dtype=np.int64)
+    S = len(q_lens)
+    max_num_seqs = max_num_seqs or S
+    assert max_num_seqs >= S and len(kv_lens) == S
+    assert (q_lens <= kv_lens).all(), "q_len must not exceed kv_len"
+    assert kv_lens.max(initial=0) <= pages_per_seq * page_size, "pages_per_seq too small for kv_lens"
+    num_pages = num_pages or max_num_seqs * pages_per_seq
+    assert num_pages >= max_num_seqs * pages_per_seq
+    rng = np.random.Generator(np.random.PCG64(seed))
+    perm = rng.permutation(num_pages) if permute_pages else np.arange(num_pages)
+    block_tables = perm[: max_num_seqs * pages_per_seq].reshape(max_num_seqs, pages_per_seq).astype(np.int32)
+
+    total = int(q_lens.sum())
+    t_alloc = ((total + 7) // 8) * 8 + slack_rows if slack_rows else total
+    cu = np.zeros(max_num_seqs + 1, dtype=np.int32)
+    cu[1:S + 1] = np.cumsum(q_lens)
+    cu[S + 1:] = total
+    ctx = np.zeros(max_num_seqs, dtype=np.int32)
+    ctx[:S] = kv_lens
+
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(int(seed))
+    queries = torch.zeros((t_alloc, num_q_heads, head_dim), dtype=dtype, device=dev)
+    if total:
+        queries[:total] = _randn_chunked((total, num_q_heads, head_dim), gen, dev, dtype)
+    # k_pages / v_pages drawn separately, then interleaved on the head axis
+    kv_pages = torch.empty((num_pages, page_size, 2 * num_kv_heads, head_dim), dtype=dtype, device=dev)
+    kv5 = kv_pages.view(num_pages, page_size, num_kv_heads, 2, head_dim)
+    pages_per_chunk = max(1, (1 << 26) // (page_size * num_kv_heads * head_dim))
+    for which in (0, 1):
+        for p0 in range(0, num_pages, pages_per_chunk):
+            p1 = min(num_pages, p0 + pages_per_chunk)
+            kv5[p0:p1, :, :, which, :] = torch.randn((p1 - p0, page_size, num_kv_heads, head_dim), generator=gen,
+                                                      device=dev, dtype=torch.float32).to(dtype)
+    return Batch(
+        queries=queries,
+        kv_pages=kv_pages,
+        context_lens=torch.from_numpy(ctx).to(dev),
+        block_tables=torch.from_numpy(block_tables).to(dev),
+        query_start_loc=torch.from_numpy(cu).to(dev),
+        num_seqs=torch.tensor([S], dtype=torch.int32, device=dev),
+        softmax_scale=float(head_dim**-0.5 if softmax_scale is None else softmax_scale),
+        sliding_window=sliding_window,
+        logits_soft_cap=logits_soft_cap,
+        q_lens=q_lens,
+        kv_lens=kv_lens,
+        name=name,
+        meta=dict(num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=page_size,
+                  pages_per_seq=pages_per_seq, num_pages=num_pages, max_num_seqs=max_num_seqs, seed=seed),
+    )
+
+
+# name -> description of the five benchmark configurations
+WORKLOADS = {
+    "decode_small": "8 seqs x 1 token, kv 64..512, 8q/2kv heads, D=128, page 16, 512 pages",
+    "decode_llama3_8b": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=128, page 16, 160k pages",
+    "mixed_prefill_decode": "16 prefill chunks x 512 tokens (prior 0..4096) + 240 decode seqs (kv 256..8192), "
+                            "32q/8kv heads, D=128, page 32",
+    "gemma2_local": "64 seqs x 4 tokens, kv 2048..32768, 16q/8kv heads, D=256, page 16, window 4096, cap 50",
+    "decode_long_context": "32 seqs x 1 token, kv 32768..131072, 64q/8kv heads, D=128, page 64, 2^18 pages",
+}
+
+
+def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bfloat16) -> Batch:
+    """Build a named workload. ``scale`` < 1 shrinks sequence counts and lengths for tests."""
+    idx = list(WORKLOADS).index(name) + 1
+    seed = 1000 + idx
+    rng = np.random.Generator(np.random.PCG64(seed))
+
+    def n(x, lo=1):
+        return max(lo, int(round(x * scale)))
+
+    def pages(tokens, page):
+        # at 64 pages and above keep a multiple of 64 (block-table windows of 64 entries then never clamp)
+        k = -(-tokens // page)
+        return k if k < 64 else -(-k // 64) * 64
+
+    if name == "decode_small":
+        S = 8
+        kv = rng.integers(64, 513, size=S)
+        return make_batch(np.ones(S, int), kv, num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16,
+                          pages_per_seq=32, num_pages=512, seed=seed, device=device, dtype=dtype, name=name)
+    if name == "decode_llama3_8b":
+        S = n(256)
+        kv = rng.integers(n(512), n(8192) + 1, size=S)
+        pps = pages(n(8192), 16)
+        pool = max(S * pps, n(160000))
+        return make_batch(np.ones(S, int), kv, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
+                          pages_per_seq=pps, num_pages=pool, seed=seed, device=device, dtype=dtype, name=name)
+    if name == "mixed_prefill_decode":
+        n_pre, n_dec = n(16), n(240)
+        chunk = n(512)
+        prior = rng.integers(0, n(4096) + 1, size=n_pre)
+        kv_dec = rng.integers(n(256), n(8192) + 1, size=n_dec)
+        q = np.concatenate([np.full(n_pre, chunk), np.ones(n_dec, int)])
+        kv = np.concatenate([prior + chunk, kv_dec])
+        order = rng.permutation(n_pre + n_dec)
+        pps = pages(max(n(8192), n(4096) + chunk), 32)
+        return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
+                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=name)
+    if name == "gemma2_local":
+        S = n(64)
+        kv = rng.integers(n(2048), n(32768) + 1, size=S)
+        pps = pages(n(32768), 16)
+        return make_batch(np.full(S, 4), kv, num_q_heads=16, num_kv_heads=8, head_dim=256, page_size=16,
+                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=name,
+                          sliding_window=n(4096), logits_soft_cap=50.0)
+    if name == "decode_long_context":
+        S = n(32)
+        kv = rng.integers(n(32768), n(131072) + 1, size=S)
+        pps = pages(n(131072), 64)
+        pool = max(S * pps, n(1 << 18))
+        return make_batch(np.ones(S, int), kv, num_q_heads=64, num_kv_heads=8, head_dim=128, page_size=64,
+                          pages_per_seq=pps, num_pages=pool, seed=seed, device=device, dtype=dtype, name=name)
+    raise KeyError(name)
+
+
+def compact_for_host(batch: Batch, seq_ids) -> Batch:
+    """Sub-batch holding only ``seq_ids`` with their pages renumbered densely, on the CPU.
+
+    Attention of a sequence depends only on its own pages, so the sub-batch yields the
+    same rows; it lets a host-side checker handle batches whose pool exceeds host RAM.
+    """
+    seq_ids = list(seq_ids)
+    page_size = batch.kv_pages.shape[1]
+    pps = batch.block_tables.shape[1]
+    bt = batch.block_tables.cpu().numpy()
+    cu = batch.query_start_loc.cpu().numpy()
+    q_rows, new_bt, phys = [], np.zeros((len(seq_ids), pps), np.int32), []
+    for i, s in enumerate(seq_ids):
+        n_pg = -(-int(batch.kv_lens[s]) // page_size)
+        new_bt[i, :n_pg] = np.arange(len(phys), len(phys) + n_pg)
+        phys.extend(bt[s, :n_pg].tolist())
+        q_rows.append(torch.arange(int(cu[s]), int(cu[s + 1])))
+    rows = torch.cat(q_rows) if q_rows else torch.zeros(0, dtype=torch.long)
+    q_lens = batch.q_lens[seq_ids]
+    kv_lens = batch.kv_lens[seq_ids]
+    total = int(q_lens.sum())
+    t_alloc = ((total + 7) // 8) * 8 + 8
+    q = torch.zeros((t_alloc,) + tuple(batch.queries.shape[1:]), dtype=batch.queries.dtype)
+    q[:total] = batch.queries[rows.to(batch.queries.device)].cpu()
+    pages = batch.kv_pages[torch.tensor(phys, dtype=torch.long, device=batch.kv_pages.device)].cpu()
+    ncu = np.zeros(len(seq_ids) + 1, np.int32)
+    ncu[1:] = np.cumsum(q_lens)
+    sub = Batch(queries=q, kv_pages=pages, context_lens=torch.from_numpy(kv_lens.astype(np.int32)),
+                block_tables=torch.from_numpy(new_bt), query_start_loc=torch.from_numpy(ncu),
+                num_seqs=torch.tensor([len(seq_ids)], dtype=torch.int32), softmax_scale=batch.softmax_scale,
+                sliding_window=batch.sliding_window, logits_soft_cap=batch.logits_soft_cap, q_lens=q_lens,
+                kv_lens=kv_lens, name=batch.name + "/sub", meta=dict(batch.meta, rows=rows))
+    return sub

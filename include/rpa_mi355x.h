@@ -1,0 +1,107 @@
+/*
+ * rpa_mi355x.h -- C ABI of the MI355X (gfx950) ragged paged attention forward.
+ *
+ * This is the boundary a foreign-function binding targets.  It replaces the backend
+ * entry point the reference registers for this operation,
+ *   ejkernel/kernels/_xla/ragged_page_attention/_interface.py:25-109
+ * (reached from ejkernel/modules/operations/ragged_page_attention.py:540-641), and is
+ * shaped like the reference's own native precedent, a custom call that receives device
+ * buffers plus a stream (ejkernel/callib/_triton_call.py:738-757).
+ *
+ * Conventions
+ *  - Every pointer in RpaParams is a DEVICE pointer owned by the caller.
+ *  - rpa_fwd_launch only enqueues work on the given HIP stream: it never allocates,
+ *    frees, or synchronises, and may be called from several host threads at once.
+ *  - All functions return 0 on success and a negative RPA_ERR_* code on failure;
+ *    rpa_last_error() gives the message of the calling thread's last failure.
+ */
+#ifndef RPA_MI355X_H_
+#define RPA_MI355X_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define RPA_ABI_VERSION 1
+
+/* element type of queries / kv_pages / out */
+#define RPA_DTYPE_BF16 0
+#define RPA_DTYPE_F32 1
+
+/* arithmetic mode */
+#define RPA_COMPUTE_BF16 0 /* bf16 MFMA contractions, fp32 online softmax, reference rounding points */
+#define RPA_COMPUTE_F32 1  /* everything in fp32 (page-gather exactness check) */
+
+#define RPA_OK 0
+#define RPA_ERR_INVALID_ARGUMENT (-1)
+#define RPA_ERR_UNSUPPORTED (-2)
+#define RPA_ERR_WORKSPACE (-3)
+#define RPA_ERR_LAUNCH (-4)
+
+/* rpa_fwd_launch flags */
+#define RPA_FLAG_FORCE_GENERIC 1u /* route every sequence through the scalar fp32 kernel */
+
+typedef struct RpaParams {
+  /* ---- device buffers (argument names follow ragged_page_attention.py:540-547) ---- */
+  const void* queries;         /* [total_tokens, num_q_heads, head_dim]                      */
+  const void* kv_pages;        /* [num_pages, page_size, 2*num_kv_heads, head_dim]; K of kv   */
+                               /* head j at combined index 2j, V at 2j+1                      */
+  const int32_t* context_lens; /* [max_num_seqs]  kv length incl. the current query tokens    */
+  const int32_t* block_tables; /* [max_num_seqs, pages_per_seq] physical page of logical page */
+  const int32_t* query_start_loc; /* [max_num_seqs + 1] cumulative query lengths             */
+  const int32_t* num_seqs;     /* [1] sequences actually present                              */
+  const float* sinks;          /* [num_q_heads, num_sinks] fp32 sink logits, or NULL          */
+  void* out;                   /* [total_tokens, num_q_heads, head_dim], same dtype as queries */
+  void* workspace;             /* >= rpa_workspace_bytes() bytes, 256-byte aligned, or NULL   */
+  uint64_t workspace_bytes;
+
+  /* ---- static shape ---- */
+  int32_t total_tokens;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t page_size;
+  int32_t num_pages;
+  int32_t max_num_seqs;
+  int32_t pages_per_seq;
+  int32_t num_sinks;
+
+  /* ---- scalars ---- */
+  float softmax_scale;    /* multiplies q . k                                   */
+  float logits_soft_cap;  /* cap * tanh(x / cap); 0 = disabled                  */
+  int32_t sliding_window; /* keys with pos > q_pos - window are kept; 0 = none  */
+  int32_t dtype;          /* RPA_DTYPE_*                                        */
+  int32_t compute;        /* RPA_COMPUTE_*                                      */
+
+  /* ---- tile overrides, 0 = library default.  They carry the fields of            */
+  /*      RaggedPageAttentionConfig (modules/operations/configs.py:242-258).        */
+  int32_t num_queries_per_block;  /* query tokens per prefill tile                   */
+  int32_t num_kv_pages_per_block; /* split length of a decode sequence, in pages      */
+  int32_t num_warps;              /* wavefronts per workgroup                         */
+  int32_t num_stages;             /* reserved                                         */
+  uint32_t flags;                 /* RPA_FLAG_*                                       */
+} RpaParams;
+
+/* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */
+uint64_t rpa_workspace_bytes(const RpaParams* dims);
+
+/* Clears the counters at the head of a freshly allocated workspace (enqueue only).
+ * A launch leaves them cleared again, so this is needed once per allocation. */
+int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stream);
+
+/* Enqueues the forward pass on `hip_stream` (a hipStream_t; NULL = default stream). */
+int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
+
+/* Message for the calling thread's most recent failure ("" if none). */
+const char* rpa_last_error(void);
+
+/* RPA_ABI_VERSION the library was built with. */
+int rpa_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RPA_MI355X_H_ */

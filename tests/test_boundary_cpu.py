@@ -1,0 +1,119 @@
+"""Host-side checks that need no GPU: the C-ABI library loads and exports what the header
+declares, the Python boundary keeps the reference's signature and config dataclass, and
+argument errors are raised the way the reference's validators raise them."""
+
+import ctypes
+import dataclasses
+import inspect
+import re
+from pathlib import Path
+
+import pytest
+import torch
+
+from ejkernel_amd import _native
+from ejkernel_amd.modules import RaggedPageAttention, RaggedPageAttentionConfig, ragged_page_attention
+from ejkernel_amd.workloads import make_batch
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def _declared_functions():
+    text = (ROOT / "include" / "rpa_mi355x.h").read_text()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rpa_[a-z_]+)\s*\(", text)))
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    lib = _native.load()
+    declared = _declared_functions()
+    assert declared == sorted(_native.EXPORTED_SYMBOLS)
+    for name in declared:
+        assert getattr(lib, name) is not None
+    assert lib.rpa_abi_version() == _native.RPA_ABI_VERSION
+
+
+def test_struct_layout_matches_header_field_order():
+    text = (ROOT / "include" / "rpa_mi355x.h").read_text()
+    body = text[text.index("typedef struct RpaParams {"):text.index("} RpaParams;")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = re.findall(r"([a-z_]+)\s*;", body)
+    assert names == [f[0] for f in _native.RpaParams._fields_]
+    assert ctypes.sizeof(_native.RpaParams) % 8 == 0
+
+
+def test_workspace_bytes_and_errors_without_gpu():
+    lib = _native.load()
+    p = _native.RpaParams()
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0  # zero dims are invalid
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = 16, 8, 2, 128
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = 16, 64, 4, 16
+    p.softmax_scale = 0.1
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) >= 256
+    assert lib.rpa_fwd_launch(ctypes.byref(p), None) == -1  # null pointers are rejected before any launch
+    assert b"null" in lib.rpa_last_error()
+    p.num_kv_heads = 3
+    assert lib.rpa_workspace_bytes(ctypes.byref(p)) == 0
+    assert lib.rpa_fwd_launch(None, None) == -1
+
+
+def test_signature_matches_reference():
+    sig = inspect.signature(ragged_page_attention)
+    params = list(sig.parameters.values())
+    positional = [p.name for p in params if p.kind is inspect.Parameter.POSITIONAL_ONLY]
+    assert positional == ["queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs",
+                          "softmax_aux"]
+    keyword = [p.name for p in params if p.kind is inspect.Parameter.KEYWORD_ONLY]
+    assert keyword == ["softmax_scale", "logits_soft_cap", "compute_dtype", "optimized", "sliding_window",
+                       "mask_value", "vmem_limit_bytes", "platform", "cfg", "mesh", "in_specs", "out_specs"]
+    assert sig.parameters["softmax_aux"].default is None
+
+
+def test_config_dataclass_fields_and_defaults():
+    fields = [(f.name, f.default) for f in dataclasses.fields(RaggedPageAttentionConfig)]
+    assert fields == [("platform", "auto"), ("backend", "any"), ("num_kv_pages_per_block", None),
+                      ("num_queries_per_block", None), ("num_warps", 4), ("num_stages", 1)]
+    k = RaggedPageAttention()
+    assert k.op_id == "ragged_page_attention"
+    assert k.heuristic_cfg(None) == RaggedPageAttentionConfig()
+    assert k.candidate_cfgs(None) == [RaggedPageAttentionConfig()]
+
+
+def _b(**kw):
+    return make_batch([2, 1], [9, 30], num_q_heads=4, num_kv_heads=2, head_dim=16, page_size=4, pages_per_seq=8,
+                      seed=1, **kw)
+
+
+def test_validation_errors_mirror_reference():
+    b = _b()
+    a = list(b.args())
+    with pytest.raises(ValueError, match="must be positive"):
+        ragged_page_attention(*a, sliding_window=0)
+    with pytest.raises(ValueError, match="must not be 0.0"):
+        ragged_page_attention(*a, logits_soft_cap=0.0)
+    with pytest.raises(ValueError, match=r"must be \(1,\)"):
+        ragged_page_attention(a[0], a[1], a[2], a[3], a[4], torch.tensor([2, 2], dtype=torch.int32))
+    with pytest.raises(ValueError, match="int32"):
+        ragged_page_attention(a[0], a[1], a[2].long(), a[3], a[4], a[5])
+    with pytest.raises(ValueError, match="context_lens.shape"):
+        ragged_page_attention(a[0], a[1], a[2][:1], a[3], a[4], a[5])
+    with pytest.raises(ValueError, match="query_start_loc.shape"):
+        ragged_page_attention(a[0], a[1], a[2], a[3], a[4][:2], a[5])
+    with pytest.raises(ValueError, match="head_dim"):
+        ragged_page_attention(a[0][..., :8], a[1], a[2], a[3], a[4], a[5])
+    with pytest.raises(ValueError, match="divisible"):
+        ragged_page_attention(a[0][:, :3], a[1], a[2], a[3], a[4], a[5])
+    with pytest.raises(ValueError, match="num_kv_pages_per_block"):
+        ragged_page_attention(*a, cfg=RaggedPageAttentionConfig(num_kv_pages_per_block=9))
+    with pytest.raises(ValueError, match="num_queries_per_block"):
+        ragged_page_attention(*a, cfg=RaggedPageAttentionConfig(num_queries_per_block=-1))
+    with pytest.raises(ValueError, match="platform"):
+        ragged_page_attention(*a, platform="tpu")
+    with pytest.raises(NotImplementedError):
+        ragged_page_attention(*a, mesh=object(), in_specs=(None,) * 7, out_specs=None)
+
+
+def test_no_cpu_fallback():
+    b = _b()
+    with pytest.raises(RuntimeError, match="no CPU implementation"):
+        ragged_page_attention(*b.args())

@@ -1,0 +1,249 @@
+"""Parity of the HIP path (called through the C ABI) against the CPU oracle.
+
+bf16: max-abs <= 2e-2 and mean-abs <= 2e-3 against ``rpa_strict`` (the restatement of the
+reference's XLA implementation, bf16 rounding points included).  fp32 mode: <= 1e-5 against
+the float64 evaluation; page gathering is checked bit-exactly on cases with a closed form.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from ejkernel_amd import _native
+from ejkernel_amd.modules import RaggedPageAttention, RaggedPageAttentionConfig, ragged_page_attention
+from ejkernel_amd.workloads import Batch, compact_for_host, make_batch, make_workload
+from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, run_exact, run_strict, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+PATHS = [pytest.param(0, id="tiled"), pytest.param(_native.RPA_FLAG_FORCE_GENERIC, id="generic")]
+
+
+def run_hip(b: Batch, flags=0, compute_dtype=None, softmax_aux=None, cfg=None):
+    if compute_dtype is None:
+        compute_dtype = b.queries.dtype
+    aux = None if softmax_aux is None else torch.as_tensor(softmax_aux, device=b.queries.device)
+    out = RaggedPageAttention().run(*b.args(), softmax_scale=b.softmax_scale, logits_soft_cap=b.logits_soft_cap,
+                                    compute_dtype=compute_dtype, sliding_window=b.sliding_window, softmax_aux=aux,
+                                    cfg=cfg or RaggedPageAttentionConfig(), _flags=flags)
+    torch.cuda.synchronize()
+    return out
+
+
+def small(q_lens, kv_lens, **kw):
+    args = dict(num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=16, seed=7, device=DEV)
+    args.update(kw)
+    return make_batch(q_lens, kv_lens, **args)
+
+
+# ----------------------------------------------------------------------------- fp32 mode: gather exactness
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_fp32_mode_matches_float64_evaluation(flags):
+    b = make_workload("decode_small", device=DEV, dtype=torch.float32)
+    out = to_np(run_hip(b, flags, compute_dtype=torch.float32))
+    rows = b.total_valid_tokens
+    mx, _ = err_stats(out, run_exact(b), rows)
+    assert mx <= F32_MAX_ABS, mx
+    assert not out[rows:].any()
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_fp32_mode_ragged_mix(flags):
+    b = small([9, 1, 0, 17, 2, 4], [40, 250, 8, 17, 133, 256], dtype=torch.float32, max_num_seqs=8)
+    out = to_np(run_hip(b, flags, compute_dtype=torch.float32))
+    mx, _ = err_stats(out, run_exact(b), b.total_valid_tokens)
+    assert mx <= F32_MAX_ABS, mx
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_single_key_gather_is_bit_exact(flags, dtype):
+    """kv_len = 1 => out == the V row of token 0, bit for bit (page, slot and head indexing)."""
+    S = 12
+    b = small(np.ones(S, int), np.ones(S, int), dtype=dtype, num_q_heads=8, num_kv_heads=4)
+    out = run_hip(b, flags)
+    bt = b.block_tables.long()
+    want = b.kv_pages[bt[:, 0], 0, 1::2, :].repeat_interleave(2, dim=1)  # [S, Hq, D]
+    assert torch.equal(out[:S], want)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_zero_query_mean_of_values_fp32(flags):
+    """q = 0 => out = mean of the visible V rows; V carries small integers so fp32 sums are exact."""
+    b = small([3, 1, 5], [37, 200, 5], dtype=torch.float32, num_q_heads=4, num_kv_heads=2, head_dim=64)
+    b.queries.zero_()
+    gen = torch.Generator(device=DEV).manual_seed(1)
+    b.kv_pages.copy_(torch.randint(-8, 9, b.kv_pages.shape, generator=gen, device=DEV).float())
+    out = to_np(run_hip(b, flags, compute_dtype=torch.float32))
+    mx, _ = err_stats(out, run_exact(b), b.total_valid_tokens)
+    assert mx <= 2e-6, mx
+
+
+# ----------------------------------------------------------------------------- bf16 parity vs the strict oracle
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_bf16_decode_small_full_size(flags):
+    b = make_workload("decode_small", device=DEV)
+    out = to_np(run_hip(b, flags))
+    assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, "decode_small")
+    assert not out[b.total_valid_tokens:].any()
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("name,scale", [("decode_llama3_8b", 0.06), ("mixed_prefill_decode", 0.08),
+                                        ("decode_long_context", 0.04)])
+def test_bf16_scaled_workloads(flags, name, scale):
+    b = make_workload(name, device=DEV, scale=scale)
+    out = to_np(run_hip(b, flags))
+    assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, name)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_bf16_gemma2_local_scaled(flags):
+    """Window + soft cap + head_dim 256.  Where the strict oracle turns NaN (a leading KV block entirely outside
+    the window) the row is compared with the float64 evaluation instead."""
+    b = make_workload("gemma2_local", device=DEV, scale=0.1)
+    out = to_np(run_hip(b, flags))
+    rows = b.total_valid_tokens
+    strict, exact = run_strict(b), run_exact(b)
+    nan_rows = np.isnan(strict[:rows]).any(axis=(1, 2))
+    ref = np.where(nan_rows[:, None, None], exact[:rows], strict[:rows])
+    assert_bf16_parity(out, ref, rows, "gemma2_local")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (8, 4), (8, 2), (16, 2), (8, 1)])
+def test_bf16_gqa_ratios(flags, hq, hkv):
+    b = small([6, 1, 1, 33], [70, 255, 256, 33], num_q_heads=hq, num_kv_heads=hkv)
+    assert_bf16_parity(to_np(run_hip(b, flags)), run_strict(b), b.total_valid_tokens, f"gqa {hq}/{hkv}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("page", [1, 4, 8, 16, 32, 64, 128])
+def test_bf16_page_sizes(flags, page):
+    pps = max(2, 512 // page)
+    b = small([5, 1, 1, 40], [300, 511, 17, 40], page_size=page, pages_per_seq=pps)
+    assert_bf16_parity(to_np(run_hip(b, flags)), run_strict(b), b.total_valid_tokens, f"page {page}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_bf16_head_dims(flags, D):
+    b = small([5, 1, 2, 40], [300, 511, 17, 40], head_dim=D, pages_per_seq=32)
+    assert_bf16_parity(to_np(run_hip(b, flags)), run_strict(b), b.total_valid_tokens, f"D {D}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_bf16_ragged_edge_cases(flags):
+    """Empty sequences, kv_len not a page multiple, padding entries, garbage beyond the pages in use."""
+    q_lens = [0, 1, 7, 0, 64, 1, 3, 130]
+    kv_lens = [5, 1, 7, 16, 100, 241, 19, 131]
+    b = small(q_lens, kv_lens, max_num_seqs=11)
+    bt = b.block_tables.clone()
+    for s, kl in enumerate(kv_lens):
+        bt[s, -(-kl // 16):] = -1 if s % 2 else 2**30
+    bt[len(q_lens):] = -5
+    ref_b = Batch(**{**b.__dict__})
+    b.block_tables = bt
+    out = to_np(run_hip(b, flags))
+    assert_bf16_parity(out, run_strict(ref_b), b.total_valid_tokens, "edge cases")
+    assert not out[b.total_valid_tokens:].any()
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("window,cap", [(16, None), (100, None), (None, 30.0), (33, 5.0)])
+def test_bf16_window_and_cap(flags, window, cap):
+    b = small([4, 1, 1, 50], [200, 255, 40, 50], sliding_window=window, logits_soft_cap=cap)
+    rows = b.total_valid_tokens
+    strict = run_strict(b)
+    assert np.isfinite(strict[:rows]).all()  # pages_per_seq < 64: one KV block, no NaN defect
+    assert_bf16_parity(to_np(run_hip(b, flags)), strict, rows, f"window {window} cap {cap}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("shape", ["per_q", "per_kv", "shared"])
+def test_bf16_sinks(flags, shape):
+    b = small([4, 1, 1, 20], [200, 255, 1, 20])
+    rng = np.random.default_rng(3)
+    aux = {"per_q": rng.standard_normal((8, 2)), "per_kv": rng.standard_normal((2, 3)),
+           "shared": rng.standard_normal(2)}[shape].astype(np.float32)
+    aux_bf = torch.from_numpy(aux).to(torch.bfloat16)
+    out = to_np(run_hip(b, flags, softmax_aux=aux_bf.to(DEV)))
+    ref = run_strict(b, softmax_aux=aux_bf.float().numpy())
+    assert_bf16_parity(out, ref, b.total_valid_tokens, f"sinks {shape}")
+    base = to_np(run_hip(b, flags))
+    assert np.abs(base - out)[: b.total_valid_tokens].max() > 1e-3  # sinks change the result
+
+
+# ----------------------------------------------------------------------------- invariants on the device result
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_window_covering_everything_equals_no_window(flags):
+    b = small([4, 1, 1, 50], [200, 255, 40, 50])
+    base = run_hip(b, flags)
+    b.sliding_window = 256
+    assert torch.equal(run_hip(b, flags), base)
+    b.logits_soft_cap = 1e6  # cap far above any logit: tanh is linear there
+    d = (run_hip(b, flags).float() - base.float()).abs().max().item()
+    assert d < 0.1, d  # bound of the reference's own property test (test_ragged_page_attention.py:437-461)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_page_permutation_invariance_is_bitwise(flags):
+    b = make_workload("mixed_prefill_decode", device=DEV, scale=0.08)
+    base = run_hip(b, flags)
+    P = b.kv_pages.shape[0]
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(9)).to(DEV)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(P, device=DEV)
+    b2 = Batch(**{**b.__dict__})
+    b2.kv_pages = b.kv_pages[perm].contiguous()
+    b2.block_tables = inv[b.block_tables.long()].to(torch.int32)
+    assert torch.equal(run_hip(b2, flags), base)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_rows_do_not_depend_on_batch_composition(flags):
+    b = small([4, 1, 1, 50, 1], [200, 255, 40, 50, 90], max_num_seqs=7)
+    full = run_hip(b, flags)
+    cu = b.query_start_loc.cpu().numpy()
+    for s in (1, 3, 4):
+        sub = compact_for_host(b, [s])
+        sub_dev = Batch(**{**sub.__dict__})
+        for f in ("queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs"):
+            setattr(sub_dev, f, getattr(sub, f).to(DEV))
+        alone = run_hip(sub_dev, flags)
+        n = int(b.q_lens[s])
+        assert torch.equal(alone[:n], full[cu[s]:cu[s] + n]), s
+
+
+def test_repeated_calls_are_deterministic():
+    b = make_workload("decode_llama3_8b", device=DEV, scale=0.1)
+    a = run_hip(b)
+    for _ in range(3):
+        assert torch.equal(run_hip(b), a)
+
+
+def test_module_function_is_the_same_path():
+    b = small([4, 1], [200, 255])
+    a = ragged_page_attention(*b.args(), softmax_scale=b.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.equal(a, run_hip(b))
+    c = ragged_page_attention(b.queries, b.kv_pages, b.context_lens, b.block_tables, b.query_start_loc, 2)
+    torch.cuda.synchronize()
+    assert torch.equal(a, c)  # num_seqs may be a plain int; scale defaults to head_dim ** -0.5
+
+
+def test_non_default_stream():
+    b = small([4, 1], [200, 255])
+    base = run_hip(b)
+    st = torch.cuda.Stream()
+    with torch.cuda.stream(st):
+        out = ragged_page_attention(*b.args(), softmax_scale=b.softmax_scale)
+    st.synchronize()
+    assert torch.equal(out, base)
