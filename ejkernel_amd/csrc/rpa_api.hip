@@ -4,6 +4,7 @@
 // ejkernel/kernels/_pallas/tpu/ragged_page_attention/_pallas_impl_fwd.py:177-230
 // (static_validate_inputs) and the named-dimension checks of
 // ejkernel/kernels/_xla/ragged_page_attention/_interface.py:26-47.
+#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 
@@ -42,6 +43,18 @@ static int validate(const RpaParams& p, bool need_pointers) {
   return RPA_OK;
 }
 
+int device_cu_count() {
+  static std::atomic<int> cache[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  int n = cache[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+    cache[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
+
 }  // namespace rpa
 
 extern "C" {
@@ -52,11 +65,18 @@ const char* rpa_last_error(void) { return rpa::g_err; }
 
 uint64_t rpa_workspace_bytes(const RpaParams* dims) {
   if (dims == nullptr || rpa::validate(*dims, false) != RPA_OK) return 0;
-  return 256;
+  rpa::WorkspaceLayout wl;
+  rpa::tiled_workspace_layout(*dims, &wl);
+  return wl.total_bytes;
 }
 
 int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stream) {
-  (void)workspace; (void)workspace_bytes; (void)hip_stream;
+  // Only the split tickets need a defined value; they sit at the head of the workspace and every launch
+  // leaves them at zero again.
+  if (workspace == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "workspace is null");
+  const uint64_t n = workspace_bytes < rpa::kWorkspaceTicketBytes ? workspace_bytes : rpa::kWorkspaceTicketBytes;
+  if (hipMemsetAsync(workspace, 0, n, static_cast<hipStream_t>(hip_stream)) != hipSuccess)
+    return rpa::fail(RPA_ERR_LAUNCH, "hipMemsetAsync on the workspace failed");
   return RPA_OK;
 }
 
@@ -66,6 +86,14 @@ int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {
   int rc = rpa::validate(p, true);
   if (rc != RPA_OK) return rc;
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if (rpa::tiled_supported(p)) {
+    rc = rpa::launch_tiled(p, stream);
+    if (rc == RPA_ERR_WORKSPACE)
+      return rpa::fail(rc, "workspace of %llu bytes is too small, rpa_workspace_bytes() asks for %llu",
+                       (unsigned long long)p.workspace_bytes, (unsigned long long)rpa_workspace_bytes(&p));
+    if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
+    return RPA_OK;
+  }
   rc = rpa::launch_generic(p, stream);
   if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));

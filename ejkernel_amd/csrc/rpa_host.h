@@ -10,6 +10,26 @@ namespace rpa {
 // Each returns RPA_OK or a negative RPA_ERR_* code; all of them only enqueue on `stream`.
 int launch_generic(const RpaParams& p, hipStream_t stream);
 
+// Tiled MFMA path (bf16, head_dim 128 or 256, page_size a multiple of 4).
+constexpr int kTiledMaxSeqs = 2048;        // schedule arrays live in LDS
+constexpr int kTiledTargetItems = 16384;   // split length is chosen so decode splits stay below this count
+
+constexpr uint64_t kWorkspaceTicketBytes = 1u << 20;  // head of the workspace, cleared by rpa_workspace_init
+
+struct WorkspaceLayout {
+  uint64_t counters_bytes;                   // split tickets at offset 0
+  uint64_t partial_o_off, partial_o_bytes;   // fp32 [slots][16][head_dim]
+  uint64_t partial_ml_off, partial_ml_bytes; // fp32 [slots][16][2] (row max, row sum)
+  uint64_t total_bytes;
+};
+
+bool tiled_supported(const RpaParams& p);
+void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl);
+int launch_tiled(const RpaParams& p, hipStream_t stream);
+
+// Compute units of the current device (cached per device).
+int device_cu_count();
+
 // Records the calling thread's error message and returns `code`.
 int fail(int code, const char* fmt, ...);
 
