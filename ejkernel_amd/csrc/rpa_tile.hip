@@ -29,6 +29,7 @@ typedef __attribute__((ext_vector_type(4))) short s16x4_t;
 typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
 
 constexpr int kWgThreads = 256;
 constexpr int kWgWaves = kWgThreads / kWave;
@@ -38,7 +39,8 @@ struct TileArgs {
   RpaParams p;
   int target_items;   // upper bound used to size split length (and the workspace)
   int user_chunk;     // tokens per split requested by the caller, 0 = automatic
-  int page_shift;     // log2(page_size) or -1
+  int page_shift;     // log2(page_size)
+  int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
   uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
   float* partial_o;   // [slots][16][D]
   float* partial_ml;  // [slots][16][2]
@@ -95,9 +97,15 @@ __device__ __forceinline__ int block_excl_scan(int v, int* wave_tot, int& total)
   return base + inc - v;
 }
 
+// Hardware round-to-nearest-even conversions (v_cvt_pk_bf16_f32): branch-free, NaN stays NaN.
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  return static_cast<uint32_t>(f32_to_bf16(lo)) | (static_cast<uint32_t>(f32_to_bf16(hi)) << 16);
+  bf16x2_t v;
+  v[0] = static_cast<__bf16>(lo);
+  v[1] = static_cast<__bf16>(hi);
+  return __builtin_bit_cast(uint32_t, v);
 }
+__device__ __forceinline__ float rbf(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
 
 template <int D, int NT, bool kMimic>
 struct Cfg {
@@ -145,7 +153,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   // ---- Q^T operands: lane (row i, group g) holds q[row][32 ks + 8 g .. +8], pre-scaled and rounded to bf16
   bf16x8_t qreg[C::NKS];
   {
-    const float scale = round_bf16(p.softmax_scale);
+    const float scale = rbf(p.softmax_scale);
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
@@ -169,49 +177,66 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 
   const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;  // elements between tokens
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
+  // Same row through the constant address space: reads with a wave-uniform index become scalar loads, which
+  // are counted apart from the vector loads of the K/V stream.  The block table is never written by this kernel.
+  const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(bt));
   const int t_last = range_hi - 1;
   const float cap = p.logits_soft_cap;
 
   u32x4_t kreg[C::NSLOT][C::NS];
   u32x4_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
 
-  // Page ids of this lane's token groups (tokens tile + 16u + 4g .. +3), read one iteration before the rows.
-  int pg[NT];
-  auto token_group = [&](int tile, int u, int& t4c) {
-    t4c = min(tile + 16 * u + 4 * g, t_last & ~3);
-  };
-  auto load_pages = [&](int tile) {
-#pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      int t4c;
-      token_group(tile, u, t4c);
-      pg[u] = bt[a.page_shift >= 0 ? (t4c >> a.page_shift) : (t4c / p.page_size)];
-    }
-  };
   // Fetch K and V of the TT tokens starting at `tile`: lane (i, g) takes tokens 16u + 4g + r (u < NT, r < 4),
-  // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.  Tokens past
-  // the end of the range are replaced by the last valid one (their scores are masked).
+  // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.
+  //
+  // Fast path (page_size >= 16, tile entirely inside the range): a 16-token sub-tile sits in one page, so the
+  // block-table entry is a scalar load (it does not share the vector-memory counter with the K/V stream) and
+  // the row address is a scalar base plus one per-lane byte offset that is constant for the whole item.
+  // Slow path (last tile of a range, small pages): per-lane page lookup; tokens past the end of the range are
+  // replaced by the last valid one (their scores are masked).
+  const char* kvb = reinterpret_cast<const char*>(kv);
+  const uint32_t stride_b = static_cast<uint32_t>(tok_stride) * 2u;  // bytes between tokens
+  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + static_cast<uint32_t>(2 * j * D * 2 + 16 * i);
   auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
+    if (a.uniform_page && tile + C::TT <= range_hi) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        const int t16 = tile + 16 * u;
+        int page = bt_c[t16 >> a.page_shift];
+        page = min(max(page, 0), p.num_pages - 1);
+        const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                            static_cast<uint64_t>(t16 & (p.page_size - 1)) * stride_b;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const char* row = sbase + static_cast<uint64_t>(r) * stride_b;
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN) {
+            kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN));
+            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN + 2u * D));
+          }
+        }
+      }
+      return;
+    }
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
-      int t4c;
-      token_group(tile, u, t4c);
+      const int t4c = min(tile + 16 * u + 4 * g, t_last & ~3);
       const int rlim = min(3, t_last - t4c);
-      const int slot = a.page_shift >= 0 ? (t4c & (p.page_size - 1)) : (t4c % p.page_size);
-      const int page = min(max(pg[u], 0), p.num_pages - 1);
-      const bf16_t* base = kv + (static_cast<size_t>(page) * p.page_size + slot) * tok_stride +
-                           static_cast<size_t>(2 * j) * D + 8 * i;
+      int page = bt[t4c >> a.page_shift];
+      page = min(max(page, 0), p.num_pages - 1);
+      const char* base = kvb + static_cast<uint64_t>(page) * page_b +
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (2 * j * D * 2 + 16 * i);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
-        const bf16_t* row = base + static_cast<size_t>(min(r, rlim)) * tok_stride;
+        const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
-          kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 128 * sN);
-          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + D + 128 * sN);
+          kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN);
+          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN + 2 * D);
         }
       }
     }
-    load_pages(tile + C::TT);
   };
 
   auto body = [&](int tile, u32x4_t (&vcur)[C::NSLOT][C::NS], u32x4_t (&vnext)[C::NSLOT][C::NS]) {
@@ -239,25 +264,32 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     // 4. online softmax; this lane: query row i, tokens tile + 16u + 4g + r
     float sv[NT][4];
     const bool need_mask = (tile + C::TT > range_hi) || (tile + C::TT - 1 > pos_min) || (W > 0 && tile <= pos_max - W);
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r];
+    if (cap != 0.f) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int tok = tile + 16 * u + 4 * g + r;
+          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W);
+          sv[u][r] = keep ? sv[u][r] : -INFINITY;
+        }
+    }
     float tmax = -INFINITY;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float x = s_acc[u][r];
-        if (kMimic) x = round_bf16(x);
-        if (cap != 0.f) {
-          if (kMimic) x = round_bf16(round_bf16(tanhf(round_bf16(x / cap))) * cap);
-          else x = cap * tanhf(x / cap);
-        }
-        if (need_mask) {
-          const int tok = tile + 16 * u + 4 * g + r;
-          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W);
-          x = keep ? x : -INFINITY;
-        }
-        sv[u][r] = x;
-        tmax = fmaxf(tmax, x);
-      }
+      for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, sv[u][r]);
     tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
     tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
     const float m_new = fmaxf(m_run, tmax);
@@ -271,9 +303,9 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         float d = sv[u][r] - m_use;
-        if (kMimic) d = round_bf16(d);
+        if (kMimic) d = rbf(d);
         float e = __builtin_amdgcn_exp2f(d * kLog2e);
-        e = round_bf16(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
+        e = rbf(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
         pv[r] = e;
         psum += e;
       }
@@ -314,7 +346,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   };
 
   if (range_hi > range_lo) {
-    load_pages(range_lo);
     issue_loads(range_lo, kreg, vbuf0);
     for (int tile = range_lo; tile < range_hi; tile += 2 * C::TT) {
       body(tile, vbuf0, vbuf1);
@@ -328,35 +359,43 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   l_run += __shfl_xor(l_run, 32, kWave);
 
   if (n_splits > 1) {
-    // ---- partial to the workspace, then take a ticket; the last split merges all of them in split order
+    // ---- partial to the workspace, then take a ticket; the last split merges all of them in split order.
+    // Partials are written and read with agent-scope relaxed atomics (write-through / cache-bypassing accesses),
+    // so no L2 write-back or invalidate is needed around the ticket: it is enough that this wave's stores have
+    // completed (the workgroup-scope release waits for them) before the ticket is taken.
     const size_t slot = static_cast<size_t>(slot_base + split);
-    float* po = a.partial_o + (slot * 16 + i) * D;
     if (row_valid) {
+      uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
 #pragma unroll
       for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float* dst = po + 128 * sN + 32 * g + 8 * r;
-          *reinterpret_cast<f32x4_t*>(dst) = f32x4_t{o_acc[sN][0][r], o_acc[sN][1][r], o_acc[sN][2][r], o_acc[sN][3][r]};
-          *reinterpret_cast<f32x4_t*>(dst + 4) = f32x4_t{o_acc[sN][4][r], o_acc[sN][5][r], o_acc[sN][6][r], o_acc[sN][7][r]};
-        }
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint64_t v = static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e][r])) |
+                               (static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e + 1][r])) << 32);
+            __hip_atomic_store(po + (128 * sN + 32 * g + 8 * r) / 2 + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
       if (g == 0) {
-        a.partial_ml[(slot * 16 + i) * 2] = m_run;
-        a.partial_ml[(slot * 16 + i) * 2 + 1] = l_run;
+        const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_run)) | (static_cast<uint64_t>(__float_as_uint(l_run)) << 32);
+        __hip_atomic_store(reinterpret_cast<uint64_t*>(a.partial_ml) + slot * 16 + i, v, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
       }
     }
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     uint32_t* ctr = a.counters + static_cast<size_t>(s) * p.num_kv_heads + j;
     uint32_t ticket = 0;
-    if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     ticket = __shfl(ticket, 0, kWave);
     if (ticket != static_cast<uint32_t>(n_splits - 1)) return;
-    __threadfence();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + static_cast<size_t>(slot_base) * 16 + i;
     float M = -INFINITY;
-    for (int k = 0; k < n_splits; ++k) {
-      const float mk = a.partial_ml[((static_cast<size_t>(slot_base) + k) * 16 + i) * 2];
-      M = fmaxf(M, row_valid ? mk : -INFINITY);
-    }
+    if (row_valid)
+      for (int k = 0; k < n_splits; ++k) {
+        const uint64_t v = __hip_atomic_load(ml + static_cast<size_t>(k) * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v)));
+      }
     const float M_use = M == -INFINITY ? 0.f : M;
     float L = 0.f;
 #pragma unroll
@@ -365,24 +404,22 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (row_valid) {
       for (int k = 0; k < n_splits; ++k) {
-        const size_t sl = static_cast<size_t>(slot_base) + k;
-        const float mk = a.partial_ml[(sl * 16 + i) * 2];
-        const float lk = a.partial_ml[(sl * 16 + i) * 2 + 1];
+        const uint64_t mlv = __hip_atomic_load(ml + static_cast<size_t>(k) * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float mk = __uint_as_float(static_cast<uint32_t>(mlv)), lk = __uint_as_float(static_cast<uint32_t>(mlv >> 32));
         const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
         L += w * lk;
-        const float* src = a.partial_o + (sl * 16 + i) * D;
+        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + ((static_cast<size_t>(slot_base) + k) * 16 + i) * D);
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(src + 128 * sN + 32 * g + 8 * r);
-            const f32x4_t x1 = *reinterpret_cast<const f32x4_t*>(src + 128 * sN + 32 * g + 8 * r + 4);
+          for (int r = 0; r < 4; ++r)
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-              o_acc[sN][c][r] += w * x0[c];
-              o_acc[sN][c + 4][r] += w * x1[c];
+            for (int e = 0; e < 4; ++e) {
+              const uint64_t v = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+              o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(v));
+              o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(v >> 32));
             }
-          }
       }
     }
     m_run = M;
@@ -421,7 +458,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   using C = Cfg<D, NT, kMimic>;
   extern __shared__ __align__(16) char smem[];
   const RpaParams& p = a.p;
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int G = p.num_q_heads / p.num_kv_heads;
   // LDS: [4 waves x K tile][item_start: S+1][slot_start: S+1][scratch 8 ints]
   char* lds_k = smem + wave * C::LDS_PER_WAVE;
@@ -445,7 +482,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   long long want = (static_cast<long long>(tot64) * 64 * p.num_kv_heads + a.target_items - 1) / a.target_items;
   int chunk = static_cast<int>(min(want, static_cast<long long>(1) << 30));
   chunk = max(chunk, a.user_chunk > 0 ? a.user_chunk : 4 * C::TT);
-  chunk = (chunk + C::TT - 1) & ~(C::TT - 1);
+  chunk = __builtin_amdgcn_readfirstlane((chunk + C::TT - 1) & ~(C::TT - 1));
 
   int my_items = 0, my_slots = 0;
   for (int s = s_begin; s < s_end; ++s) {
@@ -465,6 +502,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     item_base += p.num_kv_heads * si.n_rt * ns;
     slot_base += ns > 1 ? p.num_kv_heads * ns : 0;
   }
+  total_items = __builtin_amdgcn_readfirstlane(total_items);
   if (tid == 0) item_start[nseq] = total_items;
   __syncthreads();
 
@@ -485,15 +523,16 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       const int mid = (lo + hi) >> 1;
       if (item_start[mid] <= w) lo = mid; else hi = mid;
     }
-    const int s = lo;
+    const int s = __builtin_amdgcn_readfirstlane(lo);
     const SeqInfo si = seq_info<C::TT>(p, s, G);
     const int ns = n_splits_of(si, chunk);
-    int local = w - item_start[s];
+    int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
     const int j = local % p.num_kv_heads;
     local /= p.num_kv_heads;
     const int split = local % ns;
     const int rt = local / ns;
-    process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, split, ns, chunk, slot_start[s] + j * ns);
+    process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, split, ns, chunk,
+                                __builtin_amdgcn_readfirstlane(slot_start[s]) + j * ns);
   }
 }
 
@@ -508,7 +547,7 @@ bool tiled_supported(const RpaParams& p) {
   if (p.flags & RPA_FLAG_FORCE_GENERIC) return false;
   if (p.dtype != RPA_DTYPE_BF16 || p.compute != RPA_COMPUTE_BF16) return false;
   if (p.head_dim != 128 && p.head_dim != 256) return false;
-  if (p.page_size % 4 != 0) return false;
+  if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
   if (p.max_num_seqs > kTiledMaxSeqs) return false;
   if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kWorkspaceTicketBytes) return false;
   return true;
@@ -543,7 +582,8 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.p = p;
   a.target_items = min(kTiledTargetItems, max(64, env_int("RPA_TUNE_TARGET_ITEMS", kTiledTargetItems)));
   a.user_chunk = p.num_kv_pages_per_block > 0 ? p.num_kv_pages_per_block * p.page_size : 0;
-  a.page_shift = (p.page_size & (p.page_size - 1)) == 0 ? __builtin_ctz(p.page_size) : -1;
+  a.page_shift = __builtin_ctz(p.page_size);
+  a.uniform_page = p.page_size >= 16;
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
