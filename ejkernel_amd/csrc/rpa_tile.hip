@@ -1,12 +1,16 @@
 // Ragged paged attention on MFMA, one wavefront per work item, one launch per batch.
 //
-// Work item = (sequence, kv head, 16-row tile of the sequence's (query token, group head)
-// rows, split of the key range).  A decode sequence (1-4 query tokens) is a single row
-// tile whose key range is split along the sequence; the partial (m, l, O) of each split
-// goes to the workspace and the last split to arrive (an atomic ticket per sequence and
-// kv head) merges them in split order, so results do not depend on timing.  Work is
-// discovered on the device from query_start_loc / context_lens / num_seqs; the host
-// never reads them.
+// Rows of a sequence are its (query token, group head) pairs, handled 16 at a time (one
+// MFMA tile) per kv head.  A decode sequence (1-4 query tokens) has a single row tile.
+// All decode sequences of the batch form one stream of 32-key tiles ordered by
+// (sequence, kv head, position); every wavefront of the grid takes an equal contiguous
+// share of that stream, whatever the individual lengths are.  A wavefront whose share
+// covers only part of a (sequence, kv head) writes its partial (m, l, O) to the workspace
+// and takes a ticket; the last part to arrive merges all parts in stream order, so the
+// result does not depend on timing.  Sequences with more rows (prefill chunks) are
+// handled as (sequence, kv head, row tile) items over the full key range of the tile.
+// Work is discovered on the device from query_start_loc / context_lens / num_seqs; the
+// host never reads them.
 //
 // Per iteration a wavefront streams TT = 16*NT tokens of its kv head: K and V rows are
 // fetched with 16-byte loads in which each quarter-wave reads one whole contiguous row
@@ -37,19 +41,43 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 struct TileArgs {
   RpaParams p;
-  int target_items;   // upper bound used to size split length (and the workspace)
-  int user_chunk;     // tokens per split requested by the caller, 0 = automatic
   int page_shift;     // log2(page_size)
   int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
   uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
-  float* partial_o;   // [slots][16][D]
-  float* partial_ml;  // [slots][16][2]
+  float* partial_o;   // [2 * wavefronts of the grid][16][D]
+  float* partial_ml;  // [2 * wavefronts of the grid][16][2]
 };
+
+// Split of the decode stream over the wavefronts of the grid: the first `rem` wavefronts take q + 1 tiles, the
+// others q, so shares differ by at most one tile and empty shares (q == 0) only occur at the end.
+struct Shares {
+  int q, rem;
+  __device__ __forceinline__ int begin(int w) const { return w * q + min(w, rem); }
+  __device__ __forceinline__ int owner(int x) const {
+    const int big = rem * (q + 1);
+    return x < big ? x / (q + 1) : rem + (x - big) / q;
+  }
+};
+
+// A wavefront's part of one (sequence, kv head) of the decode stream.
+struct Part {
+  bool partial;         // the (sequence, kv head) is shared with other wavefronts
+  int slot;             // workspace slot of this part
+  int first_w, last_w;  // wavefronts sharing it (every one of them holds at least one of its tiles)
+  int stream_a;         // stream index of its first tile
+  Shares sh;
+};
+
+// Workspace slot of wavefront k's part of the (sequence, kv head) starting at stream tile stream_a: a wavefront
+// has at most two partial parts, the one its share starts inside (slot 2k) and the one it ends inside (2k + 1).
+__device__ __forceinline__ int part_slot(int k, int stream_a, const Shares& sh) {
+  return 2 * k + (sh.begin(k) < stream_a ? 1 : 0);
+}
 
 struct SeqInfo {
   int q0, q_len, kv_len, rows, n_rt;
   int lo_al, hi;  // key range of the whole sequence, start aligned down to the tile
-  bool eligible;  // single row tile: may be split along the keys
+  bool eligible;  // single row tile with keys: part of the decode stream
 };
 
 template <int TT>
@@ -60,18 +88,12 @@ __device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
   si.kv_len = p.context_lens[s];
   si.rows = si.q_len > 0 ? si.q_len * G : 0;
   si.n_rt = (si.rows + 15) >> 4;
-  si.eligible = si.n_rt == 1;
   const int pos_min = si.kv_len - si.q_len;
   int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
   si.lo_al = lo & ~(TT - 1);
   si.hi = max(si.kv_len, 0);
+  si.eligible = si.n_rt == 1 && si.hi > si.lo_al;  // a sequence without keys stays an item: its rows become zero
   return si;
-}
-
-__device__ __forceinline__ int n_splits_of(const SeqInfo& si, int chunk) {
-  if (!si.eligible) return 1;
-  const int span = si.hi - si.lo_al;
-  return span <= chunk ? 1 : (span + chunk - 1) / chunk;
 }
 
 // Exclusive prefix sum of one int per thread over the workgroup; `total` gets the sum.
@@ -120,7 +142,7 @@ struct Cfg {
 // Everything one wavefront needs for one work item.
 template <int D, int NT, bool kMimic>
 __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
-                                             int j, int rt, int split, int n_splits, int chunk, int slot_base) {
+                                             int j, int rt, int range_lo, int range_hi, const Part& part) {
   using C = Cfg<D, NT, kMimic>;
   const RpaParams& p = a.p;
   const int lane = threadIdx.x & (kWave - 1);
@@ -135,12 +157,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const int row_lo = rt * 16, row_hi = min(row_lo + 16, si.rows);
   const int qi_min = row_lo / G, qi_max = (row_hi - 1) / G;
   const int pos_min = si.kv_len - si.q_len + qi_min, pos_max = si.kv_len - si.q_len + qi_max;
-  int range_hi = min(si.kv_len, pos_max + 1);
-  int range_lo = (W > 0 ? max(0, pos_min - W + 1) : 0) & ~(C::TT - 1);
-  if (n_splits > 1) {
-    range_lo = si.lo_al + split * chunk;
-    range_hi = min(range_hi, range_lo + chunk);
-  }
   // this lane's row
   const int R = row_lo + i;
   const bool row_valid = R < si.rows;
@@ -358,12 +374,12 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   l_run += __shfl_xor(l_run, 16, kWave);
   l_run += __shfl_xor(l_run, 32, kWave);
 
-  if (n_splits > 1) {
-    // ---- partial to the workspace, then take a ticket; the last split merges all of them in split order.
+  if (part.partial) {
+    // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
     // Partials are written and read with agent-scope relaxed atomics (write-through / cache-bypassing accesses),
     // so no L2 write-back or invalidate is needed around the ticket: it is enough that this wave's stores have
     // completed (the workgroup-scope release waits for them) before the ticket is taken.
-    const size_t slot = static_cast<size_t>(slot_base + split);
+    const size_t slot = static_cast<size_t>(part.slot);
     if (row_valid) {
       uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
 #pragma unroll
@@ -387,13 +403,14 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     uint32_t ticket = 0;
     if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     ticket = __shfl(ticket, 0, kWave);
-    if (ticket != static_cast<uint32_t>(n_splits - 1)) return;
+    if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + static_cast<size_t>(slot_base) * 16 + i;
+    const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
     float M = -INFINITY;
     if (row_valid)
-      for (int k = 0; k < n_splits; ++k) {
-        const uint64_t v = __hip_atomic_load(ml + static_cast<size_t>(k) * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int k = part.first_w; k <= part.last_w; ++k) {
+        const size_t sl = part_slot(k, part.stream_a, part.sh);
+        const uint64_t v = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v)));
       }
     const float M_use = M == -INFINITY ? 0.f : M;
@@ -403,12 +420,13 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (row_valid) {
-      for (int k = 0; k < n_splits; ++k) {
-        const uint64_t mlv = __hip_atomic_load(ml + static_cast<size_t>(k) * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      for (int k = part.first_w; k <= part.last_w; ++k) {
+        const size_t sl = part_slot(k, part.stream_a, part.sh);
+        const uint64_t mlv = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const float mk = __uint_as_float(static_cast<uint32_t>(mlv)), lk = __uint_as_float(static_cast<uint32_t>(mlv >> 32));
         const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
         L += w * lk;
-        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + ((static_cast<size_t>(slot_base) + k) * 16 + i) * D);
+        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -460,50 +478,40 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   const RpaParams& p = a.p;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int G = p.num_q_heads / p.num_kv_heads;
-  // LDS: [4 waves x K tile][item_start: S+1][slot_start: S+1][scratch 8 ints]
+  // LDS: [4 waves x K tile][item_start: S+1][tile_start: S+1][scratch 8 ints]
   char* lds_k = smem + wave * C::LDS_PER_WAVE;
   int* item_start = reinterpret_cast<int*>(smem + kWgWaves * C::LDS_PER_WAVE);
-  int* slot_start = item_start + (p.max_num_seqs + 1);
-  int* scratch = slot_start + (p.max_num_seqs + 1);
+  int* tile_start = item_start + (p.max_num_seqs + 1);
+  int* scratch = tile_start + (p.max_num_seqs + 1);
 
   int nseq = p.num_seqs[0];
   nseq = min(max(nseq, 0), p.max_num_seqs);
 
-  // ---- schedule: split length from the batch's total decode keys, then items and partial slots per sequence
+  // ---- schedule: per sequence, tiles it adds to the decode stream (single row tile) or items (more row tiles)
   const int per = (nseq + kWgThreads - 1) / kWgThreads;
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
-  int my_tok = 0;
+  int my_items = 0, my_tiles = 0;
   for (int s = s_begin; s < s_end; ++s) {
     const SeqInfo si = seq_info<C::TT>(p, s, G);
-    if (si.eligible) my_tok += (si.hi - si.lo_al + 63) >> 6;  // in units of 64 keys: no overflow
+    if (si.eligible) my_tiles += p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
+    else my_items += p.num_kv_heads * si.n_rt;
   }
-  int tot64;
-  block_excl_scan(my_tok, scratch, tot64);
-  long long want = (static_cast<long long>(tot64) * 64 * p.num_kv_heads + a.target_items - 1) / a.target_items;
-  int chunk = static_cast<int>(min(want, static_cast<long long>(1) << 30));
-  chunk = max(chunk, a.user_chunk > 0 ? a.user_chunk : 4 * C::TT);
-  chunk = __builtin_amdgcn_readfirstlane((chunk + C::TT - 1) & ~(C::TT - 1));
-
-  int my_items = 0, my_slots = 0;
-  for (int s = s_begin; s < s_end; ++s) {
-    const SeqInfo si = seq_info<C::TT>(p, s, G);
-    const int ns = n_splits_of(si, chunk);
-    my_items += p.num_kv_heads * si.n_rt * ns;
-    my_slots += ns > 1 ? p.num_kv_heads * ns : 0;
-  }
-  int total_items, total_slots;
+  int total_items, total_tiles;
   int item_base = block_excl_scan(my_items, scratch, total_items);
-  int slot_base = block_excl_scan(my_slots, scratch, total_slots);
+  int tile_base = block_excl_scan(my_tiles, scratch, total_tiles);
   for (int s = s_begin; s < s_end; ++s) {
     const SeqInfo si = seq_info<C::TT>(p, s, G);
-    const int ns = n_splits_of(si, chunk);
     item_start[s] = item_base;
-    slot_start[s] = slot_base;
-    item_base += p.num_kv_heads * si.n_rt * ns;
-    slot_base += ns > 1 ? p.num_kv_heads * ns : 0;
+    tile_start[s] = tile_base;
+    if (si.eligible) tile_base += p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
+    else item_base += p.num_kv_heads * si.n_rt;
   }
   total_items = __builtin_amdgcn_readfirstlane(total_items);
-  if (tid == 0) item_start[nseq] = total_items;
+  total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
+  if (tid == 0) {
+    item_start[nseq] = total_items;
+    tile_start[nseq] = total_tiles;
+  }
   __syncthreads();
 
   // ---- rows past the ragged batch are zero
@@ -515,24 +523,58 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       for (int k = tid; k < row_u4; k += kWgThreads) o4[static_cast<size_t>(row) * row_u4 + k] = u32x4_t{0u, 0u, 0u, 0u};
   }
 
-  // ---- items, strided over all wavefronts of the grid
-  const int n_waves = gridDim.x * kWgWaves;
-  for (int w = blockIdx.x * kWgWaves + wave; w < total_items; w += n_waves) {
-    int lo = 0, hi = nseq;  // largest s with item_start[s] <= w
+  const int n_workers = gridDim.x * kWgWaves;
+  const int worker = blockIdx.x * kWgWaves + wave;
+  // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
+  // are skipped because the search keeps the last one that does not exceed x.
+  auto find = [&](const int* start, int x) {
+    int lo = 0, hi = nseq;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
-      if (item_start[mid] <= w) lo = mid; else hi = mid;
+      if (start[mid] <= x) lo = mid; else hi = mid;
     }
-    const int s = __builtin_amdgcn_readfirstlane(lo);
+    return __builtin_amdgcn_readfirstlane(lo);
+  };
+
+  // ---- sequences with several row tiles: one item per (sequence, row tile, kv head), strided over the grid
+  for (int w = worker; w < total_items; w += n_workers) {
+    const int s = find(item_start, w);
     const SeqInfo si = seq_info<C::TT>(p, s, G);
-    const int ns = n_splits_of(si, chunk);
-    int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
-    const int j = local % p.num_kv_heads;
-    local /= p.num_kv_heads;
-    const int split = local % ns;
-    const int rt = local / ns;
-    process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, split, ns, chunk,
-                                __builtin_amdgcn_readfirstlane(slot_start[s]) + j * ns);
+    const int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
+    const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
+    const int row_hi = min(rt * 16 + 16, si.rows);
+    const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
+    const int range_hi = min(si.kv_len, pos_max + 1);
+    const int range_lo = (p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0) & ~(C::TT - 1);
+    Part part;
+    part.partial = false;
+    process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+  }
+
+  // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
+  if (total_tiles > 0) {
+    Shares sh;
+    sh.q = total_tiles / n_workers;
+    sh.rem = total_tiles - sh.q * n_workers;
+    int x = sh.begin(worker);
+    const int x_end = sh.begin(worker + 1);
+    while (x < x_end) {
+      const int s = find(tile_start, x);
+      const SeqInfo si = seq_info<C::TT>(p, s, G);
+      const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
+      const int local = __builtin_amdgcn_readfirstlane(x - tile_start[s]);
+      const int j = local / per_head, t0 = local - j * per_head;
+      const int t1 = min(per_head, t0 + (x_end - x));
+      Part part;
+      part.stream_a = x - t0;
+      part.sh = sh;
+      part.first_w = sh.owner(part.stream_a);
+      part.last_w = sh.owner(part.stream_a + per_head - 1);
+      part.partial = part.first_w != part.last_w;
+      part.slot = part_slot(worker, part.stream_a, sh);
+      process_item<D, NT, kMimic>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+      x += t1 - t0;
+    }
   }
 }
 
@@ -541,6 +583,13 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 static int env_int(const char* name, int dflt) {
   const char* v = getenv(name);
   return v && *v ? atoi(v) : dflt;
+}
+
+// Workgroups of the persistent grid: one per compute unit (four wavefronts each) measured best for the
+// bandwidth-bound decode stream; RPA_TUNE_WGS_PER_CU overrides it for experiments (1..kTiledMaxWgsPerCu).
+static int tiled_grid() {
+  const int per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 1)));
+  return device_cu_count() * per_cu;
 }
 
 bool tiled_supported(const RpaParams& p) {
@@ -554,8 +603,7 @@ bool tiled_supported(const RpaParams& p) {
 }
 
 void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
-  const uint64_t n_ctr = static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads;
-  const uint64_t slots = static_cast<uint64_t>(kTiledTargetItems) + n_ctr;
+  const uint64_t slots = 2ull * kWgWaves * tiled_grid();  // two partial parts per wavefront at most
   // The ticket region has one size for every shape: a workspace reused across shapes must never hold
   // partial results where another shape keeps its tickets.
   wl->counters_bytes = kWorkspaceTicketBytes;
@@ -580,15 +628,13 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
   TileArgs a;
   a.p = p;
-  a.target_items = min(kTiledTargetItems, max(64, env_int("RPA_TUNE_TARGET_ITEMS", kTiledTargetItems)));
-  a.user_chunk = p.num_kv_pages_per_block > 0 ? p.num_kv_pages_per_block * p.page_size : 0;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
-  const int grid = device_cu_count() * max(1, env_int("RPA_TUNE_WGS_PER_CU", 2));
+  const int grid = tiled_grid();
   const bool mimic = env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
   if (p.head_dim == 128) return mimic ? launch_cfg<128, 2, true>(a, grid, stream) : launch_cfg<128, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, true>(a, grid, stream) : launch_cfg<256, 1, false>(a, grid, stream);
