@@ -32,6 +32,9 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
+                    help="instead of the benchmark, run a plain device copy of MIB MiB --steps times (a kernel of "
+                         "known traffic, used to scale the FETCH_SIZE / WRITE_SIZE counters)")
     return ap.parse_args()
 
 
@@ -99,6 +102,19 @@ def main():
     _native.load()  # fail loudly before any timing if the HIP library is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
+    if args.copy_probe:
+        n = args.copy_probe << 20
+        src = torch.full((n,), 7, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / args.steps
+        print(json.dumps({"copy_probe_bytes_read": n, "copy_probe_bytes_written": n, "steps": args.steps,
+                          "ms_per_copy": dt * 1e3, "gbps_read_plus_write": 2 * n / dt / 1e9}))
+        return
     batch = make_workload(args.workload, device=dev, scale=args.scale)
     m = batch.meta
     counts = algorithmic_counts(batch.q_lens, batch.kv_lens, num_q_heads=m["num_q_heads"],
