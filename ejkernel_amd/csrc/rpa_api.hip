@@ -43,6 +43,13 @@ static int validate(const RpaParams& p, bool need_pointers) {
   return RPA_OK;
 }
 
+// Clears the ticket region with a kernel rather than hipMemsetAsync, so the call may be recorded into a HIP graph.
+__global__ void zero_fill_kernel(uint4* dst, size_t n16) {
+  for (size_t k = blockIdx.x * static_cast<size_t>(blockDim.x) + threadIdx.x; k < n16;
+       k += static_cast<size_t>(gridDim.x) * blockDim.x)
+    dst[k] = make_uint4(0u, 0u, 0u, 0u);
+}
+
 int device_cu_count() {
   static std::atomic<int> cache[64];
   int dev = 0;
@@ -75,8 +82,12 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
   // leaves them at zero again.
   if (workspace == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "workspace is null");
   const uint64_t n = workspace_bytes < rpa::kWorkspaceTicketBytes ? workspace_bytes : rpa::kWorkspaceTicketBytes;
-  if (hipMemsetAsync(workspace, 0, n, static_cast<hipStream_t>(hip_stream)) != hipSuccess)
-    return rpa::fail(RPA_ERR_LAUNCH, "hipMemsetAsync on the workspace failed");
+  if ((reinterpret_cast<uintptr_t>(workspace) & 15u) != 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "workspace must be 16-byte aligned");
+  if (n >= 16) {
+    hipLaunchKernelGGL(rpa::zero_fill_kernel, dim3(64), dim3(256), 0, static_cast<hipStream_t>(hip_stream),
+                       static_cast<uint4*>(workspace), static_cast<size_t>(n / 16));
+    if (hipGetLastError() != hipSuccess) return rpa::fail(RPA_ERR_LAUNCH, "clearing the workspace tickets failed");
+  }
   return RPA_OK;
 }
 
