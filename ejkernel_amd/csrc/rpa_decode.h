@@ -1,0 +1,350 @@
+// Wave-level attention loop: one wavefront streams a key range of one (sequence, kv head) for up to 16 rows.
+#pragma once
+
+#include "rpa_tile_common.h"
+
+namespace rpa {
+
+template <int D, int NT, bool kMimic>
+struct Cfg {
+  static constexpr int NS = D / 128;        // 128-wide slices of head_dim
+  static constexpr int NKS = D / 32;        // k-steps of the QK^T contraction
+  static constexpr int TT = 16 * NT;        // tokens per iteration
+  static constexpr int NSLOT = 4 * NT;      // tokens each lane fetches per iteration
+  static constexpr int ROWB = D * 2 + 16;   // LDS bytes per K row (16 B pad: conflict-free b128 reads)
+  static constexpr int LDS_PER_WAVE = TT * ROWB;
+};
+
+// Everything one wavefront needs for one work item.
+template <int D, int NT, bool kMimic>
+__device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
+                                             int j, int rt, int range_lo, int range_hi, const Part& part) {
+  using C = Cfg<D, NT, kMimic>;
+  const RpaParams& p = a.p;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int i = lane & 15, g = lane >> 4;
+  const int G = p.num_q_heads / p.num_kv_heads;
+  const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
+  const bf16_t* __restrict__ kv = static_cast<const bf16_t*>(p.kv_pages);
+  bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
+  const int W = p.sliding_window;
+
+  // ---- rows of this tile and their key range
+  const int row_lo = rt * 16, row_hi = min(row_lo + 16, si.rows);
+  const int qi_min = row_lo / G, qi_max = (row_hi - 1) / G;
+  const int pos_min = si.kv_len - si.q_len + qi_min, pos_max = si.kv_len - si.q_len + qi_max;
+  // this lane's row
+  const int R = row_lo + i;
+  const bool row_valid = R < si.rows;
+  const int qi = row_valid ? R / G : 0;
+  const int hg = row_valid ? R - qi * G : 0;
+  const int pos_n = row_valid ? si.kv_len - si.q_len + qi : -1;
+  const int head = j * G + hg;
+  const size_t q_row_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * D;
+
+  // ---- Q^T operands: lane (row i, group g) holds q[row][32 ks + 8 g .. +8], pre-scaled and rounded to bf16
+  bf16x8_t qreg[C::NKS];
+  {
+    const float scale = rbf(p.softmax_scale);
+#pragma unroll
+    for (int ks = 0; ks < C::NKS; ++ks) {
+      u32x4_t raw = {0u, 0u, 0u, 0u};
+      if (row_valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
+      u32x4_t sc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = __uint_as_float(raw[e] << 16) * scale, hi = __uint_as_float(raw[e] & 0xffff0000u) * scale;
+        sc[e] = pack_bf16x2(lo, hi);
+      }
+      qreg[ks] = __builtin_bit_cast(bf16x8_t, sc);
+    }
+  }
+
+  f32x4_t o_acc[C::NS][8];
+#pragma unroll
+  for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+    for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;  // elements between tokens
+  const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
+  // Same row through the constant address space: reads with a wave-uniform index become scalar loads, which
+  // are counted apart from the vector loads of the K/V stream.  The block table is never written by this kernel.
+  const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(bt));
+  const int t_last = range_hi - 1;
+  const float cap = p.logits_soft_cap;
+
+  u32x4_t kreg[C::NSLOT][C::NS];
+  u32x4_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
+
+  // Fetch K and V of the TT tokens starting at `tile`: lane (i, g) takes tokens 16u + 4g + r (u < NT, r < 4),
+  // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.
+  //
+  // Fast path (page_size >= 16, tile entirely inside the range): a 16-token sub-tile sits in one page, so the
+  // block-table entry is a scalar load (it does not share the vector-memory counter with the K/V stream) and
+  // the row address is a scalar base plus one per-lane byte offset that is constant for the whole item.
+  // Slow path (last tile of a range, small pages): per-lane page lookup; tokens past the end of the range are
+  // replaced by the last valid one (their scores are masked).
+  const char* kvb = reinterpret_cast<const char*>(kv);
+  const uint32_t stride_b = static_cast<uint32_t>(tok_stride) * 2u;  // bytes between tokens
+  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + static_cast<uint32_t>(2 * j * D * 2 + 16 * i);
+  auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
+    if (a.uniform_page && tile + C::TT <= range_hi) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        const int t16 = tile + 16 * u;
+        int page = bt_c[t16 >> a.page_shift];
+        page = min(max(page, 0), p.num_pages - 1);
+        const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                            static_cast<uint64_t>(t16 & (p.page_size - 1)) * stride_b;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const char* row = sbase + static_cast<uint64_t>(r) * stride_b;
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN) {
+            kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN));
+            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN + 2u * D));
+          }
+        }
+      }
+      return;
+    }
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      const int t4c = min(tile + 16 * u + 4 * g, t_last & ~3);
+      const int rlim = min(3, t_last - t4c);
+      int page = bt[t4c >> a.page_shift];
+      page = min(max(page, 0), p.num_pages - 1);
+      const char* base = kvb + static_cast<uint64_t>(page) * page_b +
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (2 * j * D * 2 + 16 * i);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN) {
+          kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN);
+          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN + 2 * D);
+        }
+      }
+    }
+  };
+
+  auto body = [&](int tile, u32x4_t (&vcur)[C::NSLOT][C::NS], u32x4_t (&vnext)[C::NSLOT][C::NS]) {
+    // 1. K rows to the wave-private LDS tile: row = token within the tile, 16-byte piece i (+16 per slice)
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+          *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kreg[4 * u + r][sN];
+    // 2. next tile's K and V are requested now, a full iteration before they are needed
+    if (tile + C::TT < range_hi) issue_loads(tile + C::TT, kreg, vnext);
+    // 3. S^T = K Q^T: lane (token i of sub-tile u, group g) reads piece 4 ks + g of its row
+    f32x4_t s_acc[NT];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      s_acc[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < C::NKS; ++ks) {
+        const u32x4_t kop = *reinterpret_cast<const u32x4_t*>(lds_k + (16 * u + i) * C::ROWB + 16 * (4 * ks + g));
+        s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop), qreg[ks], s_acc[u], 0, 0, 0);
+      }
+    }
+    // 4. online softmax; this lane: query row i, tokens tile + 16u + 4g + r
+    float sv[NT][4];
+    const bool need_mask = (tile + C::TT > range_hi) || (tile + C::TT - 1 > pos_min) || (W > 0 && tile <= pos_max - W);
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r];
+    if (cap != 0.f) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
+    }
+    if (need_mask) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int tok = tile + 16 * u + 4 * g + r;
+          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W);
+          sv[u][r] = keep ? sv[u][r] : -INFINITY;
+        }
+    }
+    float tmax = -INFINITY;
+#pragma unroll
+    for (int u = 0; u < NT; ++u)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, sv[u][r]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    const float m_new = fmaxf(m_run, tmax);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
+    float psum = 0.f;
+    uint32_t pw[2 * NT];
+#pragma unroll
+    for (int u = 0; u < NT; ++u) {
+      float pv[4];
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        float d = sv[u][r] - m_use;
+        if (kMimic) d = rbf(d);
+        float e = __builtin_amdgcn_exp2f(d * kLog2e);
+        e = rbf(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
+        pv[r] = e;
+        psum += e;
+      }
+      pw[2 * u] = (__float_as_uint(pv[0]) >> 16) | (__float_as_uint(pv[1]) & 0xffff0000u);
+      pw[2 * u + 1] = (__float_as_uint(pv[2]) >> 16) | (__float_as_uint(pv[3]) & 0xffff0000u);
+    }
+    l_run = l_run * alpha + psum;
+    m_run = m_new;
+    if (__any(alpha != 1.f)) {
+#pragma unroll
+      for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o_acc[sN][c] *= alpha;
+    }
+    // 5. O^T += V^T P^T.  MFMA number c of slice sN yields d = 128 sN + 8 (row of the MFMA) + c; its A operand is
+    //    column c of every fetched 8-wide piece, gathered from the token rows by byte permutes.
+#pragma unroll
+    for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) {
+        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+        uint32_t aw[2 * NT];
+#pragma unroll
+        for (int h = 0; h < 2 * NT; ++h)
+          aw[h] = __builtin_amdgcn_perm(vcur[2 * h + 1][sN][c >> 1], vcur[2 * h][sN][c >> 1], sel);
+        if constexpr (NT == 2) {
+          const u32x4_t av = {aw[0], aw[1], aw[2], aw[3]};
+          const u32x4_t pvv = {pw[0], pw[1], pw[2], pw[3]};
+          o_acc[sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
+                                                                 __builtin_bit_cast(bf16x8_t, pvv), o_acc[sN][c], 0, 0, 0);
+        } else {
+          const u32x2_t av = {aw[0], aw[1]};
+          const u32x2_t pvv = {pw[0], pw[1]};
+          o_acc[sN][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, av),
+                                                                   __builtin_bit_cast(s16x4_t, pvv), o_acc[sN][c], 0, 0, 0);
+        }
+      }
+  };
+
+  if (range_hi > range_lo) {
+    issue_loads(range_lo, kreg, vbuf0);
+    for (int tile = range_lo; tile < range_hi; tile += 2 * C::TT) {
+      body(tile, vbuf0, vbuf1);
+      if (tile + C::TT >= range_hi) break;
+      body(tile + C::TT, vbuf1, vbuf0);
+    }
+  }
+
+  // ---- row sum across the four lane groups
+  l_run += __shfl_xor(l_run, 16, kWave);
+  l_run += __shfl_xor(l_run, 32, kWave);
+
+  if (part.partial) {
+    // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
+    // Partials are written and read with agent-scope relaxed atomics (write-through / cache-bypassing accesses),
+    // so no L2 write-back or invalidate is needed around the ticket: it is enough that this wave's stores have
+    // completed (the workgroup-scope release waits for them) before the ticket is taken.
+    const size_t slot = static_cast<size_t>(part.slot);
+    if (row_valid) {
+      uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
+#pragma unroll
+      for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint64_t v = static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e][r])) |
+                               (static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e + 1][r])) << 32);
+            __hip_atomic_store(po + (128 * sN + 32 * g + 8 * r) / 2 + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          }
+      if (g == 0) {
+        const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_run)) | (static_cast<uint64_t>(__float_as_uint(l_run)) << 32);
+        __hip_atomic_store(reinterpret_cast<uint64_t*>(a.partial_ml) + slot * 16 + i, v, __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    uint32_t* ctr = a.counters + static_cast<size_t>(s) * p.num_kv_heads + j;
+    uint32_t ticket = 0;
+    if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    ticket = __shfl(ticket, 0, kWave);
+    if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
+    float M = -INFINITY;
+    if (row_valid)
+      for (int k = part.first_w; k <= part.last_w; ++k) {
+        const size_t sl = part_slot(k, part.stream_a, part.sh);
+        const uint64_t v = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v)));
+      }
+    const float M_use = M == -INFINITY ? 0.f : M;
+    float L = 0.f;
+#pragma unroll
+    for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    if (row_valid) {
+      for (int k = part.first_w; k <= part.last_w; ++k) {
+        const size_t sl = part_slot(k, part.stream_a, part.sh);
+        const uint64_t mlv = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float mk = __uint_as_float(static_cast<uint32_t>(mlv)), lk = __uint_as_float(static_cast<uint32_t>(mlv >> 32));
+        const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
+        L += w * lk;
+        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const uint64_t v = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+              o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(v));
+              o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(v >> 32));
+            }
+      }
+    }
+    m_run = M;
+    l_run = L;
+    if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
+  // ---- normalise (with optional sinks) and store
+  if (!row_valid) return;
+  float num_scale = 1.f, denom = l_run;
+  if (p.sinks != nullptr && p.num_sinks > 0) {
+    const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
+    float smax = -INFINITY;
+    for (int k = 0; k < p.num_sinks; ++k) smax = fmaxf(smax, sk[k]);
+    const float mt = fmaxf(m_run, smax);
+    float ssum = 0.f;
+    for (int k = 0; k < p.num_sinks; ++k) ssum += expf(sk[k] - mt);
+    num_scale = m_run == -INFINITY ? 0.f : expf(m_run - mt);
+    denom = num_scale * l_run + ssum;
+  }
+  const float inv = num_scale / fmaxf(denom, 1e-6f);
+  bf16_t* orow = out + q_row_off;
+#pragma unroll
+  for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      u32x4_t w;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[sN][2 * e][r] * inv, o_acc[sN][2 * e + 1][r] * inv);
+      *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+    }
+}
+
+}  // namespace rpa

@@ -1,0 +1,292 @@
+// Workgroup-level attention tile for sequences with many rows (prefill chunks).
+//
+// One workgroup (4 wavefronts) owns WGROWS = 4 * 16 * MRT consecutive rows of one sequence and
+// one kv head -- (query token, group head) pairs, so 64 tokens x 4 heads at MRT = 4, G = 4 --
+// and walks the keys those rows can see once.  K and V tiles of TK tokens go from HBM straight
+// into a double-buffered LDS tile with 16-byte direct-to-LDS loads (global_load_lds_dwordx4: no
+// staging registers; 16 consecutive lanes read one contiguous 256-byte row), issued one step
+// ahead: one barrier per step.  Rows are stored unpadded with their 16-byte pieces XOR-swizzled
+// by the row number, which keeps both MFMA operand read patterns free of bank conflicts.  Each
+// wavefront then computes S^T = K Q^T and O^T += V^T P^T for its own 16 * MRT rows: every K and V operand read from LDS feeds MRT MFMAs, Q stays in registers, and
+// each lane owns one row per row tile, so the online softmax is lane-local as in the decode loop.
+// The row sums come from one extra MFMA against a vector of ones (they add exactly the bf16
+// probabilities that enter P V).  Halves of a step that lie entirely in a wavefront's causal
+// future or left of its window are skipped.
+#pragma once
+
+#include "rpa_tile_common.h"
+
+namespace rpa {
+
+template <int D, int MRT>
+struct PCfg {
+  static constexpr int NS = D / 128;                 // 128-wide slices of head_dim
+  static constexpr int NKS = D / 32;                 // k-steps of the QK^T contraction
+  static constexpr int NH = D == 128 ? 2 : 1;        // 32-token halves per step
+  static constexpr int TK = 32 * NH;                 // tokens per step
+  static constexpr int ROWB = D * 2;                 // LDS bytes per row
+  static constexpr int WROWS = 16 * MRT;             // rows per wavefront
+  static constexpr int WGROWS = kWgWaves * WROWS;    // rows per workgroup
+  static constexpr int TILE_B = TK * ROWB;           // one K (or V) tile: 16 KiB
+  static constexpr int LDS = 4 * TILE_B;             // K and V, double buffered
+  static constexpr int PR = D / 8;                   // 16-byte pieces per row
+  static constexpr int RB = kWave / PR;              // rows one wave-wide load instruction covers
+  static constexpr int BLOCKS = TK / RB;             // load instructions per K (or V) tile: 16
+  static constexpr int BPW = 2 * BLOCKS / kWgWaves;  // load instructions per wavefront and step
+};
+
+template <int D, int MRT, bool kMimic>
+__device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
+                                             int qt) {
+  using C = PCfg<D, MRT>;
+  const RpaParams& p = a.p;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int i = lane & 15, g = lane >> 4;
+  const int G = p.num_q_heads / p.num_kv_heads;
+  const int W = p.sliding_window;
+  const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
+  bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
+  const char* kvb = static_cast<const char*>(p.kv_pages);
+  const float cap = p.logits_soft_cap;
+  const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
+
+  // ---- key range of the workgroup's rows
+  const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
+  const int wg_pos_min = pos0 + wg_row_lo / G, wg_pos_max = pos0 + (wg_row_hi - 1) / G;
+  const int range_hi = min(si.kv_len, wg_pos_max + 1);
+  const int range_lo = (W > 0 ? max(0, wg_pos_min - W + 1) : 0) & ~(C::TK - 1);
+  const int t_last = range_hi - 1;
+
+  // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
+  const int w_row_lo = wg_row_lo + wave * C::WROWS;
+  bool row_valid[MRT];
+  int pos_n[MRT];
+  size_t q_off[MRT];
+  int head[MRT];
+  int t_pos_lo[MRT], t_pos_hi[MRT];  // positions spanned by the valid rows of the row tile (wave-uniform)
+  bool t_any[MRT];
+  bf16x8_t qreg[MRT][C::NKS];
+  const float scale = rbf(p.softmax_scale);
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    const int R = w_row_lo + 16 * m + i;
+    row_valid[m] = R < si.rows;
+    const int qi = row_valid[m] ? R / G : 0;
+    head[m] = j * G + (row_valid[m] ? R - qi * G : 0);
+    pos_n[m] = row_valid[m] ? pos0 + qi : -1;
+    q_off[m] = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head[m]) * D;
+    const int tr_lo = w_row_lo + 16 * m, tr_hi = min(tr_lo + 16, si.rows);
+    t_any[m] = tr_hi > tr_lo;
+    t_pos_lo[m] = pos0 + tr_lo / G;
+    t_pos_hi[m] = pos0 + (max(tr_hi, tr_lo + 1) - 1) / G;
+#pragma unroll
+    for (int ks = 0; ks < C::NKS; ++ks) {
+      u32x4_t raw = {0u, 0u, 0u, 0u};
+      if (row_valid[m]) raw = *reinterpret_cast<const u32x4_t*>(q + q_off[m] + 32 * ks + 8 * g);
+      u32x4_t sc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        sc[e] = pack_bf16x2(__uint_as_float(raw[e] << 16) * scale, __uint_as_float(raw[e] & 0xffff0000u) * scale);
+      qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
+    }
+  }
+  const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;  // < w_pos_lo when the wave has no rows
+  const int w_pos_lo = pos0 + w_row_lo / G;
+  const bool w_any = w_row_lo < si.rows;
+
+  f32x4_t o_acc[MRT][C::NS][8];
+  f32x4_t l_acc[MRT];
+  float m_run[MRT];
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    m_run[m] = -INFINITY;
+    l_acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+      for (int c = 0; c < 8; ++c) o_acc[m][sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- cooperative fetch.  Block b of a step (b < BLOCKS: K rows RB*b .., else V rows) is one wave-wide
+  // direct-to-LDS load: the LDS side is 1 KiB in lane order, so lane l fills piece slot l % PR of row l / PR and
+  // fetches the piece that the swizzle assigns to that slot.  The RB rows of a block share a page (RB <= 4 <=
+  // page_size), so the block-table entry is a scalar load.
+  const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * D) * 2u;
+  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
+  const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
+      reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
+  const int l_row = lane / C::PR, l_slot = lane % C::PR;
+  auto fetch_tile = [&](int tile, int buf) {
+#pragma unroll
+    for (int n = 0; n < C::BPW; ++n) {
+      const int b = wave + kWgWaves * n;          // 0 .. 2*BLOCKS-1
+      const int is_v = b / C::BLOCKS, rb = b % C::BLOCKS;
+      const int t_c = min(tile + C::RB * rb, t_last & ~(C::RB - 1));  // past the range: repeat the last keys (masked)
+      const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
+      const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b;
+      const int tok = min(t_c + l_row, t_last);
+      const int t_local = C::RB * rb + l_row;     // row inside the tile
+      const int piece = l_slot ^ (t_local & 15);
+      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b +
+                           static_cast<uint32_t>((2 * j + is_v) * D * 2 + 16 * piece);
+      char* dst = lds + (2 * buf + is_v) * C::TILE_B + rb * 1024;
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
+                                       (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
+    }
+  };
+  // This wave's direct-to-LDS loads have landed (vmcnt(0)); the barrier that follows publishes them.
+  auto wait_fetch = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
+
+  const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
+
+  if (range_hi > range_lo) {
+    __syncthreads();  // every wavefront has left the previous item's tiles
+    fetch_tile(range_lo, 0);
+    wait_fetch();
+    __syncthreads();
+    int buf = 0;
+    for (int tile = range_lo; tile < range_hi; tile += C::TK, buf ^= 1) {
+      const bool more = tile + C::TK < range_hi;
+      if (more) fetch_tile(tile + C::TK, buf ^ 1);
+      const char* kt = lds + buf * 2 * C::TILE_B;
+      const char* vt = kt + C::TILE_B;
+#pragma unroll 1
+      for (int h = 0; h < C::NH; ++h) {
+        const int a0 = tile + 32 * h;  // first key of this half
+        const bool w_skip = !w_any || a0 >= range_hi || a0 > w_pos_hi || (W > 0 && a0 + 31 <= w_pos_lo - W);
+        if (w_skip) continue;
+        bool act[MRT];
+#pragma unroll
+        for (int m = 0; m < MRT; ++m) act[m] = t_any[m] && a0 <= t_pos_hi[m] && !(W > 0 && a0 + 31 <= t_pos_lo[m] - W);
+        // S^T = K Q^T for the two 16-key sub-tiles; each K operand feeds every active row tile
+        f32x4_t s_acc[MRT][2];
+#pragma unroll
+        for (int m = 0; m < MRT; ++m) s_acc[m][0] = s_acc[m][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+          for (int ks = 0; ks < C::NKS; ++ks) {
+            const bf16x8_t kop = __builtin_bit_cast(
+                bf16x8_t, *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u + i) * C::ROWB + 16 * ((4 * ks + g) ^ i)));
+#pragma unroll
+            for (int m = 0; m < MRT; ++m)
+              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[m][ks], s_acc[m][u], 0, 0, 0);
+          }
+        __builtin_amdgcn_sched_barrier(0);  // keep the phases apart: bounds the registers the scheduler may use
+        // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
+        u32x4_t pw[MRT];
+#pragma unroll
+        for (int m = 0; m < MRT; ++m) {
+          float sv[2][4];
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[m][u][r]) : s_acc[m][u][r];
+          if (cap != 0.f) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+                sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
+          }
+          // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
+          const bool need_mask = !act[m] || a0 + 31 > t_pos_lo[m] || a0 + 32 > range_hi || (W > 0 && a0 <= t_pos_hi[m] - W);
+          if (need_mask) {
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const int tok = a0 + 16 * u + 4 * g + r;
+                const bool keep = tok <= pos_n[m] && tok < range_hi && (W <= 0 || tok > pos_n[m] - W);
+                sv[u][r] = keep ? sv[u][r] : -INFINITY;
+              }
+          }
+          float tmax = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
+                             fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
+          tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+          const float m_new = fmaxf(m_run[m], tmax);
+          const float m_use = m_new == -INFINITY ? 0.f : m_new;
+          const float alpha = __builtin_amdgcn_exp2f((m_run[m] - m_use) * kLog2e);
+          m_run[m] = m_new;
+          const float neg = -m_use * kLog2e;
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            float e0 = __builtin_amdgcn_exp2f(fmaf(sv[u][0], kLog2e, neg));
+            float e1 = __builtin_amdgcn_exp2f(fmaf(sv[u][1], kLog2e, neg));
+            float e2 = __builtin_amdgcn_exp2f(fmaf(sv[u][2], kLog2e, neg));
+            float e3 = __builtin_amdgcn_exp2f(fmaf(sv[u][3], kLog2e, neg));
+            pw[m][2 * u] = pack_bf16x2(e0, e1);
+            pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
+          }
+          if (__any(alpha != 1.f)) {
+            l_acc[m] *= alpha;
+#pragma unroll
+            for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+              for (int c = 0; c < 8; ++c) o_acc[m][sN][c] *= alpha;
+          }
+          l_acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ones),
+                                                            __builtin_bit_cast(bf16x8_t, pw[m]), l_acc[m], 0, 0, 0);
+        }
+        // O^T += V^T P^T: the eight fetched pieces of a slice give eight A operands, each used by every row tile
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN) {
+          __builtin_amdgcn_sched_barrier(0);
+          u32x4_t vch[8];
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            vch[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2) + 4 * g + (e & 3)) * C::ROWB +
+                                                       16 * ((i + 16 * sN) ^ (4 * g + (e & 3))));
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+            u32x4_t av;
+#pragma unroll
+            for (int hh = 0; hh < 4; ++hh) av[hh] = __builtin_amdgcn_perm(vch[2 * hh + 1][c >> 1], vch[2 * hh][c >> 1], sel);
+#pragma unroll
+            for (int m = 0; m < MRT; ++m)
+              o_acc[m][sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, pw[m]), o_acc[m][sN][c], 0, 0, 0);
+          }
+        }
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      wait_fetch();
+      __syncthreads();
+    }
+  }
+
+  // ---- normalise (with optional sinks) and store
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    if (!row_valid[m]) continue;
+    const float l_run = l_acc[m][0];
+    float num_scale = 1.f, denom = l_run;
+    if (p.sinks != nullptr && p.num_sinks > 0) {
+      const float* __restrict__ sk = p.sinks + static_cast<size_t>(head[m]) * p.num_sinks;
+      float smax = -INFINITY;
+      for (int k = 0; k < p.num_sinks; ++k) smax = fmaxf(smax, sk[k]);
+      const float mt = fmaxf(m_run[m], smax);
+      float ssum = 0.f;
+      for (int k = 0; k < p.num_sinks; ++k) ssum += expf(sk[k] - mt);
+      num_scale = m_run[m] == -INFINITY ? 0.f : expf(m_run[m] - mt);
+      denom = num_scale * l_run + ssum;
+    }
+    const float inv = num_scale / fmaxf(denom, 1e-6f);
+    bf16_t* orow = out + q_off[m];
+#pragma unroll
+    for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        u32x4_t w;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[m][sN][2 * e][r] * inv, o_acc[m][sN][2 * e + 1][r] * inv);
+        *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+      }
+  }
+}
+
+}  // namespace rpa

@@ -24,493 +24,78 @@
 // q is pre-multiplied by the bf16 scale and rounded to bf16, logits are rounded to bf16,
 // probabilities are bf16, accumulation is fp32.
 #include "rpa_device.h"
-#include "rpa_host.h"
+#include <atomic>
+
+#include "rpa_decode.h"
+#include "rpa_prefill.h"
 
 namespace rpa {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
-typedef __attribute__((ext_vector_type(4))) short s16x4_t;
-typedef __attribute__((ext_vector_type(4))) float f32x4_t;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
-typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
 
-constexpr int kWgThreads = 256;
-constexpr int kWgWaves = kWgThreads / kWave;
-constexpr float kLog2e = 1.4426950408889634f;
-
-struct TileArgs {
-  RpaParams p;
-  int page_shift;     // log2(page_size)
-  int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
-  uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
-  float* partial_o;   // [2 * wavefronts of the grid][16][D]
-  float* partial_ml;  // [2 * wavefronts of the grid][16][2]
-};
-
-// Split of the decode stream over the wavefronts of the grid: the first `rem` wavefronts take q + 1 tiles, the
-// others q, so shares differ by at most one tile and empty shares (q == 0) only occur at the end.
-struct Shares {
-  int q, rem;
-  __device__ __forceinline__ int begin(int w) const { return w * q + min(w, rem); }
-  __device__ __forceinline__ int owner(int x) const {
-    const int big = rem * (q + 1);
-    return x < big ? x / (q + 1) : rem + (x - big) / q;
-  }
-};
-
-// A wavefront's part of one (sequence, kv head) of the decode stream.
-struct Part {
-  bool partial;         // the (sequence, kv head) is shared with other wavefronts
-  int slot;             // workspace slot of this part
-  int first_w, last_w;  // wavefronts sharing it (every one of them holds at least one of its tiles)
-  int stream_a;         // stream index of its first tile
-  Shares sh;
-};
-
-// Workspace slot of wavefront k's part of the (sequence, kv head) starting at stream tile stream_a: a wavefront
-// has at most two partial parts, the one its share starts inside (slot 2k) and the one it ends inside (2k + 1).
-__device__ __forceinline__ int part_slot(int k, int stream_a, const Shares& sh) {
-  return 2 * k + (sh.begin(k) < stream_a ? 1 : 0);
+// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints and 8 ints of scratch, then the data region
+// shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
+__host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
+  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 8) * sizeof(int) + 15) & ~static_cast<size_t>(15);
 }
 
-struct SeqInfo {
-  int q0, q_len, kv_len, rows, n_rt;
-  int lo_al, hi;  // key range of the whole sequence, start aligned down to the tile
-  bool eligible;  // single row tile with keys: part of the decode stream
-};
-
-template <int TT>
-__device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
-  SeqInfo si;
-  si.q0 = p.query_start_loc[s];
-  si.q_len = p.query_start_loc[s + 1] - si.q0;
-  si.kv_len = p.context_lens[s];
-  si.rows = si.q_len > 0 ? si.q_len * G : 0;
-  si.n_rt = (si.rows + 15) >> 4;
-  const int pos_min = si.kv_len - si.q_len;
-  int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
-  si.lo_al = lo & ~(TT - 1);
-  si.hi = max(si.kv_len, 0);
-  si.eligible = si.n_rt == 1 && si.hi > si.lo_al;  // a sequence without keys stays an item: its rows become zero
-  return si;
-}
-
-// Exclusive prefix sum of one int per thread over the workgroup; `total` gets the sum.
-__device__ __forceinline__ int block_excl_scan(int v, int* wave_tot, int& total) {
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  int inc = v;
-#pragma unroll
-  for (int o = 1; o < kWave; o <<= 1) {
-    int t = __shfl_up(inc, o, kWave);
-    if (lane >= o) inc += t;
-  }
-  __syncthreads();
-  if (lane == kWave - 1) wave_tot[wave] = inc;
-  __syncthreads();
-  int base = 0, tot = 0;
-#pragma unroll
-  for (int w = 0; w < kWgWaves; ++w) {
-    const int t = wave_tot[w];
-    if (w < wave) base += t;
-    tot += t;
-  }
-  total = tot;
-  return base + inc - v;
-}
-
-// Hardware round-to-nearest-even conversions (v_cvt_pk_bf16_f32): branch-free, NaN stays NaN.
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
-__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
-  bf16x2_t v;
-  v[0] = static_cast<__bf16>(lo);
-  v[1] = static_cast<__bf16>(hi);
-  return __builtin_bit_cast(uint32_t, v);
-}
-__device__ __forceinline__ float rbf(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
-
-template <int D, int NT, bool kMimic>
-struct Cfg {
-  static constexpr int NS = D / 128;        // 128-wide slices of head_dim
-  static constexpr int NKS = D / 32;        // k-steps of the QK^T contraction
-  static constexpr int TT = 16 * NT;        // tokens per iteration
-  static constexpr int NSLOT = 4 * NT;      // tokens each lane fetches per iteration
-  static constexpr int ROWB = D * 2 + 16;   // LDS bytes per K row (16 B pad: conflict-free b128 reads)
-  static constexpr int LDS_PER_WAVE = TT * ROWB;
-};
-
-// Everything one wavefront needs for one work item.
-template <int D, int NT, bool kMimic>
-__device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
-                                             int j, int rt, int range_lo, int range_hi, const Part& part) {
+template <int D, int NT, int MRT, bool kMimic>
+__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void rpa_tile_kernel(TileArgs a) {
   using C = Cfg<D, NT, kMimic>;
-  const RpaParams& p = a.p;
-  const int lane = threadIdx.x & (kWave - 1);
-  const int i = lane & 15, g = lane >> 4;
-  const int G = p.num_q_heads / p.num_kv_heads;
-  const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
-  const bf16_t* __restrict__ kv = static_cast<const bf16_t*>(p.kv_pages);
-  bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
-  const int W = p.sliding_window;
-
-  // ---- rows of this tile and their key range
-  const int row_lo = rt * 16, row_hi = min(row_lo + 16, si.rows);
-  const int qi_min = row_lo / G, qi_max = (row_hi - 1) / G;
-  const int pos_min = si.kv_len - si.q_len + qi_min, pos_max = si.kv_len - si.q_len + qi_max;
-  // this lane's row
-  const int R = row_lo + i;
-  const bool row_valid = R < si.rows;
-  const int qi = row_valid ? R / G : 0;
-  const int hg = row_valid ? R - qi * G : 0;
-  const int pos_n = row_valid ? si.kv_len - si.q_len + qi : -1;
-  const int head = j * G + hg;
-  const size_t q_row_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * D;
-
-  // ---- Q^T operands: lane (row i, group g) holds q[row][32 ks + 8 g .. +8], pre-scaled and rounded to bf16
-  bf16x8_t qreg[C::NKS];
-  {
-    const float scale = rbf(p.softmax_scale);
-#pragma unroll
-    for (int ks = 0; ks < C::NKS; ++ks) {
-      u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (row_valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
-      u32x4_t sc;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const float lo = __uint_as_float(raw[e] << 16) * scale, hi = __uint_as_float(raw[e] & 0xffff0000u) * scale;
-        sc[e] = pack_bf16x2(lo, hi);
-      }
-      qreg[ks] = __builtin_bit_cast(bf16x8_t, sc);
-    }
-  }
-
-  f32x4_t o_acc[C::NS][8];
-#pragma unroll
-  for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-    for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
-
-  const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;  // elements between tokens
-  const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
-  // Same row through the constant address space: reads with a wave-uniform index become scalar loads, which
-  // are counted apart from the vector loads of the K/V stream.  The block table is never written by this kernel.
-  const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(bt));
-  const int t_last = range_hi - 1;
-  const float cap = p.logits_soft_cap;
-
-  u32x4_t kreg[C::NSLOT][C::NS];
-  u32x4_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
-
-  // Fetch K and V of the TT tokens starting at `tile`: lane (i, g) takes tokens 16u + 4g + r (u < NT, r < 4),
-  // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.
-  //
-  // Fast path (page_size >= 16, tile entirely inside the range): a 16-token sub-tile sits in one page, so the
-  // block-table entry is a scalar load (it does not share the vector-memory counter with the K/V stream) and
-  // the row address is a scalar base plus one per-lane byte offset that is constant for the whole item.
-  // Slow path (last tile of a range, small pages): per-lane page lookup; tokens past the end of the range are
-  // replaced by the last valid one (their scores are masked).
-  const char* kvb = reinterpret_cast<const char*>(kv);
-  const uint32_t stride_b = static_cast<uint32_t>(tok_stride) * 2u;  // bytes between tokens
-  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
-  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + static_cast<uint32_t>(2 * j * D * 2 + 16 * i);
-  auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
-    if (a.uniform_page && tile + C::TT <= range_hi) {
-#pragma unroll
-      for (int u = 0; u < NT; ++u) {
-        const int t16 = tile + 16 * u;
-        int page = bt_c[t16 >> a.page_shift];
-        page = min(max(page, 0), p.num_pages - 1);
-        const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                            static_cast<uint64_t>(t16 & (p.page_size - 1)) * stride_b;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const char* row = sbase + static_cast<uint64_t>(r) * stride_b;
-#pragma unroll
-          for (int sN = 0; sN < C::NS; ++sN) {
-            kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN));
-            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN + 2u * D));
-          }
-        }
-      }
-      return;
-    }
-#pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      const int t4c = min(tile + 16 * u + 4 * g, t_last & ~3);
-      const int rlim = min(3, t_last - t4c);
-      int page = bt[t4c >> a.page_shift];
-      page = min(max(page, 0), p.num_pages - 1);
-      const char* base = kvb + static_cast<uint64_t>(page) * page_b +
-                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (2 * j * D * 2 + 16 * i);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
-#pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN) {
-          kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN);
-          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN + 2 * D);
-        }
-      }
-    }
-  };
-
-  auto body = [&](int tile, u32x4_t (&vcur)[C::NSLOT][C::NS], u32x4_t (&vnext)[C::NSLOT][C::NS]) {
-    // 1. K rows to the wave-private LDS tile: row = token within the tile, 16-byte piece i (+16 per slice)
-#pragma unroll
-    for (int u = 0; u < NT; ++u)
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-#pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN)
-          *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kreg[4 * u + r][sN];
-    // 2. next tile's K and V are requested now, a full iteration before they are needed
-    if (tile + C::TT < range_hi) issue_loads(tile + C::TT, kreg, vnext);
-    // 3. S^T = K Q^T: lane (token i of sub-tile u, group g) reads piece 4 ks + g of its row
-    f32x4_t s_acc[NT];
-#pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      s_acc[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < C::NKS; ++ks) {
-        const u32x4_t kop = *reinterpret_cast<const u32x4_t*>(lds_k + (16 * u + i) * C::ROWB + 16 * (4 * ks + g));
-        s_acc[u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop), qreg[ks], s_acc[u], 0, 0, 0);
-      }
-    }
-    // 4. online softmax; this lane: query row i, tokens tile + 16u + 4g + r
-    float sv[NT][4];
-    const bool need_mask = (tile + C::TT > range_hi) || (tile + C::TT - 1 > pos_min) || (W > 0 && tile <= pos_max - W);
-#pragma unroll
-    for (int u = 0; u < NT; ++u)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r];
-    if (cap != 0.f) {
-#pragma unroll
-      for (int u = 0; u < NT; ++u)
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
-    }
-    if (need_mask) {
-#pragma unroll
-      for (int u = 0; u < NT; ++u)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const int tok = tile + 16 * u + 4 * g + r;
-          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W);
-          sv[u][r] = keep ? sv[u][r] : -INFINITY;
-        }
-    }
-    float tmax = -INFINITY;
-#pragma unroll
-    for (int u = 0; u < NT; ++u)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, sv[u][r]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-    const float m_new = fmaxf(m_run, tmax);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
-    float psum = 0.f;
-    uint32_t pw[2 * NT];
-#pragma unroll
-    for (int u = 0; u < NT; ++u) {
-      float pv[4];
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        float d = sv[u][r] - m_use;
-        if (kMimic) d = rbf(d);
-        float e = __builtin_amdgcn_exp2f(d * kLog2e);
-        e = rbf(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
-        pv[r] = e;
-        psum += e;
-      }
-      pw[2 * u] = (__float_as_uint(pv[0]) >> 16) | (__float_as_uint(pv[1]) & 0xffff0000u);
-      pw[2 * u + 1] = (__float_as_uint(pv[2]) >> 16) | (__float_as_uint(pv[3]) & 0xffff0000u);
-    }
-    l_run = l_run * alpha + psum;
-    m_run = m_new;
-    if (__any(alpha != 1.f)) {
-#pragma unroll
-      for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-        for (int c = 0; c < 8; ++c) o_acc[sN][c] *= alpha;
-    }
-    // 5. O^T += V^T P^T.  MFMA number c of slice sN yields d = 128 sN + 8 (row of the MFMA) + c; its A operand is
-    //    column c of every fetched 8-wide piece, gathered from the token rows by byte permutes.
-#pragma unroll
-    for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-        uint32_t aw[2 * NT];
-#pragma unroll
-        for (int h = 0; h < 2 * NT; ++h)
-          aw[h] = __builtin_amdgcn_perm(vcur[2 * h + 1][sN][c >> 1], vcur[2 * h][sN][c >> 1], sel);
-        if constexpr (NT == 2) {
-          const u32x4_t av = {aw[0], aw[1], aw[2], aw[3]};
-          const u32x4_t pvv = {pw[0], pw[1], pw[2], pw[3]};
-          o_acc[sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, av),
-                                                                 __builtin_bit_cast(bf16x8_t, pvv), o_acc[sN][c], 0, 0, 0);
-        } else {
-          const u32x2_t av = {aw[0], aw[1]};
-          const u32x2_t pvv = {pw[0], pw[1]};
-          o_acc[sN][c] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(s16x4_t, av),
-                                                                   __builtin_bit_cast(s16x4_t, pvv), o_acc[sN][c], 0, 0, 0);
-        }
-      }
-  };
-
-  if (range_hi > range_lo) {
-    issue_loads(range_lo, kreg, vbuf0);
-    for (int tile = range_lo; tile < range_hi; tile += 2 * C::TT) {
-      body(tile, vbuf0, vbuf1);
-      if (tile + C::TT >= range_hi) break;
-      body(tile + C::TT, vbuf1, vbuf0);
-    }
-  }
-
-  // ---- row sum across the four lane groups
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
-
-  if (part.partial) {
-    // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
-    // Partials are written and read with agent-scope relaxed atomics (write-through / cache-bypassing accesses),
-    // so no L2 write-back or invalidate is needed around the ticket: it is enough that this wave's stores have
-    // completed (the workgroup-scope release waits for them) before the ticket is taken.
-    const size_t slot = static_cast<size_t>(part.slot);
-    if (row_valid) {
-      uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
-#pragma unroll
-      for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const uint64_t v = static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e][r])) |
-                               (static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e + 1][r])) << 32);
-            __hip_atomic_store(po + (128 * sN + 32 * g + 8 * r) / 2 + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
-      if (g == 0) {
-        const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_run)) | (static_cast<uint64_t>(__float_as_uint(l_run)) << 32);
-        __hip_atomic_store(reinterpret_cast<uint64_t*>(a.partial_ml) + slot * 16 + i, v, __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-      }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    uint32_t* ctr = a.counters + static_cast<size_t>(s) * p.num_kv_heads + j;
-    uint32_t ticket = 0;
-    if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    ticket = __shfl(ticket, 0, kWave);
-    if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
-    float M = -INFINITY;
-    if (row_valid)
-      for (int k = part.first_w; k <= part.last_w; ++k) {
-        const size_t sl = part_slot(k, part.stream_a, part.sh);
-        const uint64_t v = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v)));
-      }
-    const float M_use = M == -INFINITY ? 0.f : M;
-    float L = 0.f;
-#pragma unroll
-    for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-      for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    if (row_valid) {
-      for (int k = part.first_w; k <= part.last_w; ++k) {
-        const size_t sl = part_slot(k, part.stream_a, part.sh);
-        const uint64_t mlv = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float mk = __uint_as_float(static_cast<uint32_t>(mlv)), lk = __uint_as_float(static_cast<uint32_t>(mlv >> 32));
-        const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
-        L += w * lk;
-        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
-#pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const uint64_t v = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-              o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(v));
-              o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(v >> 32));
-            }
-      }
-    }
-    m_run = M;
-    l_run = L;
-    if (lane == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  }
-
-  // ---- normalise (with optional sinks) and store
-  if (!row_valid) return;
-  float num_scale = 1.f, denom = l_run;
-  if (p.sinks != nullptr && p.num_sinks > 0) {
-    const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
-    float smax = -INFINITY;
-    for (int k = 0; k < p.num_sinks; ++k) smax = fmaxf(smax, sk[k]);
-    const float mt = fmaxf(m_run, smax);
-    float ssum = 0.f;
-    for (int k = 0; k < p.num_sinks; ++k) ssum += expf(sk[k] - mt);
-    num_scale = m_run == -INFINITY ? 0.f : expf(m_run - mt);
-    denom = num_scale * l_run + ssum;
-  }
-  const float inv = num_scale / fmaxf(denom, 1e-6f);
-  bf16_t* orow = out + q_row_off;
-#pragma unroll
-  for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      u32x4_t w;
-#pragma unroll
-      for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[sN][2 * e][r] * inv, o_acc[sN][2 * e + 1][r] * inv);
-      *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
-    }
-}
-
-template <int D, int NT, bool kMimic>
-__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
-  using C = Cfg<D, NT, kMimic>;
+  using PC = PCfg<D, MRT>;
   extern __shared__ __align__(16) char smem[];
   const RpaParams& p = a.p;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int G = p.num_q_heads / p.num_kv_heads;
-  // LDS: [4 waves x K tile][item_start: S+1][tile_start: S+1][scratch 8 ints]
-  char* lds_k = smem + wave * C::LDS_PER_WAVE;
-  int* item_start = reinterpret_cast<int*>(smem + kWgWaves * C::LDS_PER_WAVE);
-  int* tile_start = item_start + (p.max_num_seqs + 1);
-  int* scratch = tile_start + (p.max_num_seqs + 1);
+  int* item_start = reinterpret_cast<int*>(smem);            // wave-level items
+  int* tile_start = item_start + (p.max_num_seqs + 1);       // decode stream tiles
+  int* wg_start = tile_start + (p.max_num_seqs + 1);         // workgroup-level prefill tiles
+  int* scratch = wg_start + (p.max_num_seqs + 1);
+  char* lds_data = smem + sched_bytes(p.max_num_seqs);
+  char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
   int nseq = p.num_seqs[0];
   nseq = min(max(nseq, 0), p.max_num_seqs);
 
-  // ---- schedule: per sequence, tiles it adds to the decode stream (single row tile) or items (more row tiles)
+  // ---- schedule.  Per sequence: tiles it adds to the decode stream (one row tile, has keys), workgroup tiles
+  // (more than kWaveItemMaxRowTiles row tiles), or wave-level items (everything else).
+  auto classify = [&](const SeqInfo& si, int& tiles, int& items, int& wg_items) {
+    tiles = items = wg_items = 0;
+    if (si.eligible) tiles = p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
+    else if (si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
+    else items = p.num_kv_heads * si.n_rt;
+  };
   const int per = (nseq + kWgThreads - 1) / kWgThreads;
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
-  int my_items = 0, my_tiles = 0;
+  int my_items = 0, my_tiles = 0, my_wg = 0;
   for (int s = s_begin; s < s_end; ++s) {
-    const SeqInfo si = seq_info<C::TT>(p, s, G);
-    if (si.eligible) my_tiles += p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
-    else my_items += p.num_kv_heads * si.n_rt;
+    int t, it, wg;
+    classify(seq_info<C::TT>(p, s, G), t, it, wg);
+    my_tiles += t;
+    my_items += it;
+    my_wg += wg;
   }
-  int total_items, total_tiles;
+  int total_items, total_tiles, total_wg;
   int item_base = block_excl_scan(my_items, scratch, total_items);
   int tile_base = block_excl_scan(my_tiles, scratch, total_tiles);
+  int wg_base = block_excl_scan(my_wg, scratch, total_wg);
   for (int s = s_begin; s < s_end; ++s) {
-    const SeqInfo si = seq_info<C::TT>(p, s, G);
+    int t, it, wg;
+    classify(seq_info<C::TT>(p, s, G), t, it, wg);
     item_start[s] = item_base;
     tile_start[s] = tile_base;
-    if (si.eligible) tile_base += p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
-    else item_base += p.num_kv_heads * si.n_rt;
+    wg_start[s] = wg_base;
+    item_base += it;
+    tile_base += t;
+    wg_base += wg;
   }
   total_items = __builtin_amdgcn_readfirstlane(total_items);
   total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
+  total_wg = __builtin_amdgcn_readfirstlane(total_wg);
   if (tid == 0) {
     item_start[nseq] = total_items;
     tile_start[nseq] = total_tiles;
+    wg_start[nseq] = total_wg;
   }
   __syncthreads();
 
@@ -536,7 +121,15 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     return __builtin_amdgcn_readfirstlane(lo);
   };
 
-  // ---- sequences with several row tiles: one item per (sequence, row tile, kv head), strided over the grid
+  // ---- prefill: one item per (sequence, tile of WGROWS rows, kv head), strided over the workgroups
+  for (int w = blockIdx.x; w < total_wg; w += gridDim.x) {
+    const int s = find(wg_start, w);
+    const SeqInfo si = seq_info<C::TT>(p, s, G);
+    const int local = __builtin_amdgcn_readfirstlane(w - wg_start[s]);
+    prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, local % p.num_kv_heads, local / p.num_kv_heads);
+  }
+
+  // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
   for (int w = worker; w < total_items; w += n_workers) {
     const int s = find(item_start, w);
     const SeqInfo si = seq_info<C::TT>(p, s, G);
@@ -614,11 +207,23 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
 }
 
-template <int D, int NT, bool kMimic>
+template <int D, int NT, int MRT, bool kMimic>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<D, NT, kMimic>;
-  const size_t lds = static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE + (2 * (a.p.max_num_seqs + 1) + 8) * sizeof(int);
-  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, kMimic>), dim3(grid), dim3(kWgThreads), lds, stream, a);
+  using PC = PCfg<D, MRT>;
+  const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE, static_cast<size_t>(PC::LDS));
+  const size_t lds = sched_bytes(a.p.max_num_seqs) + data;
+  // More than 64 KiB of dynamic LDS has to be allowed once per kernel (and device); the call is idempotent.
+  static std::atomic<uint64_t> allowed[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+  if (allowed[dev].load(std::memory_order_acquire) < lds) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
+      return RPA_ERR_LAUNCH;
+    allowed[dev].store(lds, std::memory_order_release);
+  }
+  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic>), dim3(grid), dim3(kWgThreads), lds, stream, a);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
@@ -636,8 +241,9 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
   const bool mimic = env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
-  if (p.head_dim == 128) return mimic ? launch_cfg<128, 2, true>(a, grid, stream) : launch_cfg<128, 2, false>(a, grid, stream);
-  return mimic ? launch_cfg<256, 1, true>(a, grid, stream) : launch_cfg<256, 1, false>(a, grid, stream);
+  if (p.head_dim == 128)
+    return mimic ? launch_cfg<128, 2, 4, true>(a, grid, stream) : launch_cfg<128, 2, 4, false>(a, grid, stream);
+  return mimic ? launch_cfg<256, 1, 2, true>(a, grid, stream) : launch_cfg<256, 1, 2, false>(a, grid, stream);
 }
 
 }  // namespace rpa

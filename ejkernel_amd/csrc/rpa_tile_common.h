@@ -1,0 +1,110 @@
+// Types and helpers shared by the wave-level (decode) and workgroup-level (prefill) attention loops.
+#pragma once
+
+#include "rpa_device.h"
+#include "rpa_host.h"
+
+namespace rpa {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) short s16x4_t;
+typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
+typedef const int32_t __attribute__((address_space(4))) * const_i32_ptr;
+
+constexpr int kWgThreads = 256;
+constexpr int kWgWaves = kWgThreads / kWave;
+constexpr float kLog2e = 1.4426950408889634f;
+
+struct TileArgs {
+  RpaParams p;
+  int page_shift;     // log2(page_size)
+  int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
+  uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
+  float* partial_o;   // [2 * wavefronts of the grid][16][D]
+  float* partial_ml;  // [2 * wavefronts of the grid][16][2]
+};
+
+// Split of the decode stream over the wavefronts of the grid: the first `rem` wavefronts take q + 1 tiles, the
+// others q, so shares differ by at most one tile and empty shares (q == 0) only occur at the end.
+struct Shares {
+  int q, rem;
+  __device__ __forceinline__ int begin(int w) const { return w * q + min(w, rem); }
+  __device__ __forceinline__ int owner(int x) const {
+    const int big = rem * (q + 1);
+    return x < big ? x / (q + 1) : rem + (x - big) / q;
+  }
+};
+
+// A wavefront's part of one (sequence, kv head) of the decode stream.
+struct Part {
+  bool partial;         // the (sequence, kv head) is shared with other wavefronts
+  int slot;             // workspace slot of this part
+  int first_w, last_w;  // wavefronts sharing it (every one of them holds at least one of its tiles)
+  int stream_a;         // stream index of its first tile
+  Shares sh;
+};
+
+// Workspace slot of wavefront k's part of the (sequence, kv head) starting at stream tile stream_a: a wavefront
+// has at most two partial parts, the one its share starts inside (slot 2k) and the one it ends inside (2k + 1).
+__device__ __forceinline__ int part_slot(int k, int stream_a, const Shares& sh) {
+  return 2 * k + (sh.begin(k) < stream_a ? 1 : 0);
+}
+
+struct SeqInfo {
+  int q0, q_len, kv_len, rows, n_rt;
+  int lo_al, hi;  // key range of the whole sequence, start aligned down to the tile
+  bool eligible;  // single row tile with keys: part of the decode stream
+};
+
+template <int TT>
+__device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
+  SeqInfo si;
+  si.q0 = p.query_start_loc[s];
+  si.q_len = p.query_start_loc[s + 1] - si.q0;
+  si.kv_len = p.context_lens[s];
+  si.rows = si.q_len > 0 ? si.q_len * G : 0;
+  si.n_rt = (si.rows + 15) >> 4;
+  const int pos_min = si.kv_len - si.q_len;
+  int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
+  si.lo_al = lo & ~(TT - 1);
+  si.hi = max(si.kv_len, 0);
+  si.eligible = si.n_rt == 1 && si.hi > si.lo_al;  // a sequence without keys stays an item: its rows become zero
+  return si;
+}
+
+// Exclusive prefix sum of one int per thread over the workgroup; `total` gets the sum.
+__device__ __forceinline__ int block_excl_scan(int v, int* wave_tot, int& total) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int inc = v;
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+    int t = __shfl_up(inc, o, kWave);
+    if (lane >= o) inc += t;
+  }
+  __syncthreads();
+  if (lane == kWave - 1) wave_tot[wave] = inc;
+  __syncthreads();
+  int base = 0, tot = 0;
+#pragma unroll
+  for (int w = 0; w < kWgWaves; ++w) {
+    const int t = wave_tot[w];
+    if (w < wave) base += t;
+    tot += t;
+  }
+  total = tot;
+  return base + inc - v;
+}
+
+// Hardware round-to-nearest-even conversions (v_cvt_pk_bf16_f32): branch-free, NaN stays NaN.
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+  bf16x2_t v;
+  v[0] = static_cast<__bf16>(lo);
+  v[1] = static_cast<__bf16>(hi);
+  return __builtin_bit_cast(uint32_t, v);
+}
+__device__ __forceinline__ float rbf(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
+
+}  // namespace rpa
