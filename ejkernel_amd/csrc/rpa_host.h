@@ -11,7 +11,7 @@ namespace rpa {
 int launch_generic(const RpaParams& p, hipStream_t stream);
 
 // Tiled MFMA path (bf16, head_dim 128 or 256, page_size a multiple of 4).
-constexpr int kTiledMaxSeqs = 2048;        // schedule arrays live in LDS
+constexpr int kTiledMaxSeqs = 1024;        // schedule arrays live in LDS
 constexpr int kTiledMaxWgsPerCu = 4;        // persistent grid = compute units x this, at most
 
 constexpr uint64_t kWorkspaceTicketBytes = 1u << 20;  // head of the workspace, cleared by rpa_workspace_init

@@ -28,12 +28,15 @@ struct PCfg {
   static constexpr int WROWS = 16 * MRT;             // rows per wavefront
   static constexpr int WGROWS = kWgWaves * WROWS;    // rows per workgroup
   static constexpr int TILE_B = TK * ROWB;           // one K (or V) tile: 16 KiB
-  static constexpr int LDS = 4 * TILE_B;             // K and V, double buffered
+  static constexpr int NSTG = 2;                     // LDS stages: tiles requested ahead of the one in use + 1
+  static constexpr int LDS = 2 * NSTG * TILE_B;      // K and V tile per stage
   static constexpr int PR = D / 8;                   // 16-byte pieces per row
   static constexpr int RB = kWave / PR;              // rows one wave-wide load instruction covers
   static constexpr int BLOCKS = TK / RB;             // load instructions per K (or V) tile: 16
   static constexpr int BPW = 2 * BLOCKS / kWgWaves;  // load instructions per wavefront and step
 };
+
+constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point by this much before O is rescaled
 
 template <int D, int MRT, bool kMimic>
 __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
@@ -136,20 +139,29 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                                        (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
     }
   };
-  // This wave's direct-to-LDS loads have landed (vmcnt(0)); the barrier that follows publishes them.
-  auto wait_fetch = [&]() { __builtin_amdgcn_s_waitcnt(0x0F70); };
+  // Wait until at most `ahead` later tiles of this wave's direct-to-LDS loads are outstanding (they complete in
+  // order); the barrier that follows publishes the oldest tile.  s_waitcnt takes an immediate: vmcnt is bits
+  // [3:0] and [15:14]; 0x0F70 leaves the other counters unconstrained.
+  auto wait_fetch = [&](int ahead) {
+    static_assert(C::BPW == 8 && C::NSTG <= 4, "vmcnt immediates below assume 8 loads per tile, <= 2 tiles ahead");
+    if (ahead <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
+    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F78);
+    else __builtin_amdgcn_s_waitcnt(0x4F70);
+  };
 
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
 
   if (range_hi > range_lo) {
+    const int n_tiles = (range_hi - range_lo + C::TK - 1) / C::TK;
     __syncthreads();  // every wavefront has left the previous item's tiles
-    fetch_tile(range_lo, 0);
-    wait_fetch();
-    __syncthreads();
-    int buf = 0;
-    for (int tile = range_lo; tile < range_hi; tile += C::TK, buf ^= 1) {
-      const bool more = tile + C::TK < range_hi;
-      if (more) fetch_tile(tile + C::TK, buf ^ 1);
+    for (int t = 0; t < min(C::NSTG - 1, n_tiles); ++t) fetch_tile(range_lo + t * C::TK, t);
+    for (int kt_i = 0; kt_i < n_tiles; ++kt_i) {
+      const int tile = range_lo + kt_i * C::TK;
+      const int buf = kt_i % C::NSTG;
+      wait_fetch(min(n_tiles - 1 - kt_i, C::NSTG - 2));
+      // publishes tile kt_i, and every wavefront has finished the previous tile, whose stage is refilled next
+      __syncthreads();
+      if (kt_i + C::NSTG - 1 < n_tiles) fetch_tile(tile + (C::NSTG - 1) * C::TK, (kt_i + C::NSTG - 1) % C::NSTG);
       const char* kt = lds + buf * 2 * C::TILE_B;
       const char* vt = kt + C::TILE_B;
 #pragma unroll 1
@@ -160,20 +172,24 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         bool act[MRT];
 #pragma unroll
         for (int m = 0; m < MRT; ++m) act[m] = t_any[m] && a0 <= t_pos_hi[m] && !(W > 0 && a0 + 31 <= t_pos_lo[m] - W);
-        // S^T = K Q^T for the two 16-key sub-tiles; each K operand feeds every active row tile
+        // S^T = K Q^T for the two 16-key sub-tiles.  All K operands of a sub-tile are requested before the first
+        // MFMA, so LDS latency overlaps the matrix work; each operand feeds every row tile.
         f32x4_t s_acc[MRT][2];
 #pragma unroll
-        for (int m = 0; m < MRT; ++m) s_acc[m][0] = s_acc[m][1] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int u = 0; u < 2; ++u) {
+          u32x4_t kop[C::NKS];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+          for (int ks = 0; ks < C::NKS; ++ks)
+            kop[ks] = *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u + i) * C::ROWB + 16 * ((4 * ks + g) ^ i));
 #pragma unroll
-          for (int ks = 0; ks < C::NKS; ++ks) {
-            const bf16x8_t kop = __builtin_bit_cast(
-                bf16x8_t, *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u + i) * C::ROWB + 16 * ((4 * ks + g) ^ i)));
+          for (int m = 0; m < MRT; ++m) s_acc[m][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int ks = 0; ks < C::NKS; ++ks)
 #pragma unroll
             for (int m = 0; m < MRT; ++m)
-              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kop, qreg[m][ks], s_acc[m][u], 0, 0, 0);
-          }
+              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[ks]), qreg[m][ks],
+                                                                    s_acc[m][u], 0, 0, 0);
+        }
         __builtin_amdgcn_sched_barrier(0);  // keep the phases apart: bounds the registers the scheduler may use
         // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
         u32x4_t pw[MRT];
@@ -207,9 +223,12 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                              fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
           tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
           tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-          const float m_new = fmaxf(m_run[m], tmax);
+          // Lazy rescale: the reference point m_run only moves when the tile maximum exceeds it by more than
+          // kLazy (probabilities then stay below e^kLazy, far inside bf16/fp32 range), so rescaling O is rare.
+          const bool bump = tmax > m_run[m] + kLazy;
+          const float m_new = bump ? tmax : m_run[m];
           const float m_use = m_new == -INFINITY ? 0.f : m_new;
-          const float alpha = __builtin_amdgcn_exp2f((m_run[m] - m_use) * kLog2e);
+          const float alpha = bump ? __builtin_amdgcn_exp2f((m_run[m] - m_use) * kLog2e) : 1.f;
           m_run[m] = m_new;
           const float neg = -m_use * kLog2e;
 #pragma unroll
@@ -221,7 +240,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
             pw[m][2 * u] = pack_bf16x2(e0, e1);
             pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
           }
-          if (__any(alpha != 1.f)) {
+          if (__builtin_expect(__any(bump), 0)) {
             l_acc[m] *= alpha;
 #pragma unroll
             for (int sN = 0; sN < C::NS; ++sN)
@@ -253,9 +272,6 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           }
         }
       }
-      __builtin_amdgcn_sched_barrier(0);
-      wait_fetch();
-      __syncthreads();
     }
   }
 

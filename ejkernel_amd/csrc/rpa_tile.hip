@@ -40,7 +40,7 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 }
 
 template <int D, int NT, int MRT, bool kMimic>
-__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(1, 1))) void rpa_tile_kernel(TileArgs a) {
+__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
   extern __shared__ __align__(16) char smem[];
@@ -128,6 +128,9 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(1, 1
     const int local = __builtin_amdgcn_readfirstlane(w - wg_start[s]);
     prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, local % p.num_kv_heads, local / p.num_kv_heads);
   }
+  // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
+  // workgroup has finished reading them.
+  __syncthreads();
 
   // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
   for (int w = worker; w < total_items; w += n_workers) {
@@ -242,7 +245,7 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   const int grid = tiled_grid();
   const bool mimic = env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
   if (p.head_dim == 128)
-    return mimic ? launch_cfg<128, 2, 4, true>(a, grid, stream) : launch_cfg<128, 2, 4, false>(a, grid, stream);
+    return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 2, true>(a, grid, stream) : launch_cfg<256, 1, 2, false>(a, grid, stream);
 }
 
