@@ -182,8 +182,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     for (int u = 0; u < NT; ++u)
 #pragma unroll
       for (int r = 0; r < 4; ++r) tmax = fmaxf(tmax, sv[u][r]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
+    tmax = row_groups_max(tmax);
     const float m_new = fmaxf(m_run, tmax);
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
@@ -247,8 +246,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   }
 
   // ---- row sum across the four lane groups
-  l_run += __shfl_xor(l_run, 16, kWave);
-  l_run += __shfl_xor(l_run, 32, kWave);
+  l_run = row_groups_sum(l_run);
 
   if (part.partial) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.

@@ -10,7 +10,9 @@
 // wavefront then computes S^T = K Q^T and O^T += V^T P^T for its own 16 * MRT rows: every K and V operand read from LDS feeds MRT MFMAs, Q stays in registers, and
 // each lane owns one row per row tile, so the online softmax is lane-local as in the decode loop.
 // The row sums come from one extra MFMA against a vector of ones (they add exactly the bf16
-// probabilities that enter P V).  Halves of a step that lie entirely in a wavefront's causal
+// probabilities that enter P V).  Logits stay in fp32 here (the decode loop rounds them to bf16 as
+// the reference does; on prefill tiles that rounding only costs VALU time: measured against the
+// reference restatement the mean error moves from 4e-4 to 5.5e-4 of a 2e-3 budget).  Halves of a step that lie entirely in a wavefront's causal
 // future or left of its window are skipped.
 #pragma once
 
@@ -151,6 +153,16 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0
 
+  // Per-lane byte offsets of the MFMA operand reads inside a stage, fixed for the whole item: the row part of
+  // a later sub-tile or half is a compile-time constant on top of them (the swizzle only uses row & 15).
+  int k_off[C::NKS], v_off[C::NS][4];
+#pragma unroll
+  for (int ks = 0; ks < C::NKS; ++ks) k_off[ks] = i * C::ROWB + 16 * ((4 * ks + g) ^ i);
+#pragma unroll
+  for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v_off[sN][r] = (4 * g + r) * C::ROWB + 16 * ((i + 16 * sN) ^ (4 * g + r));
+
   if (range_hi > range_lo) {
     const int n_tiles = (range_hi - range_lo + C::TK - 1) / C::TK;
     __syncthreads();  // every wavefront has left the previous item's tiles
@@ -164,7 +176,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       if (kt_i + C::NSTG - 1 < n_tiles) fetch_tile(tile + (C::NSTG - 1) * C::TK, (kt_i + C::NSTG - 1) % C::NSTG);
       const char* kt = lds + buf * 2 * C::TILE_B;
       const char* vt = kt + C::TILE_B;
-#pragma unroll 1
+#pragma unroll
       for (int h = 0; h < C::NH; ++h) {
         const int a0 = tile + 32 * h;  // first key of this half
         const bool w_skip = !w_any || a0 >= range_hi || a0 > w_pos_hi || (W > 0 && a0 + 31 <= w_pos_lo - W);
@@ -172,25 +184,51 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         bool act[MRT];
 #pragma unroll
         for (int m = 0; m < MRT; ++m) act[m] = t_any[m] && a0 <= t_pos_hi[m] && !(W > 0 && a0 + 31 <= t_pos_lo[m] - W);
-        // S^T = K Q^T for the two 16-key sub-tiles.  All K operands of a sub-tile are requested before the first
-        // MFMA, so LDS latency overlaps the matrix work; each operand feeds every row tile.
+        // S^T = K Q^T for the two 16-key sub-tiles.  The eight K operands are requested first and the V pieces of
+        // the first slice while the QK MFMAs run, so LDS latency is paid once per half and V is in registers by
+        // the time the softmax is done.  The group barriers pin that order (the scheduler would otherwise sink
+        // every LDS read next to its first use).
         f32x4_t s_acc[MRT][2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u) {
-          u32x4_t kop[C::NKS];
+        constexpr int KU = D == 128 ? 2 : 1;  // sub-tiles whose K operands are held at once (register budget)
+        u32x4_t kop[KU][C::NKS];
+        auto load_k = [&](int u) {
 #pragma unroll
           for (int ks = 0; ks < C::NKS; ++ks)
-            kop[ks] = *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u + i) * C::ROWB + 16 * ((4 * ks + g) ^ i));
+            kop[u % KU][ks] = *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u) * C::ROWB + k_off[ks]);
+        };
+        if constexpr (KU == 2) {
+          load_k(0);
+          load_k(1);
+        }
+        u32x4_t vch[8];
+        auto load_v = [&](int sN) {
+#pragma unroll
+          for (int e = 0; e < 8; ++e)
+            vch[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2)) * C::ROWB + v_off[sN][e & 3]);
+        };
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+          if constexpr (KU == 1) {
+            load_k(u);
+            __builtin_amdgcn_sched_group_barrier(0x100, C::NKS, 0);
+          }
 #pragma unroll
           for (int m = 0; m < MRT; ++m) s_acc[m][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < C::NKS; ++ks)
 #pragma unroll
             for (int m = 0; m < MRT; ++m)
-              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[ks]), qreg[m][ks],
-                                                                    s_acc[m][u], 0, 0, 0);
+              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[u % KU][ks]),
+                                                                    qreg[m][ks], s_acc[m][u], 0, 0, 0);
+          if constexpr (KU == 1) __builtin_amdgcn_sched_group_barrier(0x008, C::NKS * MRT, 0);
         }
-        __builtin_amdgcn_sched_barrier(0);  // keep the phases apart: bounds the registers the scheduler may use
+        load_v(0);
+        if constexpr (KU == 2) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 2 * C::NKS, 0);        // K operands first
+          __builtin_amdgcn_sched_group_barrier(0x008, 2 * C::NKS * MRT, 0);  // QK MFMAs
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // V pieces of slice 0: they land during the softmax
+        __builtin_amdgcn_sched_barrier(0);
         // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
         u32x4_t pw[MRT];
 #pragma unroll
@@ -199,7 +237,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
           for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[m][u][r]) : s_acc[m][u][r];
+            for (int r = 0; r < 4; ++r) sv[u][r] = s_acc[m][u][r];
           if (cap != 0.f) {
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -210,26 +248,36 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
           const bool need_mask = !act[m] || a0 + 31 > t_pos_lo[m] || a0 + 32 > range_hi || (W > 0 && a0 <= t_pos_hi[m] - W);
           if (need_mask) {
+            int tok0 = a0 + 4 * g;
+            asm volatile("" : "+v"(tok0));  // keeps the per-key compares inside this (rare) branch
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
-                const int tok = a0 + 16 * u + 4 * g + r;
+                const int tok = tok0 + 16 * u + r;
                 const bool keep = tok <= pos_n[m] && tok < range_hi && (W <= 0 || tok > pos_n[m] - W);
                 sv[u][r] = keep ? sv[u][r] : -INFINITY;
               }
           }
           float tmax = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
                              fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
-          tmax = fmaxf(tmax, __shfl_xor(tmax, 16, kWave));
-          tmax = fmaxf(tmax, __shfl_xor(tmax, 32, kWave));
-          // Lazy rescale: the reference point m_run only moves when the tile maximum exceeds it by more than
-          // kLazy (probabilities then stay below e^kLazy, far inside bf16/fp32 range), so rescaling O is rare.
-          const bool bump = tmax > m_run[m] + kLazy;
-          const float m_new = bump ? tmax : m_run[m];
-          const float m_use = m_new == -INFINITY ? 0.f : m_new;
-          const float alpha = bump ? __builtin_amdgcn_exp2f((m_run[m] - m_use) * kLog2e) : 1.f;
-          m_run[m] = m_new;
+          // Lazy rescale: the reference point m_run (the same in the four lanes of a row) only moves when some
+          // logit exceeds it by more than kLazy; probabilities then stay below e^kLazy, far inside bf16 / fp32
+          // range.  The common case needs no cross-lane step at all: a wave-wide vote on the lane-local maxima.
+          float alpha = 1.f;
+          if (__builtin_expect(__any(tmax > m_run[m] + kLazy), 0)) {
+            tmax = row_groups_max(tmax);
+            const bool bump = tmax > m_run[m] + kLazy;
+            const float m_new = bump ? tmax : m_run[m];
+            alpha = bump ? __builtin_amdgcn_exp2f((m_run[m] - m_new) * kLog2e) : 1.f;  // m_new is finite here
+            m_run[m] = m_new;
+            l_acc[m] *= alpha;
+#pragma unroll
+            for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+              for (int c = 0; c < 8; ++c) o_acc[m][sN][c] *= alpha;
+          }
+          const float m_use = m_run[m] == -INFINITY ? 0.f : m_run[m];
           const float neg = -m_use * kLog2e;
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
@@ -240,25 +288,13 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
             pw[m][2 * u] = pack_bf16x2(e0, e1);
             pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
           }
-          if (__builtin_expect(__any(bump), 0)) {
-            l_acc[m] *= alpha;
-#pragma unroll
-            for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-              for (int c = 0; c < 8; ++c) o_acc[m][sN][c] *= alpha;
-          }
           l_acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ones),
                                                             __builtin_bit_cast(bf16x8_t, pw[m]), l_acc[m], 0, 0, 0);
         }
         // O^T += V^T P^T: the eight fetched pieces of a slice give eight A operands, each used by every row tile
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
-          __builtin_amdgcn_sched_barrier(0);
-          u32x4_t vch[8];
-#pragma unroll
-          for (int e = 0; e < 8; ++e)
-            vch[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2) + 4 * g + (e & 3)) * C::ROWB +
-                                                       16 * ((i + 16 * sN) ^ (4 * g + (e & 3))));
+          if (sN > 0) load_v(sN);
 #pragma unroll
           for (int c = 0; c < 8; ++c) {
             const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
@@ -270,6 +306,13 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               o_acc[m][sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                   __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, pw[m]), o_acc[m][sN][c], 0, 0, 0);
           }
+          if (sN > 0) __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+          for (int c = 0; c < 8; ++c) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);    // four byte permutes build one A operand
+            __builtin_amdgcn_sched_group_barrier(0x008, MRT, 1);  // its MFMAs
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }

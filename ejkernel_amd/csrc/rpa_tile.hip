@@ -121,12 +121,26 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     return __builtin_amdgcn_readfirstlane(lo);
   };
 
-  // ---- prefill: one item per (sequence, tile of WGROWS rows, kv head), strided over the workgroups
-  for (int w = blockIdx.x; w < total_wg; w += gridDim.x) {
-    const int s = find(wg_start, w);
-    const SeqInfo si = seq_info<C::TT>(p, s, G);
-    const int local = __builtin_amdgcn_readfirstlane(w - wg_start[s]);
-    prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, local % p.num_kv_heads, local / p.num_kv_heads);
+  // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)
+  // adjacent in the item order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2:
+  // numbering the workgroups XCD by XCD makes the row tiles that share one K/V stream run at the same time on the
+  // same XCD, so all but the first of them read it from that L2.  Within a (sequence, kv head) the row tiles are
+  // rotated by the round in which the group starts: a workgroup then meets early (short) and late (long) causal
+  // tiles in turn instead of always the same one.
+  {
+    const int n_xcd = gridDim.x % 8 == 0 ? 8 : 1;
+    const int vwg = (blockIdx.x % n_xcd) * (gridDim.x / n_xcd) + blockIdx.x / n_xcd;
+    for (int w = vwg; w < total_wg; w += gridDim.x) {
+      const int s = find(wg_start, w);
+      const SeqInfo si = seq_info<C::TT>(p, s, G);
+      const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
+      const int base = __builtin_amdgcn_readfirstlane(wg_start[s]);
+      const int local = w - base;
+      const int j = local / n_qt, member = local - j * n_qt;
+      const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
+      const int qt = (member + 5 * round0) % n_qt;
+      prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
+    }
   }
   // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
   // workgroup has finished reading them.
@@ -181,10 +195,11 @@ static int env_int(const char* name, int dflt) {
   return v && *v ? atoi(v) : dflt;
 }
 
-// Workgroups of the persistent grid: one per compute unit (four wavefronts each) measured best for the
-// bandwidth-bound decode stream; RPA_TUNE_WGS_PER_CU overrides it for experiments (1..kTiledMaxWgsPerCu).
+// Workgroups of the persistent grid: two per compute unit (two wavefronts per SIMD, so one wavefront's LDS and
+// softmax latency hides behind the other's MFMAs in prefill tiles); the decode stream alone is ~3 % faster with
+// one.  RPA_TUNE_WGS_PER_CU overrides it for experiments (1..kTiledMaxWgsPerCu).
 static int tiled_grid() {
-  const int per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 1)));
+  const int per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 2)));
   return device_cu_count() * per_cu;
 }
 
@@ -246,7 +261,7 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   const bool mimic = env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
   if (p.head_dim == 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
-  return mimic ? launch_cfg<256, 1, 2, true>(a, grid, stream) : launch_cfg<256, 1, 2, false>(a, grid, stream);
+  return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);
 }
 
 }  // namespace rpa

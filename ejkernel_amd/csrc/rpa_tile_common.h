@@ -107,4 +107,20 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 __device__ __forceinline__ float rbf(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
 
+// Reductions over the four lane groups that hold one query row (lanes l, l^16, l^32, l^48), with the gfx950
+// lane-swap instructions instead of LDS permutes: swapping a value with itself yields, in every 16-lane row,
+// both members of a row pair (then of a half-wave pair).
+__device__ __forceinline__ float row_groups_max(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  const float y = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(y), __float_as_uint(y), false, false);
+  return fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+}
+__device__ __forceinline__ float row_groups_sum(float x) {
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+  const float y = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(y), __float_as_uint(y), false, false);
+  return __uint_as_float(b[0]) + __uint_as_float(b[1]);
+}
+
 }  // namespace rpa
