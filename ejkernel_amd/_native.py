@@ -7,9 +7,11 @@ op fails with an error that says how to build it.
 from __future__ import annotations
 
 import ctypes
+import os
 from pathlib import Path
 
-LIB_PATH = Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so"
+# RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
+LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
 RPA_ABI_VERSION = 1
 RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1

@@ -24,13 +24,19 @@ template <int D, int MRT>
 struct PCfg {
   static constexpr int NS = D / 128;                 // 128-wide slices of head_dim
   static constexpr int NKS = D / 32;                 // k-steps of the QK^T contraction
-  static constexpr int NH = D == 128 ? 2 : 1;        // 32-token halves per step
+#ifndef RPA_PF_NH
+#define RPA_PF_NH 2
+#endif
+#ifndef RPA_PF_NSTG
+#define RPA_PF_NSTG 2
+#endif
+  static constexpr int NH = D == 128 ? RPA_PF_NH : 1;  // 32-token halves per step
   static constexpr int TK = 32 * NH;                 // tokens per step
   static constexpr int ROWB = D * 2;                 // LDS bytes per row
   static constexpr int WROWS = 16 * MRT;             // rows per wavefront
   static constexpr int WGROWS = kWgWaves * WROWS;    // rows per workgroup
   static constexpr int TILE_B = TK * ROWB;           // one K (or V) tile: 16 KiB
-  static constexpr int NSTG = 2;                     // LDS stages: tiles requested ahead of the one in use + 1
+  static constexpr int NSTG = RPA_PF_NSTG;           // LDS stages: tiles requested ahead of the one in use + 1
   static constexpr int LDS = 2 * NSTG * TILE_B;      // K and V tile per stage
   static constexpr int PR = D / 8;                   // 16-byte pieces per row
   static constexpr int RB = kWave / PR;              // rows one wave-wide load instruction covers
@@ -145,10 +151,15 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // order); the barrier that follows publishes the oldest tile.  s_waitcnt takes an immediate: vmcnt is bits
   // [3:0] and [15:14]; 0x0F70 leaves the other counters unconstrained.
   auto wait_fetch = [&](int ahead) {
-    static_assert(C::BPW == 8 && C::NSTG <= 4, "vmcnt immediates below assume 8 loads per tile, <= 2 tiles ahead");
-    if (ahead <= 0) __builtin_amdgcn_s_waitcnt(0x0F70);
-    else if (ahead == 1) __builtin_amdgcn_s_waitcnt(0x0F78);
-    else __builtin_amdgcn_s_waitcnt(0x4F70);
+    static_assert(C::BPW * (C::NSTG - 2) <= 24, "extend the immediates below");
+    switch (ahead * C::BPW) {
+      case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
+      case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
+      case 8: __builtin_amdgcn_s_waitcnt(0x0F78); break;
+      case 12: __builtin_amdgcn_s_waitcnt(0x0F7C); break;
+      case 16: __builtin_amdgcn_s_waitcnt(0x4F70); break;
+      default: __builtin_amdgcn_s_waitcnt(0x4F78); break;  // 24
+    }
   };
 
   const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};  // eight bf16 1.0

@@ -130,11 +130,17 @@ WORKLOADS = {
                             "32q/8kv heads, D=128, page 32",
     "gemma2_local": "64 seqs x 4 tokens, kv 2048..32768, 16q/8kv heads, D=256, page 16, window 4096, cap 50",
     "decode_long_context": "32 seqs x 1 token, kv 32768..131072, 64q/8kv heads, D=128, page 64, 2^18 pages",
+    # the two halves of mixed_prefill_decode on their own (same lengths), to price each against its own roofline
+    "mixed_prefill_only": "the 16 prefill chunks of mixed_prefill_decode: 512 tokens each, prior 0..4096",
+    "mixed_decode_only": "the 240 decode sequences of mixed_prefill_decode: 1 token each, kv 256..8192",
 }
 
 
 def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bfloat16) -> Batch:
     """Build a named workload. ``scale`` < 1 shrinks sequence counts and lengths for tests."""
+    only = None
+    if name in ("mixed_prefill_only", "mixed_decode_only"):
+        only, name = name, "mixed_prefill_decode"
     idx = list(WORKLOADS).index(name) + 1
     seed = 1000 + idx
     rng = np.random.Generator(np.random.PCG64(seed))
@@ -167,9 +173,11 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         q = np.concatenate([np.full(n_pre, chunk), np.ones(n_dec, int)])
         kv = np.concatenate([prior + chunk, kv_dec])
         order = rng.permutation(n_pre + n_dec)
+        if only is not None:
+            order = np.array([o for o in order if (o < n_pre) == (only == "mixed_prefill_only")])
         pps = pages(max(n(8192), n(4096) + chunk), 32)
         return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
-                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=name)
+                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=only or name)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)
