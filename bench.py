@@ -38,50 +38,59 @@ def parse():
     return ap.parse_args()
 
 
-def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs):
-    """Runs the CPU oracle on a sample of the batch's sequences: times it and checks the device rows."""
+def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs, budget_s=12.0):
+    """Times the CPU restatement of the reference's XLA path (oracle/rpa_oracle.c, OpenMP over all host cores)
+    on a bounded sample of the batch's sequences and checks the device rows of that sample against it."""
     import numpy as np
-    import torch
-    from threadpoolctl import threadpool_info
 
     from ejkernel_amd.workloads import compact_for_host
-    from tests.helpers import err_stats, run_exact, run_strict, to_np
+    from oracle import rpa_oracle_c
+    from tests.helpers import err_stats, oracle_args, run_exact, to_np
 
     S = len(batch.q_lens)
     rng = np.random.default_rng(0)
     cand = [int(s) for s in rng.permutation(S) if batch.q_lens[s] > 0]
+    threads = rpa_oracle_c.max_threads()
+
+    def run(ids):
+        sub = compact_for_host(batch, sorted(ids))
+        args = oracle_args(sub)
+        t0 = time.perf_counter()
+        ref = rpa_oracle_c.rpa_strict_c(*args, softmax_scale=sub.softmax_scale, logits_soft_cap=sub.logits_soft_cap,
+                                        sliding_window=sub.sliding_window, io_dtype="bfloat16", threads=threads)
+        return sub, ref, time.perf_counter() - t0
+
     if n_seqs <= 0:
-        # about 2e9 key-row-head products per second for the NumPy port; aim at ~10 s
-        budget, n_seqs, acc = 2.0e10, 0, 0.0
-        Hq, D = batch.queries.shape[1], batch.queries.shape[2]
+        # probe with a few sequences, then size the sample for about `budget_s` seconds of CPU work
+        probe = cand[:max(1, min(len(cand), threads // 8 or 1))]
+        sub, _, dt = run(probe)
+        work = lambda ids: float(sum((-(-int(batch.q_lens[s]) // 8)) * int(batch.kv_lens[s]) for s in ids))  # noqa: E731
+        rate = work(probe) / max(dt, 1e-3)
+        n_seqs, acc = 0, 0.0
         for s in cand:
-            rows8 = -(-int(batch.q_lens[s]) // 8) * 8
-            acc += rows8 * float(batch.kv_lens[s]) * Hq * D
+            acc += work([s])
             n_seqs += 1
-            if acc > budget:
+            if acc / rate > budget_s:
                 break
-    ids = sorted(cand[:max(1, n_seqs)])
-    sub = compact_for_host(batch, ids)
-    t0 = time.perf_counter()
-    ref = run_strict(sub)
-    dt = time.perf_counter() - t0
+    ids = cand[:max(1, n_seqs)]
+    sub, ref, dt = run(ids)
     rows = sub.total_valid_tokens
     res = {}
     if want_parity:
         got = to_np(out[sub.meta["rows"].to(out.device)])
         bad = np.isnan(ref[:rows]).any(axis=(1, 2))
-        if bad.any():  # strict oracle NaN rows (window defect of the reference): compare with the float64 form
+        if bad.any():  # NaN rows of the reference program (window defect): compare with the float64 evaluation
             ref = ref.copy()
             ref[:rows][bad] = run_exact(sub)[:rows][bad]
         mx, mean = err_stats(got, ref, rows)
         res["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": rows, "oracle_nan_rows": int(bad.sum()),
                          "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
     if want_baseline:
-        threads = max([i.get("num_threads", 1) for i in threadpool_info()] or [1])
         res["cpu_baseline"] = {
             "value": rows / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
-            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens), "
-                      f"NumPy restatement of the XLA path, {dt:.2f} s",
+            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens) in "
+                      f"{dt:.2f} s; C restatement of the reference's XLA path (8-row query blocks, 64-page KV blocks, "
+                      f"bf16 rounding points), OpenMP over {threads} threads",
         }
     return res
 

@@ -366,3 +366,46 @@ def test_algorithmic_counts_small_case():
     cw = O.algorithmic_counts([10, 7], [0, 3, 4], [2], num_q_heads=4, num_kv_heads=2, head_dim=8, page_size=4,
                               sliding_window=2)
     assert cw["pairs"] == 2 * 4 and cw["kv_bytes"] == (min(10, 3 + 1) + min(7, 1 + 1)) * 2 * 2 * 8 * 2
+
+
+# ----------------------------------------------------------------------------- C restatement vs NumPy restatement
+
+
+def _c_strict(b, softmax_aux=None, threads=2):
+    from oracle.rpa_oracle_c import rpa_strict_c
+
+    dt = "bfloat16" if b.queries.dtype == torch.bfloat16 else "float32"
+    return rpa_strict_c(*oracle_args(b), softmax_scale=b.softmax_scale, logits_soft_cap=b.logits_soft_cap,
+                        sliding_window=b.sliding_window, softmax_aux=softmax_aux, io_dtype=dt, threads=threads)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_c_restatement_matches_numpy_restatement(dtype):
+    """Same algorithm, same rounding points: only fp32 summation order may differ (a last-place flip at most)."""
+    rng = np.random.default_rng(8)
+    sinks = rng.standard_normal((2, 2)).astype(np.float32)
+    cases = [
+        (make_workload("decode_small", dtype=dtype), None),
+        (make_batch([9, 1, 0, 17, 2], [40, 64, 8, 17, 33], num_q_heads=8, num_kv_heads=2, head_dim=32, page_size=8,
+                    pages_per_seq=8, seed=1, dtype=dtype, sliding_window=20, logits_soft_cap=5.0, max_num_seqs=7), None),
+        (make_batch([5, 1], [500, 1000], num_q_heads=4, num_kv_heads=2, head_dim=64, page_size=8, pages_per_seq=128,
+                    seed=11, dtype=dtype), sinks),
+    ]
+    for b, aux in cases:
+        rows = b.total_valid_tokens
+        want = run_strict(b, softmax_aux=aux)
+        got = _c_strict(b, softmax_aux=aux)
+        d = np.abs(got[:rows] - want[:rows])
+        if dtype == torch.bfloat16:  # rounded results: identical except where a sum sat on a rounding boundary
+            assert d.max() <= 4e-3 and (d > 0).mean() < 2e-3, (d.max(), (d > 0).mean())
+        else:
+            assert d.max() <= 2e-6, d.max()
+        assert not got[rows:].any()
+
+
+def test_c_restatement_reproduces_window_nan():
+    b = make_batch([2], [400], num_q_heads=2, num_kv_heads=1, head_dim=16, page_size=4, pages_per_seq=128, seed=4,
+                   dtype=torch.float32, sliding_window=50)
+    assert np.isnan(_c_strict(b)[:2]).all()
+    b.sliding_window = 200
+    assert np.abs(_c_strict(b)[:2] - run_exact(b)[:2]).max() < 1e-5
