@@ -74,6 +74,11 @@ def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs, budget
                 break
     ids = cand[:max(1, n_seqs)]
     sub, ref, dt = run(ids)
+    reps = 1
+    while dt * reps < budget_s and reps < 20:  # a fast host: repeat the sample until ~budget_s of CPU work is timed
+        _, _, dt_k = run(ids)
+        dt = (dt * reps + dt_k) / (reps + 1)
+        reps += 1
     rows = sub.total_valid_tokens
     res = {}
     if want_parity:
@@ -88,8 +93,8 @@ def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs, budget
     if want_baseline:
         res["cpu_baseline"] = {
             "value": rows / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
-            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens) in "
-                      f"{dt:.2f} s; C restatement of the reference's XLA path (8-row query blocks, 64-page KV blocks, "
+            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens), mean of "
+                      f"{reps} runs of {dt:.2f} s; C restatement of the reference's XLA path (8-row query blocks, 64-page KV blocks, "
                       f"bf16 rounding points), OpenMP over {threads} threads",
         }
     return res

@@ -108,7 +108,11 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       for (int k = tid; k < row_u4; k += kWgThreads) o4[static_cast<size_t>(row) * row_u4 + k] = u32x4_t{0u, 0u, 0u, 0u};
   }
 
-  const int n_workers = gridDim.x * kWgWaves;
+  // A batch without prefill tiles is pure streaming: it runs fastest with one workgroup per compute unit, so
+  // the second half of the grid (dispatched after every unit has one workgroup) leaves at once.
+  const int grid_wgs = total_wg == 0 ? min(static_cast<int>(gridDim.x), a.decode_grid) : static_cast<int>(gridDim.x);
+  if (static_cast<int>(blockIdx.x) >= grid_wgs) return;
+  const int n_workers = grid_wgs * kWgWaves;
   const int worker = blockIdx.x * kWgWaves + wave;
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
@@ -253,6 +257,7 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.p = p;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
+  a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 1));
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
