@@ -1,0 +1,82 @@
+"""The five benchmark workloads at their full sizes on the device.
+
+At these sizes the whole batch cannot go through the CPU oracle in seconds, so each workload is checked
+(a) on a seeded sample of its sequences against the C restatement of the reference (same tolerance as the
+small cases: max-abs <= 2e-2, mean-abs <= 2e-3; rows where the reference program yields NaN -- a leading KV
+block entirely left of the sliding window -- are compared with the float64 evaluation), and (b) through
+properties that do not depend on size: finite output, zero rows past the batch, bitwise invariance under a
+permutation of the physical pages, bitwise reproducibility, and agreement of every decode row with the same
+sequence run alone (identical up to the fp32 rounding of a different split, i.e. a last-place bf16 flip).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from ejkernel_amd.modules import ragged_page_attention
+from ejkernel_amd.workloads import Batch, compact_for_host, make_workload
+from oracle import rpa_oracle_c
+from tests.helpers import BF16_MAX_ABS, BF16_MEAN_ABS, err_stats, oracle_args, run_exact, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def run(b):
+    out = ragged_page_attention(*b.args(), **b.kwargs())
+    torch.cuda.synchronize()
+    return out
+
+
+def check_sample(b, out, n_seqs, seed=0):
+    rng = np.random.default_rng(seed)
+    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:n_seqs])
+    sub = compact_for_host(b, ids)
+    ref = rpa_oracle_c.rpa_strict_c(*oracle_args(sub), softmax_scale=sub.softmax_scale,
+                                    logits_soft_cap=sub.logits_soft_cap, sliding_window=sub.sliding_window)
+    rows = sub.total_valid_tokens
+    nan_rows = np.isnan(ref[:rows]).any(axis=(1, 2))
+    if nan_rows.any():
+        ref[:rows][nan_rows] = run_exact(sub)[:rows][nan_rows]
+    got = to_np(out[sub.meta["rows"].to(out.device)])
+    mx, mean = err_stats(got, ref, rows)
+    assert mx <= BF16_MAX_ABS and mean <= BF16_MEAN_ABS, (b.name, mx, mean)
+    return sub, int(nan_rows.sum())
+
+
+def permuted(b, seed=9):
+    P = b.kv_pages.shape[0]
+    perm = torch.randperm(P, generator=torch.Generator().manual_seed(seed)).to(DEV)
+    inv = torch.empty_like(perm)
+    inv[perm] = torch.arange(P, device=DEV)
+    b2 = Batch(**{**b.__dict__})
+    b2.kv_pages = b.kv_pages[perm]
+    b2.block_tables = inv[b.block_tables.long()].to(torch.int32)
+    return b2
+
+
+@pytest.mark.parametrize("name,n_sample,permute", [("decode_small", 8, True), ("decode_llama3_8b", 12, True),
+                                                   ("mixed_prefill_decode", 14, True), ("gemma2_local", 4, False),
+                                                   ("decode_long_context", 2, False)])
+def test_full_size_workload(name, n_sample, permute):
+    b = make_workload(name, device=DEV)
+    out = run(b)
+    total = b.total_valid_tokens
+    assert torch.isfinite(out.float()).all()
+    assert not out[total:].any()
+    assert torch.equal(run(b), out)  # reproducible bit for bit
+    sub, _ = check_sample(b, out, n_sample)
+    if permute:
+        assert torch.equal(run(permuted(b)), out)
+    # one sampled sequence on its own: same rows up to a last-place flip
+    s = int(np.argmax(b.q_lens == b.q_lens.min()))
+    alone = compact_for_host(b, [s])
+    dev = Batch(**{**alone.__dict__})
+    for f in ("queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs"):
+        setattr(dev, f, getattr(alone, f).to(DEV))
+    got = run(dev)[: int(b.q_lens[s])].float()
+    cu = b.query_start_loc.cpu().numpy()
+    want = out[cu[s]:cu[s + 1]].float()
+    assert (got - want).abs().max().item() <= 2.0 ** -7 * max(1.0, want.abs().max().item())
+    del b, out
+    torch.cuda.empty_cache()
