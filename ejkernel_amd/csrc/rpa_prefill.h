@@ -102,6 +102,17 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
     }
   }
+  // First key of a 32-key half, a0, against per-row-tile thresholds (wave-uniform, fixed for the item):
+  //   a0 > act_hi or a0 <= act_lo   the row tile sees none of the half's keys
+  //   a0 <= nomask_hi and a0 > nomask_lo   it sees all of them: no per-key mask needed
+  int act_hi[MRT], act_lo[MRT], nomask_hi[MRT], nomask_lo[MRT];
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    act_hi[m] = t_any[m] ? t_pos_hi[m] : -0x7fffffff;
+    act_lo[m] = W > 0 ? t_pos_lo[m] - W - 31 : -0x7fffffff;
+    nomask_hi[m] = min(t_pos_lo[m] - 31, range_hi - 32);
+    nomask_lo[m] = W > 0 ? t_pos_hi[m] - W : -0x7fffffff;
+  }
   const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;  // < w_pos_lo when the wave has no rows
   const int w_pos_lo = pos0 + w_row_lo / G;
   const bool w_any = w_row_lo < si.rows;
@@ -119,32 +130,54 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       for (int c = 0; c < 8; ++c) o_acc[m][sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
-  // ---- cooperative fetch.  Block b of a step (b < BLOCKS: K rows RB*b .., else V rows) is one wave-wide
-  // direct-to-LDS load: the LDS side is 1 KiB in lane order, so lane l fills piece slot l % PR of row l / PR and
-  // fetches the piece that the swizzle assigns to that slot.  The RB rows of a block share a page (RB <= 4 <=
-  // page_size), so the block-table entry is a scalar load.
+  // ---- cooperative fetch.  One wave-wide direct-to-LDS load moves a block of RB rows: the LDS side is 1 KiB in
+  // lane order, so lane l fills piece slot l % PR of row l / PR and fetches the piece that the swizzle assigns
+  // to that slot.  Block-table entries are scalar loads (the rows of a block always share a page).
   const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * D) * 2u;
   const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
       reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
   const int l_row = lane / C::PR, l_slot = lane % C::PR;
-  auto fetch_tile = [&](int tile, int buf) {
+  // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
+  constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
+  uint32_t pre_off[HB];  // per-lane byte offset of block n inside the group: row part + swizzled piece
 #pragma unroll
-    for (int n = 0; n < C::BPW; ++n) {
-      const int b = wave + kWgWaves * n;          // 0 .. 2*BLOCKS-1
-      const int is_v = b / C::BLOCKS, rb = b % C::BLOCKS;
-      const int t_c = min(tile + C::RB * rb, t_last & ~(C::RB - 1));  // past the range: repeat the last keys (masked)
+  for (int n = 0; n < HB; ++n) {
+    const int t_local = GROUP * wave + C::RB * n + l_row;
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
+  }
+  const bool group_in_page = p.page_size >= GROUP;
+  auto fetch_tile = [&](int tile, int buf) {
+    const int t_first = tile + GROUP * wave;
+    char* dst = lds + 2 * buf * C::TILE_B + HB * wave * 1024;
+    if (group_in_page && t_first + GROUP - 1 <= t_last) {
+      // the whole group lies in one page and inside the range: one block-table entry, one base address
+      const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
+      const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * D * 2;
+#pragma unroll
+      for (int n = 0; n < HB; ++n) {
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n]),
+                                         (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n] + D * 2),
+                                         (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+      }
+      return;
+    }
+    // last tile of the range or small pages: per block, keys past the range repeat the last one (masked)
+#pragma unroll
+    for (int n = 0; n < HB; ++n) {
+      const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
       const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b;
+                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * D * 2;
       const int tok = min(t_c + l_row, t_last);
-      const int t_local = C::RB * rb + l_row;     // row inside the tile
-      const int piece = l_slot ^ (t_local & 15);
-      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b +
-                           static_cast<uint32_t>((2 * j + is_v) * D * 2 + 16 * piece);
-      char* dst = lds + (2 * buf + is_v) * C::TILE_B + rb * 1024;
+      const int t_local = GROUP * wave + C::RB * n + l_row;
+      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
-                                       (__attribute__((address_space(3))) void*)(dst), 16, 0, 0);
+                                       (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off + D * 2),
+                                       (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
     }
   };
   // Wait until at most `ahead` later tiles of this wave's direct-to-LDS loads are outstanding (they complete in
@@ -192,9 +225,6 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         const int a0 = tile + 32 * h;  // first key of this half
         const bool w_skip = !w_any || a0 >= range_hi || a0 > w_pos_hi || (W > 0 && a0 + 31 <= w_pos_lo - W);
         if (w_skip) continue;
-        bool act[MRT];
-#pragma unroll
-        for (int m = 0; m < MRT; ++m) act[m] = t_any[m] && a0 <= t_pos_hi[m] && !(W > 0 && a0 + 31 <= t_pos_lo[m] - W);
         // S^T = K Q^T for the two 16-key sub-tiles.  The eight K operands are requested first and the V pieces of
         // the first slice while the QK MFMAs run, so LDS latency is paid once per half and V is in registers by
         // the time the softmax is done.  The group barriers pin that order (the scheduler would otherwise sink
@@ -257,7 +287,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                 sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
           }
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
-          const bool need_mask = !act[m] || a0 + 31 > t_pos_lo[m] || a0 + 32 > range_hi || (W > 0 && a0 <= t_pos_hi[m] - W);
+          const bool need_mask = a0 > nomask_hi[m] || a0 <= nomask_lo[m] || a0 > act_hi[m] || a0 <= act_lo[m];
           if (need_mask) {
             int tok0 = a0 + 4 * g;
             asm volatile("" : "+v"(tok0));  // keeps the per-key compares inside this (rare) branch

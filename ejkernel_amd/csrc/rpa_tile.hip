@@ -125,69 +125,81 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     return __builtin_amdgcn_readfirstlane(lo);
   };
 
-  // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)
-  // adjacent in the item order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2:
-  // numbering the workgroups XCD by XCD makes the row tiles that share one K/V stream run at the same time on the
-  // same XCD, so all but the first of them read it from that L2.  Within a (sequence, kv head) the row tiles are
-  // rotated by the round in which the group starts: a workgroup then meets early (short) and late (long) causal
-  // tiles in turn instead of always the same one.
-  {
-    const int n_xcd = gridDim.x % 8 == 0 ? 8 : 1;
-    const int vwg = (blockIdx.x % n_xcd) * (gridDim.x / n_xcd) + blockIdx.x / n_xcd;
-    for (int w = vwg; w < total_wg; w += gridDim.x) {
-      const int s = find(wg_start, w);
-      const SeqInfo si = seq_info<C::TT>(p, s, G);
-      const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
-      const int base = __builtin_amdgcn_readfirstlane(wg_start[s]);
-      const int local = w - base;
-      const int j = local / n_qt, member = local - j * n_qt;
-      const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
-      const int qt = (member + 5 * round0) % n_qt;
-      prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
-    }
-  }
-  // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
-  // workgroup has finished reading them.
-  __syncthreads();
+  // Prefill tiles are compute-bound and the decode stream is bandwidth-bound: the two workgroups that share a
+  // compute unit take the two kinds of work in opposite order, so each unit has matrix work and memory traffic
+  // in flight at the same time instead of one after the other.
+  const bool stream_first = total_wg > 0 && (a.phase_mode == 1 ? static_cast<int>(blockIdx.x) >= a.decode_grid
+                                            : a.phase_mode == 2 ? (blockIdx.x & 1) != 0
+                                            : a.phase_mode == 3 ? ((blockIdx.x >> 3) & 1) != 0 : false);
+#pragma unroll 1
+  for (int phase = 0; phase < 2; ++phase) {
+    if ((phase == 0) != stream_first) {
+      // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)
+      // adjacent in the item order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2:
+      // numbering the workgroups XCD by XCD makes the row tiles that share one K/V stream run at the same time on the
+      // same XCD, so all but the first of them read it from that L2.  Within a (sequence, kv head) the row tiles are
+      // rotated by the round in which the group starts: a workgroup then meets early (short) and late (long) causal
+      // tiles in turn instead of always the same one.
+      {
+        const int n_xcd = gridDim.x % 8 == 0 ? 8 : 1;
+        const int vwg = (blockIdx.x % n_xcd) * (gridDim.x / n_xcd) + blockIdx.x / n_xcd;
+        for (int w = vwg; w < total_wg; w += gridDim.x) {
+          const int s = find(wg_start, w);
+          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
+          const int base = __builtin_amdgcn_readfirstlane(wg_start[s]);
+          const int local = w - base;
+          const int j = local / n_qt, member = local - j * n_qt;
+          const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
+          const int qt = (member + 5 * round0) % n_qt;
+          prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
+        }
+      }
+      // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
+      // workgroup has finished reading them.
+      __syncthreads();
 
-  // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
-  for (int w = worker; w < total_items; w += n_workers) {
-    const int s = find(item_start, w);
-    const SeqInfo si = seq_info<C::TT>(p, s, G);
-    const int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
-    const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
-    const int row_hi = min(rt * 16 + 16, si.rows);
-    const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
-    const int range_hi = min(si.kv_len, pos_max + 1);
-    const int range_lo = (p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0) & ~(C::TT - 1);
-    Part part;
-    part.partial = false;
-    process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
-  }
+    } else {
+      // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
+      for (int w = worker; w < total_items; w += n_workers) {
+        const int s = find(item_start, w);
+        const SeqInfo si = seq_info<C::TT>(p, s, G);
+        const int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
+        const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
+        const int row_hi = min(rt * 16 + 16, si.rows);
+        const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
+        const int range_hi = min(si.kv_len, pos_max + 1);
+        const int range_lo = (p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0) & ~(C::TT - 1);
+        Part part;
+        part.partial = false;
+        process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+      }
 
-  // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
-  if (total_tiles > 0) {
-    Shares sh;
-    sh.q = total_tiles / n_workers;
-    sh.rem = total_tiles - sh.q * n_workers;
-    int x = sh.begin(worker);
-    const int x_end = sh.begin(worker + 1);
-    while (x < x_end) {
-      const int s = find(tile_start, x);
-      const SeqInfo si = seq_info<C::TT>(p, s, G);
-      const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
-      const int local = __builtin_amdgcn_readfirstlane(x - tile_start[s]);
-      const int j = local / per_head, t0 = local - j * per_head;
-      const int t1 = min(per_head, t0 + (x_end - x));
-      Part part;
-      part.stream_a = x - t0;
-      part.sh = sh;
-      part.first_w = sh.owner(part.stream_a);
-      part.last_w = sh.owner(part.stream_a + per_head - 1);
-      part.partial = part.first_w != part.last_w;
-      part.slot = part_slot(worker, part.stream_a, sh);
-      process_item<D, NT, kMimic>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
-      x += t1 - t0;
+      // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
+      if (total_tiles > 0) {
+        Shares sh;
+        sh.q = total_tiles / n_workers;
+        sh.rem = total_tiles - sh.q * n_workers;
+        int x = sh.begin(worker);
+        const int x_end = sh.begin(worker + 1);
+        while (x < x_end) {
+          const int s = find(tile_start, x);
+          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
+          const int local = __builtin_amdgcn_readfirstlane(x - tile_start[s]);
+          const int j = local / per_head, t0 = local - j * per_head;
+          const int t1 = min(per_head, t0 + (x_end - x));
+          Part part;
+          part.stream_a = x - t0;
+          part.sh = sh;
+          part.first_w = sh.owner(part.stream_a);
+          part.last_w = sh.owner(part.stream_a + per_head - 1);
+          part.partial = part.first_w != part.last_w;
+          part.slot = part_slot(worker, part.stream_a, sh);
+          process_item<D, NT, kMimic>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+          x += t1 - t0;
+        }
+      }
     }
   }
 }
@@ -257,6 +269,7 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.p = p;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
+  a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 1);
   a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 1));
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);

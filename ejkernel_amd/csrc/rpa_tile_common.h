@@ -22,6 +22,7 @@ struct TileArgs {
   int page_shift;     // log2(page_size)
   int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
   int decode_grid;    // workgroups that take part when the batch has no prefill tiles
+  int phase_mode;     // which workgroups stream first in a mixed batch (0 none, 1 upper half of the grid, 2 odd, 3 odd octets)
   uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
   float* partial_o;   // [2 * wavefronts of the grid][16][D]
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
