@@ -74,6 +74,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(bt));
   const int t_last = range_hi - 1;
   const float cap = p.logits_soft_cap;
+  const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
 
   u32x4_t kreg[C::NSLOT][C::NS];
   u32x4_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
@@ -165,7 +166,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       for (int u = 0; u < NT; ++u)
 #pragma unroll
         for (int r = 0; r < 4; ++r)
-          sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
+          sv[u][r] = soft_cap<kMimic>(sv[u][r], cap, inv_cap);
     }
     if (need_mask) {
 #pragma unroll

@@ -60,6 +60,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
   const char* kvb = static_cast<const char*>(p.kv_pages);
   const float cap = p.logits_soft_cap;
+  const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
   const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
 
   // ---- key range of the workgroup's rows
@@ -284,7 +285,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
             for (int u = 0; u < 2; ++u)
 #pragma unroll
               for (int r = 0; r < 4; ++r)
-                sv[u][r] = kMimic ? rbf(rbf(tanhf(rbf(sv[u][r] / cap))) * cap) : cap * tanhf(sv[u][r] / cap);
+                sv[u][r] = soft_cap<kMimic>(sv[u][r], cap, inv_cap);
           }
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
           const bool need_mask = a0 > nomask_hi[m] || a0 <= nomask_lo[m] || a0 > act_hi[m] || a0 <= act_lo[m];

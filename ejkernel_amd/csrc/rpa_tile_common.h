@@ -109,6 +109,23 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 }
 __device__ __forceinline__ float rbf(float x) { return static_cast<float>(static_cast<__bf16>(x)); }
 
+// tanh through the hardware exp2 and reciprocal: 1 - 2 / (1 + e^(2x)), which saturates correctly for large |x|
+// and has an absolute error near 1e-7; below |x| = 1/16, where that would be a large relative error, the odd
+// series x (1 - x^2/3 + 2 x^4/15) takes over (relative error < 1e-8 there).  Branch-free.
+__device__ __forceinline__ float tanh_fast(float x) {
+  const float e = __builtin_amdgcn_exp2f(x * (2.f * kLog2e));
+  const float big = fmaf(-2.f, __builtin_amdgcn_rcpf(1.f + e), 1.f);
+  const float x2 = x * x;
+  const float small = x * fmaf(x2, fmaf(x2, 2.f / 15.f, -1.f / 3.f), 1.f);
+  return fabsf(x) < 0.0625f ? small : big;
+}
+// cap * tanh(x / cap) with the reference's bf16 rounding after each op (kMimic) or in plain fp32.
+template <bool kMimic>
+__device__ __forceinline__ float soft_cap(float x, float cap, float inv_cap) {
+  if (kMimic) return rbf(rbf(tanh_fast(rbf(x * inv_cap))) * cap);
+  return cap * tanh_fast(x * inv_cap);
+}
+
 // Reductions over the four lane groups that hold one query row (lanes l, l^16, l^32, l^48), with the gfx950
 // lane-swap instructions instead of LDS permutes: swapping a value with itself yields, in every 16-lane row,
 // both members of a row pair (then of a half-wave pair).
