@@ -22,6 +22,14 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes (scaled by a plain 1 GiB device copy); a
+# workload without a counter run reports null.
+MEASURED_TRAFFIC_BYTES = {
+    "decode_llama3_8b": (2184613 * 2.0 + 18592 * 1.0) * 1024,
+    "mixed_prefill_decode": (2222888 * 2.0 + 96627 * 1.0) * 1024,
+}
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -165,7 +173,7 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
-    roof.update({"traffic": None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
+    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.scale == 1.0 else None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
                  "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
                  "algorithmic_flops": counts["flops"], "tflops": tflops, "gbps": gbps})
 
