@@ -15,6 +15,9 @@ constexpr int kTiledMaxSeqs = 1024;        // schedule arrays live in LDS
 constexpr int kTiledMaxWgsPerCu = 4;        // persistent grid = compute units x this, at most
 
 constexpr uint64_t kWorkspaceTicketBytes = 1u << 20;  // head of the workspace, cleared by rpa_workspace_init
+// The last 16 words of the ticket region hold the prefill queue counters (8 queues, 1 exit count); the split
+// tickets, one word per (sequence, kv head), lie below them.
+constexpr uint32_t kQueueCounterIndex = (1u << 20) / 4 - 16;
 
 struct WorkspaceLayout {
   uint64_t counters_bytes;                   // split tickets at offset 0

@@ -32,6 +32,7 @@
 namespace rpa {
 
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
+constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
 
 // Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints and 8 ints of scratch, then the data region
 // shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
@@ -110,10 +111,9 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 
   // A batch without prefill tiles is pure streaming: it runs fastest with one workgroup per compute unit, so
   // the second half of the grid (dispatched after every unit has one workgroup) leaves at once.
-  const int grid_wgs = total_wg == 0 ? min(static_cast<int>(gridDim.x), a.decode_grid) : static_cast<int>(gridDim.x);
+  const int grid_all = static_cast<int>(gridDim.x);
+  const int grid_wgs = total_wg == 0 ? min(grid_all, a.decode_grid) : grid_all;
   if (static_cast<int>(blockIdx.x) >= grid_wgs) return;
-  const int n_workers = grid_wgs * kWgWaves;
-  const int worker = blockIdx.x * kWgWaves + wave;
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
   auto find = [&](const int* start, int x) {
@@ -125,22 +125,78 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     return __builtin_amdgcn_readfirstlane(lo);
   };
 
-  // Prefill tiles are compute-bound and the decode stream is bandwidth-bound: the two workgroups that share a
-  // compute unit take the two kinds of work in opposite order, so each unit has matrix work and memory traffic
-  // in flight at the same time instead of one after the other.
+  // Prefill tiles are compute-bound and the decode stream is bandwidth-bound, and one workgroup per compute unit
+  // already saturates the memory system.  In a mixed batch the second workgroup of every unit (the upper part of
+  // the grid) therefore takes the whole decode stream while the first one starts on the prefill tiles at once;
+  // prefill tiles are handed out from queues, so the streaming workgroups join in when the stream is done, and
+  // whichever kind of work is longer sets the time.  phase_mode 0..3 keep the static split for experiments.
+  const bool queued = total_wg > 0 && a.phase_mode == 4;
+  const bool split = queued && grid_all > a.decode_grid;
+  const bool do_stream = !split || static_cast<int>(blockIdx.x) >= a.decode_grid;
+  const int stream_wg0 = split ? a.decode_grid : 0;
+  const int stream_wgs = grid_wgs - stream_wg0;
+  const int n_workers = stream_wgs * kWgWaves;
+  // Workgroup b runs on XCD b % 8.  The XCDs do not stream from memory at the same rate (on MI355X the odd ones
+  // are about a tenth slower), so the wavefronts on even XCDs are numbered first and their region of the stream
+  // is made larger; with equal shares the slower XCDs would set the time.
+  const bool by_xcd = stream_wgs % 8 == 0 && stream_wg0 % 8 == 0;
+  int worker = (static_cast<int>(blockIdx.x) - stream_wg0) * kWgWaves + wave;
+  if (by_xcd) {
+    const int rel = static_cast<int>(blockIdx.x) - stream_wg0, xcd = rel & 7;
+    worker = (xcd & 1) * (n_workers / 2) + (((rel >> 3) * 4 + (xcd >> 1)) * kWgWaves + wave);
+  }
   const bool stream_first = total_wg > 0 && (a.phase_mode == 1 ? static_cast<int>(blockIdx.x) >= a.decode_grid
                                             : a.phase_mode == 2 ? (blockIdx.x & 1) != 0
-                                            : a.phase_mode == 3 ? ((blockIdx.x >> 3) & 1) != 0 : false);
+                                            : a.phase_mode == 3 ? ((blockIdx.x >> 3) & 1) != 0
+                                            : a.phase_mode == 4);
 #pragma unroll 1
   for (int phase = 0; phase < 2; ++phase) {
     if ((phase == 0) != stream_first) {
       // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)
       // adjacent in the item order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2:
-      // numbering the workgroups XCD by XCD makes the row tiles that share one K/V stream run at the same time on the
-      // same XCD, so all but the first of them read it from that L2.  Within a (sequence, kv head) the row tiles are
-      // rotated by the round in which the group starts: a workgroup then meets early (short) and late (long) causal
-      // tiles in turn instead of always the same one.
-      {
+      // row tiles that share one K/V stream should run at the same time on the same XCD, so that all but the first
+      // of them read it from that L2.
+      if (queued) {
+        // Eight queues, one per XCD: aligned runs of kQueueRun consecutive items go to the queues in turn.  A
+        // workgroup draws from the queue of its own XCD until that is empty, then from the others.  Within a
+        // (sequence, kv head) the late causal tiles (most keys) come first.  The last workgroup to find every
+        // queue empty clears the counters for the next launch.
+        uint32_t* qctr = a.counters + kQueueCounterIndex;
+        const int home = blockIdx.x & 7;
+        int probe = 0;
+        while (true) {
+          int w = -1;
+          while (probe < 8) {
+            const int x = (home + probe) & 7;
+            if (tid == 0)
+              scratch[0] = static_cast<int>(__hip_atomic_fetch_add(&qctr[x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+            __syncthreads();
+            const int t = __builtin_amdgcn_readfirstlane(scratch[0]);
+            __syncthreads();
+            const int cand = ((t / kQueueRun) * 8 + x) * kQueueRun + t % kQueueRun;
+            if (cand < total_wg) {
+              w = cand;
+              break;
+            }
+            ++probe;
+          }
+          if (w < 0) break;
+          const int s = find(wg_start, w);
+          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
+          const int local = w - __builtin_amdgcn_readfirstlane(wg_start[s]);
+          const int j = local / n_qt, member = local - j * n_qt;
+          prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, n_qt - 1 - member);
+        }
+        if (tid == 0) {
+          const uint32_t done = __hip_atomic_fetch_add(&qctr[8], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (done == static_cast<uint32_t>(grid_all) - 1)
+            for (int i = 0; i < 9; ++i) __hip_atomic_store(&qctr[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      } else {
+        // Static split: numbering the workgroups XCD by XCD keeps the row tiles of one K/V stream on one XCD; within
+        // a (sequence, kv head) the row tiles are rotated by the round in which the group starts, so a workgroup
+        // meets early (short) and late (long) causal tiles in turn instead of always the same one.
         const int n_xcd = gridDim.x % 8 == 0 ? 8 : 1;
         const int vwg = (blockIdx.x % n_xcd) * (gridDim.x / n_xcd) + blockIdx.x / n_xcd;
         for (int w = vwg; w < total_wg; w += gridDim.x) {
@@ -159,7 +215,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       // workgroup has finished reading them.
       __syncthreads();
 
-    } else {
+    } else if (do_stream) {
       // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
       for (int w = worker; w < total_items; w += n_workers) {
         const int s = find(item_start, w);
@@ -178,8 +234,15 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
       if (total_tiles > 0) {
         Shares sh;
-        sh.q = total_tiles / n_workers;
-        sh.rem = total_tiles - sh.q * n_workers;
+        {
+          // Equal shares when there are only a few tiles per wavefront (every non-empty share must stay in front
+          // of every empty one), weighted regions otherwise.
+          const int q = total_tiles / n_workers, rem = total_tiles - q * n_workers, half = n_workers / 2;
+          int first_tiles = half * q + min(half, rem);
+          if (by_xcd && q >= 4)
+            first_tiles = static_cast<int>(static_cast<long long>(total_tiles) * a.even_xcd_permille / 1000);
+          sh.set(total_tiles, n_workers, half, first_tiles);
+        }
         int x = sh.begin(worker);
         const int x_end = sh.begin(worker + 1);
         while (x < x_end) {
@@ -225,7 +288,7 @@ bool tiled_supported(const RpaParams& p) {
   if (p.head_dim != 128 && p.head_dim != 256) return false;
   if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
   if (p.max_num_seqs > kTiledMaxSeqs) return false;
-  if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kWorkspaceTicketBytes) return false;
+  if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kQueueCounterIndex * 4ull) return false;
   return true;
 }
 
@@ -269,7 +332,8 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.p = p;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
-  a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 1);
+  a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
+  a.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
   a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 1));
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);

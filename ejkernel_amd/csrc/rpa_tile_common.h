@@ -22,20 +22,40 @@ struct TileArgs {
   int page_shift;     // log2(page_size)
   int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
   int decode_grid;    // workgroups that take part when the batch has no prefill tiles
-  int phase_mode;     // which workgroups stream first in a mixed batch (0 none, 1 upper half of the grid, 2 odd, 3 odd octets)
-  uint32_t* counters; // [max_num_seqs * num_kv_heads], zero between launches
+  int even_xcd_permille;  // share of the decode stream given to the workgroups on even XCDs, in 1/1000
+  int phase_mode;     // mixed batches: 4 = upper half of the grid streams, prefill tiles from queues; 0..3 = static
+                      // split, streaming first on no / upper-half / odd / odd-octet workgroups
+  uint32_t* counters; // split tickets [max_num_seqs * num_kv_heads], then the queue counters; zero between launches
   float* partial_o;   // [2 * wavefronts of the grid][16][D]
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
 };
 
-// Split of the decode stream over the wavefronts of the grid: the first `rem` wavefronts take q + 1 tiles, the
-// others q, so shares differ by at most one tile and empty shares (q == 0) only occur at the end.
+// Split of the decode stream over the wavefronts of the grid, in two regions that are each cut evenly: workers
+// [0, h) share the first n_a tiles, workers [h, ...) the rest.  Within a region the first `rem` workers take
+// q + 1 tiles and the others q.  The caller chooses n_a so that every non-empty share lies in front of every
+// empty one: the merge of a split (sequence, kv head) counts on a part from each worker between its first and last.
 struct Shares {
-  int q, rem;
-  __device__ __forceinline__ int begin(int w) const { return w * q + min(w, rem); }
+  int h, n_a, q_a, rem_a, q_b, rem_b;
+  __device__ __forceinline__ void set(int total, int n_workers, int first_region_workers, int first_region_tiles) {
+    h = first_region_workers;
+    n_a = first_region_tiles;
+    const int nb = n_workers - h;
+    q_a = h > 0 ? n_a / h : 0;
+    rem_a = n_a - q_a * h;
+    q_b = nb > 0 ? (total - n_a) / nb : 0;
+    rem_b = (total - n_a) - q_b * nb;
+  }
+  __device__ __forceinline__ int begin(int w) const {
+    return w < h ? w * q_a + min(w, rem_a) : n_a + (w - h) * q_b + min(w - h, rem_b);
+  }
   __device__ __forceinline__ int owner(int x) const {
-    const int big = rem * (q + 1);
-    return x < big ? x / (q + 1) : rem + (x - big) / q;
+    if (x < n_a) {
+      const int big = rem_a * (q_a + 1);
+      return x < big ? x / (q_a + 1) : rem_a + (x - big) / q_a;
+    }
+    x -= n_a;
+    const int big = rem_b * (q_b + 1);
+    return h + (x < big ? x / (q_b + 1) : rem_b + (x - big) / q_b);
   }
 };
 
