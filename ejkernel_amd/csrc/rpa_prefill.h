@@ -139,14 +139,19 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
       reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
   const int l_row = lane / C::PR, l_slot = lane % C::PR;
+  // V blocks are laid out for the transposing operand read instead: [32-byte column unit][row of the block], so the
+  // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
+  const int v_row = (lane >> 1) % C::RB;
+  const uint32_t v_src = 16u * static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1));  // byte offset in the row
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
-  uint32_t pre_off[HB];  // per-lane byte offset of block n inside the group: row part + swizzled piece
+  uint32_t pre_off[HB];  // per-lane byte offset of K block n inside the group: row part + swizzled piece
 #pragma unroll
   for (int n = 0; n < HB; ++n) {
     const int t_local = GROUP * wave + C::RB * n + l_row;
     pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
   }
+  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + D * 2;  // V block 0; block n adds RB rows
   const bool group_in_page = p.page_size >= GROUP;
   auto fetch_tile = [&](int tile, int buf) {
     const int t_first = tile + GROUP * wave;
@@ -160,7 +165,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       for (int n = 0; n < HB; ++n) {
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n]),
                                          (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n] + D * 2),
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + v_pre_off + n * C::RB * stride_b),
                                          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
       }
       return;
@@ -177,8 +182,10 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
                                        (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off + D * 2),
-                                       (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+      const int v_tok = min(t_c + v_row, t_last);
+      __builtin_amdgcn_global_load_lds(
+          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_src + D * 2),
+          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
     }
   };
   // Wait until at most `ahead` later tiles of this wave's direct-to-LDS loads are outstanding (they complete in
@@ -200,13 +207,15 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 
   // Per-lane byte offsets of the MFMA operand reads inside a stage, fixed for the whole item: the row part of
   // a later sub-tile or half is a compile-time constant on top of them (the swizzle only uses row & 15).
-  int k_off[C::NKS], v_off[C::NS][4];
+  int k_off[C::NKS];
 #pragma unroll
   for (int ks = 0; ks < C::NKS; ++ks) k_off[ks] = i * C::ROWB + 16 * ((4 * ks + g) ^ i);
-#pragma unroll
-  for (int sN = 0; sN < C::NS; ++sN)
-#pragma unroll
-    for (int r = 0; r < 4; ++r) v_off[sN][r] = (4 * g + r) * C::ROWB + 16 * ((i + 16 * sN) ^ (4 * g + r));
+  // V^T operands come from the transposing 64-bit LDS read: in each group of 16 lanes, lanes 4e..4e+3 point at
+  // 16 consecutive elements of row e (8 bytes per lane) and lane x receives element x of rows 0..3.  Rows are the
+  // four keys 4g..4g+3 of a 16-key sub-tile, the elements one 32-byte column unit; everything else about the
+  // address (half, sub-tile, unit) is a compile-time offset.
+  const int v_key = 4 * g + (i >> 2);
+  const int v_rd = (v_key / C::RB) * 1024 + (v_key % C::RB) * 32 + 8 * (i & 3);
 
   if (range_hi > range_lo) {
     const int n_tiles = (range_hi - range_lo + C::TK - 1) / C::TK;
@@ -242,11 +251,14 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           load_k(0);
           load_k(1);
         }
-        u32x4_t vch[8];
+        s16x4_t vop[8][2];  // per column unit c: keys 4g..4g+3 of the two sub-tiles = one A operand
         auto load_v = [&](int sN) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e)
-            vch[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2)) * C::ROWB + v_off[sN][e & 3]);
+          for (int c = 0; c < 8; ++c)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+              vop[c][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
+                  vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + 8 * sN) * (C::RB * 32)));
         };
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -269,7 +281,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           __builtin_amdgcn_sched_group_barrier(0x100, 2 * C::NKS, 0);        // K operands first
           __builtin_amdgcn_sched_group_barrier(0x008, 2 * C::NKS * MRT, 0);  // QK MFMAs
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);  // V pieces of slice 0: they land during the softmax
+        __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);  // V operands of slice 0: they land during the softmax
         __builtin_amdgcn_sched_barrier(0);
         // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
         u32x4_t pw[MRT];
@@ -339,20 +351,12 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           if (sN > 0) load_v(sN);
 #pragma unroll
           for (int c = 0; c < 8; ++c) {
-            const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-            u32x4_t av;
-#pragma unroll
-            for (int hh = 0; hh < 4; ++hh) av[hh] = __builtin_amdgcn_perm(vch[2 * hh + 1][c >> 1], vch[2 * hh][c >> 1], sel);
+            typedef __attribute__((ext_vector_type(8))) short s16x8_t;
+            const s16x8_t av = __builtin_shufflevector(vop[c][0], vop[c][1], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
             for (int m = 0; m < MRT; ++m)
               o_acc[m][sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                   __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, pw[m]), o_acc[m][sN][c], 0, 0, 0);
-          }
-          if (sN > 0) __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
-#pragma unroll
-          for (int c = 0; c < 8; ++c) {
-            __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);    // four byte permutes build one A operand
-            __builtin_amdgcn_sched_group_barrier(0x008, MRT, 1);  // its MFMAs
           }
           __builtin_amdgcn_sched_barrier(0);
         }
@@ -377,15 +381,16 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       denom = num_scale * l_run + ssum;
     }
     const float inv = num_scale / fmaxf(denom, 1e-6f);
+    // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row
     bf16_t* orow = out + q_off[m];
 #pragma unroll
     for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        u32x4_t w;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[m][sN][2 * e][r] * inv, o_acc[m][sN][2 * e + 1][r] * inv);
-        *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+      for (int c = 0; c < 8; ++c) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(o_acc[m][sN][c][0] * inv, o_acc[m][sN][c][1] * inv);
+        w[1] = pack_bf16x2(o_acc[m][sN][c][2] * inv, o_acc[m][sN][c][3] * inv);
+        *reinterpret_cast<u32x2_t*>(orow + 128 * sN + 16 * c + 4 * g) = w;
       }
   }
 }
