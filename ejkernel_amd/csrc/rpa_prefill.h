@@ -42,6 +42,10 @@ struct PCfg {
   static constexpr int RB = kWave / PR;              // rows one wave-wide load instruction covers
   static constexpr int BLOCKS = TK / RB;             // load instructions per K (or V) tile: 16
   static constexpr int BPW = 2 * BLOCKS / kWgWaves;  // load instructions per wavefront and step
+  // V^T operands come from the transposing LDS read (V tile stored by column units) or, where the tile is LDS-bound
+  // (16 rows per wavefront at head_dim 256), from 16-byte reads of a row-major tile plus byte permutes: the
+  // transposing read moves 8 bytes per lane and takes more LDS time for the same operands.
+  static constexpr bool TRV = D == 128;
 };
 
 constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point by this much before O is rescaled
@@ -141,7 +145,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const int l_row = lane / C::PR, l_slot = lane % C::PR;
   // V blocks are laid out for the transposing operand read instead: [32-byte column unit][row of the block], so the
   // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
-  const int v_row = (lane >> 1) % C::RB;
+  // (Without the transposing read the V tile is laid out like the K tile.)
+  const int v_row = C::TRV ? (lane >> 1) % C::RB : l_row;
   const uint32_t v_src = 16u * static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1));  // byte offset in the row
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
@@ -152,6 +157,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
   }
   const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + D * 2;  // V block 0; block n adds RB rows
+  auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
+    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + D * 2;
+  };
   const bool group_in_page = p.page_size >= GROUP;
   auto fetch_tile = [&](int tile, int buf) {
     const int t_first = tile + GROUP * wave;
@@ -165,7 +173,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       for (int n = 0; n < HB; ++n) {
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n]),
                                          (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + v_pre_off + n * C::RB * stride_b),
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + v_src_off(n)),
                                          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
       }
       return;
@@ -183,8 +191,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
                                        (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
       const int v_tok = min(t_c + v_row, t_last);
+      const uint32_t v_piece = C::TRV ? v_src : 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
       __builtin_amdgcn_global_load_lds(
-          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_src + D * 2),
+          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + D * 2),
           (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
     }
   };
@@ -216,75 +225,93 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // address (half, sub-tile, unit) is a compile-time offset.
   const int v_key = 4 * g + (i >> 2);
   const int v_rd = (v_key / C::RB) * 1024 + (v_key % C::RB) * 32 + 8 * (i & 3);
+  // Row-major V tile: lane (i, g) reads piece i (+ 16 per slice) of rows 4g..4g+3 and transposes in registers.
+  int v_off[C::NS][4];
+#pragma unroll
+  for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) v_off[sN][r] = (4 * g + r) * C::ROWB + 16 * ((i + 16 * sN) ^ (4 * g + r));
 
   if (range_hi > range_lo) {
     const int n_tiles = (range_hi - range_lo + C::TK - 1) / C::TK;
     __syncthreads();  // every wavefront has left the previous item's tiles
     for (int t = 0; t < min(C::NSTG - 1, n_tiles); ++t) fetch_tile(range_lo + t * C::TK, t);
+    wait_fetch(min(n_tiles - 1, C::NSTG - 2));
+    __syncthreads();  // publishes tile 0
+    if (C::NSTG - 1 < n_tiles) fetch_tile(range_lo + (C::NSTG - 1) * C::TK, C::NSTG - 1);
+    // The K operands of a half are requested one half ahead, right before the P V MFMAs of the half in progress,
+    // so their LDS latency (and the barrier that publishes the next tile) hides behind matrix work.  At head_dim
+    // 256 only the first sub-tile's operands are held that long, for lack of registers; the second sub-tile's are
+    // requested when the half starts and land while the first sub-tile's MFMAs run.
+    constexpr int KAHEAD = D == 128 ? 2 : 1;
+    u32x4_t kop[2][C::NKS];
+    auto load_k_sub = [&](const char* kt_n, int h_n, int u) {
+#pragma unroll
+      for (int ks = 0; ks < C::NKS; ++ks)
+        kop[u][ks] = *reinterpret_cast<const u32x4_t*>(kt_n + (32 * h_n + 16 * u) * C::ROWB + k_off[ks]);
+    };
+    auto load_k = [&](const char* kt_n, int h_n) {
+#pragma unroll
+      for (int u = 0; u < KAHEAD; ++u) load_k_sub(kt_n, h_n, u);
+    };
+    load_k(lds, 0);
     for (int kt_i = 0; kt_i < n_tiles; ++kt_i) {
       const int tile = range_lo + kt_i * C::TK;
       const int buf = kt_i % C::NSTG;
-      wait_fetch(min(n_tiles - 1 - kt_i, C::NSTG - 2));
-      // publishes tile kt_i, and every wavefront has finished the previous tile, whose stage is refilled next
-      __syncthreads();
-      if (kt_i + C::NSTG - 1 < n_tiles) fetch_tile(tile + (C::NSTG - 1) * C::TK, (kt_i + C::NSTG - 1) % C::NSTG);
       const char* kt = lds + buf * 2 * C::TILE_B;
       const char* vt = kt + C::TILE_B;
 #pragma unroll
       for (int h = 0; h < C::NH; ++h) {
         const int a0 = tile + 32 * h;  // first key of this half
-        const bool w_skip = !w_any || a0 >= range_hi || a0 > w_pos_hi || (W > 0 && a0 + 31 <= w_pos_lo - W);
-        if (w_skip) continue;
-        // S^T = K Q^T for the two 16-key sub-tiles.  The eight K operands are requested first and the V pieces of
-        // the first slice while the QK MFMAs run, so LDS latency is paid once per half and V is in registers by
-        // the time the softmax is done.  The group barriers pin that order (the scheduler would otherwise sink
-        // every LDS read next to its first use).
-        f32x4_t s_acc[MRT][2];
-        constexpr int KU = D == 128 ? 2 : 1;  // sub-tiles whose K operands are held at once (register budget)
-        u32x4_t kop[KU][C::NKS];
-        auto load_k = [&](int u) {
-#pragma unroll
-          for (int ks = 0; ks < C::NKS; ++ks)
-            kop[u % KU][ks] = *reinterpret_cast<const u32x4_t*>(kt + (32 * h + 16 * u) * C::ROWB + k_off[ks]);
-        };
-        if constexpr (KU == 2) {
-          load_k(0);
-          load_k(1);
-        }
-        s16x4_t vop[8][2];  // per column unit c: keys 4g..4g+3 of the two sub-tiles = one A operand
+        // halves that lie entirely in this wavefront's causal future or left of its window are skipped
+        const bool active = w_any && a0 < range_hi && a0 <= w_pos_hi && !(W > 0 && a0 + 31 <= w_pos_lo - W);
+        // V of one slice: with the transposing read, per column unit c the keys 4g..4g+3 of the two sub-tiles (one
+        // A operand); otherwise eight 16-byte pieces (rows 4g..4g+3 of the two sub-tiles, piece i)
+        u32x4_t vraw[8];
         auto load_v = [&](int sN) {
+          if constexpr (C::TRV) {
 #pragma unroll
-          for (int c = 0; c < 8; ++c)
+            for (int c = 0; c < 8; ++c)
 #pragma unroll
-            for (int u = 0; u < 2; ++u)
-              vop[c][u] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
-                  vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + 8 * sN) * (C::RB * 32)));
+              for (int u = 0; u < 2; ++u) {
+                const s16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
+                    vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + 8 * sN) * (C::RB * 32)));
+                const u32x2_t t2 = __builtin_bit_cast(u32x2_t, t);
+                vraw[c][2 * u] = t2[0];
+                vraw[c][2 * u + 1] = t2[1];
+              }
+          } else {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              vraw[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2)) * C::ROWB + v_off[sN][e & 3]);
+          }
         };
+        constexpr int V_READS = C::TRV ? 16 : 8;
+        u32x4_t pw[MRT];
+        if (active) {
+        // S^T = K Q^T for the two 16-key sub-tiles, then the V operands of the first slice are requested: they
+        // land during the softmax.  The group barriers pin that order.
+        f32x4_t s_acc[MRT][2];
+        if constexpr (KAHEAD == 1) {
+          load_k_sub(kt, h, 1);
+          __builtin_amdgcn_sched_group_barrier(0x100, C::NKS, 0);
+        }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
-          if constexpr (KU == 1) {
-            load_k(u);
-            __builtin_amdgcn_sched_group_barrier(0x100, C::NKS, 0);
-          }
 #pragma unroll
           for (int m = 0; m < MRT; ++m) s_acc[m][u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int ks = 0; ks < C::NKS; ++ks)
 #pragma unroll
             for (int m = 0; m < MRT; ++m)
-              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[u % KU][ks]),
-                                                                    qreg[m][ks], s_acc[m][u], 0, 0, 0);
-          if constexpr (KU == 1) __builtin_amdgcn_sched_group_barrier(0x008, C::NKS * MRT, 0);
+              s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[u][ks]), qreg[m][ks],
+                                                                    s_acc[m][u], 0, 0, 0);
         }
         load_v(0);
-        if constexpr (KU == 2) {
-          __builtin_amdgcn_sched_group_barrier(0x100, 2 * C::NKS, 0);        // K operands first
-          __builtin_amdgcn_sched_group_barrier(0x008, 2 * C::NKS * MRT, 0);  // QK MFMAs
-        }
-        __builtin_amdgcn_sched_group_barrier(0x100, 16, 0);  // V operands of slice 0: they land during the softmax
+        __builtin_amdgcn_sched_group_barrier(0x008, 2 * C::NKS * MRT, 0);  // QK MFMAs
+        __builtin_amdgcn_sched_group_barrier(0x100, V_READS, 0);           // V of slice 0
         __builtin_amdgcn_sched_barrier(0);
         // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
-        u32x4_t pw[MRT];
 #pragma unroll
         for (int m = 0; m < MRT; ++m) {
           float sv[2][4];
@@ -345,20 +372,51 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           l_acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ones),
                                                             __builtin_bit_cast(bf16x8_t, pw[m]), l_acc[m], 0, 0, 0);
         }
-        // O^T += V^T P^T: the eight fetched pieces of a slice give eight A operands, each used by every row tile
+        }  // active
+        __builtin_amdgcn_sched_barrier(0);
+        // ---- K operands of the next half.  At the end of a tile the next one is published first: this wavefront's
+        // own part of it has landed (wait_fetch), and after the barrier so has everybody's; by then every wavefront
+        // also holds its last V operands of the current tile in registers, so that stage can be refilled.
+        if (h + 1 < C::NH) {
+          load_k(kt, h + 1);
+        } else if (kt_i + 1 < n_tiles) {
+          wait_fetch(min(n_tiles - 2 - kt_i, C::NSTG - 2));
+          __syncthreads();
+          if (kt_i + C::NSTG < n_tiles) fetch_tile(tile + C::NSTG * C::TK, buf);
+          load_k(lds + ((kt_i + 1) % C::NSTG) * 2 * C::TILE_B, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        // O^T += V^T P^T: one A operand per MFMA column block c, used by every row tile
+        if (active) {
 #pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN) {
-          if (sN > 0) load_v(sN);
+          for (int sN = 0; sN < C::NS; ++sN) {
+            if (sN > 0) load_v(sN);
 #pragma unroll
-          for (int c = 0; c < 8; ++c) {
-            typedef __attribute__((ext_vector_type(8))) short s16x8_t;
-            const s16x8_t av = __builtin_shufflevector(vop[c][0], vop[c][1], 0, 1, 2, 3, 4, 5, 6, 7);
+            for (int c = 0; c < 8; ++c) {
+              u32x4_t av;
+              if constexpr (C::TRV) {
+                av = vraw[c];
+              } else {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
 #pragma unroll
-            for (int m = 0; m < MRT; ++m)
-              o_acc[m][sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                  __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, pw[m]), o_acc[m][sN][c], 0, 0, 0);
+                for (int hh = 0; hh < 4; ++hh)
+                  av[hh] = __builtin_amdgcn_perm(vraw[2 * hh + 1][c >> 1], vraw[2 * hh][c >> 1], sel);
+              }
+#pragma unroll
+              for (int m = 0; m < MRT; ++m)
+                o_acc[m][sN][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    __builtin_bit_cast(bf16x8_t, av), __builtin_bit_cast(bf16x8_t, pw[m]), o_acc[m][sN][c], 0, 0, 0);
+            }
+            if constexpr (!C::TRV) {
+              if (sN > 0) __builtin_amdgcn_sched_group_barrier(0x100, 8, 1);
+#pragma unroll
+              for (int c = 0; c < 8; ++c) {
+                __builtin_amdgcn_sched_group_barrier(0x002, 4, 1);    // four byte permutes build one A operand
+                __builtin_amdgcn_sched_group_barrier(0x008, MRT, 1);  // its MFMAs
+              }
+            }
+            __builtin_amdgcn_sched_barrier(0);
           }
-          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -381,17 +439,30 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       denom = num_scale * l_run + ssum;
     }
     const float inv = num_scale / fmaxf(denom, 1e-6f);
-    // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row
     bf16_t* orow = out + q_off[m];
+    if constexpr (C::TRV) {
+      // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row
 #pragma unroll
-    for (int sN = 0; sN < C::NS; ++sN)
+      for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-      for (int c = 0; c < 8; ++c) {
-        u32x2_t w;
-        w[0] = pack_bf16x2(o_acc[m][sN][c][0] * inv, o_acc[m][sN][c][1] * inv);
-        w[1] = pack_bf16x2(o_acc[m][sN][c][2] * inv, o_acc[m][sN][c][3] * inv);
-        *reinterpret_cast<u32x2_t*>(orow + 128 * sN + 16 * c + 4 * g) = w;
-      }
+        for (int c = 0; c < 8; ++c) {
+          u32x2_t w;
+          w[0] = pack_bf16x2(o_acc[m][sN][c][0] * inv, o_acc[m][sN][c][1] * inv);
+          w[1] = pack_bf16x2(o_acc[m][sN][c][2] * inv, o_acc[m][sN][c][3] * inv);
+          *reinterpret_cast<u32x2_t*>(orow + 128 * sN + 16 * c + 4 * g) = w;
+        }
+    } else {
+      // MFMA c of a slice holds head_dim elements 8 (4 g + r) + c of this lane's row
+#pragma unroll
+      for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          u32x4_t w;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[m][sN][2 * e][r] * inv, o_acc[m][sN][2 * e + 1][r] * inv);
+          *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+        }
+    }
   }
 }
 
