@@ -25,8 +25,8 @@ if ROOT not in sys.path:
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes (scaled by a plain 1 GiB device copy); a
 # workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_llama3_8b": (2184613 * 2.0 + 18592 * 1.0) * 1024,
-    "mixed_prefill_decode": (2222888 * 2.0 + 96627 * 1.0) * 1024,
+    "decode_llama3_8b": (2185792 * 2.0 + 21519 * 1.0) * 1024,
+    "mixed_prefill_decode": (2162317 * 2.0 + 90297 * 1.0) * 1024,
 }
 
 
