@@ -13,10 +13,11 @@ from pathlib import Path
 # RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
-RPA_ABI_VERSION = 1
+RPA_ABI_VERSION = 2
 RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
+RPA_FLAG_FP32_LOGITS = 2
 
 EXPORTED_SYMBOLS = (
     "rpa_abi_version",
@@ -24,6 +25,7 @@ EXPORTED_SYMBOLS = (
     "rpa_workspace_bytes",
     "rpa_workspace_init",
     "rpa_fwd_launch",
+    "rpa_v3_launch",
 )
 
 
@@ -60,6 +62,19 @@ class RpaParams(ctypes.Structure):
         ("num_warps", ctypes.c_int32),
         ("num_stages", ctypes.c_int32),
         ("flags", ctypes.c_uint32),
+        ("q_scale", ctypes.c_float),
+        ("k_scale", ctypes.c_float),
+        ("v_scale", ctypes.c_float),
+    ]
+
+
+class RpaV3Params(ctypes.Structure):
+    """Field-for-field image of ``struct RpaV3Params``."""
+
+    _fields_ = [
+        ("attn", RpaParams),
+        ("new_keys", ctypes.c_void_p),
+        ("new_values", ctypes.c_void_p),
     ]
 
 
@@ -97,6 +112,8 @@ def load() -> ctypes.CDLL:
     lib.rpa_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     lib.rpa_fwd_launch.restype = ctypes.c_int
     lib.rpa_fwd_launch.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
+    lib.rpa_v3_launch.restype = ctypes.c_int
+    lib.rpa_v3_launch.argtypes = [ctypes.POINTER(RpaV3Params), ctypes.c_void_p]
     if lib.rpa_abi_version() != RPA_ABI_VERSION:
         raise NativeLibraryError(
             f"{LIB_PATH} has ABI version {lib.rpa_abi_version()}, this package expects {RPA_ABI_VERSION}: rebuild it"

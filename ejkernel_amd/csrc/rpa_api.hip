@@ -35,6 +35,8 @@ static int validate(const RpaParams& p, bool need_pointers) {
     return fail(RPA_ERR_INVALID_ARGUMENT, "unknown compute mode %d", p.compute);
   if (!(p.softmax_scale == p.softmax_scale)) return fail(RPA_ERR_INVALID_ARGUMENT, "softmax_scale is NaN");
   if (!(p.logits_soft_cap == p.logits_soft_cap)) return fail(RPA_ERR_INVALID_ARGUMENT, "logits_soft_cap is NaN");
+  if (!(p.q_scale >= 0.f) || !(p.k_scale >= 0.f) || !(p.v_scale >= 0.f))
+    return fail(RPA_ERR_INVALID_ARGUMENT, "q_scale / k_scale / v_scale must be positive (0 = absent)");
   if (need_pointers) {
     if (!p.queries || !p.kv_pages || !p.context_lens || !p.block_tables || !p.query_start_loc || !p.num_seqs || !p.out)
       return fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaParams");
@@ -109,6 +111,21 @@ int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {
   if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
   return RPA_OK;
+}
+
+int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
+  if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
+  RpaV3Params v = *params;
+  v.attn.flags |= RPA_FLAG_FP32_LOGITS;
+  int rc = rpa::validate(v.attn, true);
+  if (rc != RPA_OK) return rc;
+  if (!v.new_keys || !v.new_values) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null new_keys / new_values");
+  if (v.attn.num_sinks != 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "ragged_page_attention_v3 has no sinks");
+  rc = rpa::launch_kv_cache_update(v, static_cast<hipStream_t>(hip_stream));
+  if (rc == RPA_ERR_UNSUPPORTED)
+    return rpa::fail(rc, "head_dim=%d rows are not a multiple of 16 bytes", v.attn.head_dim);
+  if (rc != RPA_OK) return rpa::fail(rc, "cache update launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return rpa_fwd_launch(&v.attn, hip_stream);
 }
 
 }  // extern "C"

@@ -53,13 +53,14 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float lo = __uint_as_float(raw[e] << 16) * scale, hi = __uint_as_float(raw[e] & 0xffff0000u) * scale;
-        sc[e] = pack_bf16x2(lo, hi);
+        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
+                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
       }
       qreg[ks] = __builtin_bit_cast(bf16x8_t, sc);
     }
   }
 
+  const float post_scale = logit_scale(p);
   f32x4_t o_acc[C::NS][8];
 #pragma unroll
   for (int sN = 0; sN < C::NS; ++sN)
@@ -160,7 +161,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r];
+      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r] * post_scale;
     if (cap != 0.f) {
 #pragma unroll
       for (int u = 0; u < NT; ++u)
@@ -333,7 +334,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     num_scale = m_run == -INFINITY ? 0.f : expf(m_run - mt);
     denom = num_scale * l_run + ssum;
   }
-  const float inv = num_scale / fmaxf(denom, 1e-6f);
+  const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
   bf16_t* orow = out + q_row_off;
 #pragma unroll
   for (int sN = 0; sN < C::NS; ++sN)

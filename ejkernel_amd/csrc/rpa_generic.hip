@@ -42,7 +42,13 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
   const int lo = p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0;
 
   const bool t_is_bf16 = sizeof(T) == 2;
+  // RPA_FLAG_FP32_LOGITS: q enters the dot product unscaled (divided by q_scale and rounded to the storage type, if
+  // given), the fp32 logit is multiplied by softmax_scale * k_scale * q_scale, probabilities are rounded to the
+  // storage type before P V (ragged_page_attention_v3, _kernel.py:221-262).
+  const bool v3 = (p.flags & RPA_FLAG_FP32_LOGITS) != 0;
   const float scale = t_is_bf16 ? round_bf16(p.softmax_scale) : p.softmax_scale;
+  const float post = p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f);
+  const float o_scale = p.v_scale > 0.f ? p.v_scale : 1.f;
   const float cap = p.logits_soft_cap;
   const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
@@ -51,8 +57,16 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
     const int h = j * G + g;
     __syncthreads();
     for (int d = lane; d < D; d += kWave) {
-      float v = Elem<T>::load(q + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d) * scale;
-      if (t_is_bf16 || kBf16Compute) v = round_bf16(v);
+      float v = Elem<T>::load(q + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d);
+      if (v3) {
+        if (p.q_scale > 0.f) {
+          v = v / p.q_scale;
+          if (t_is_bf16) v = round_bf16(v);
+        }
+      } else {
+        v *= scale;
+        if (t_is_bf16 || kBf16Compute) v = round_bf16(v);
+      }
       q_lds[d] = v;
     }
     __syncthreads();
@@ -76,9 +90,10 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
         if (kBf16Compute && !t_is_bf16) kvv = round_bf16(kvv);
         sc = fmaf(q_lds[d], kvv, sc);
       }
-      if (kBf16Compute) sc = round_bf16(sc);
+      if (v3) sc *= post;
+      else if (kBf16Compute) sc = round_bf16(sc);
       if (cap != 0.f) {
-        if (kBf16Compute) {
+        if (kBf16Compute && !v3) {
           sc = round_bf16(round_bf16(tanhf(round_bf16(sc / cap))) * cap);
         } else {
           sc = cap * tanhf(sc / cap);
@@ -87,7 +102,10 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
       if (!valid) sc = -INFINITY;
       const float m_new = fmaxf(m, wave_max(sc));
       float pr;
-      if (kBf16Compute) {
+      if (v3) {
+        pr = valid ? expf(sc - m_new) : 0.f;
+        if (t_is_bf16) pr = round_bf16(pr);
+      } else if (kBf16Compute) {
         pr = valid ? round_bf16(expf(round_bf16(sc - m_new))) : 0.f;
       } else {
         pr = valid ? expf(sc - m_new) : 0.f;
@@ -130,7 +148,7 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
 #pragma unroll
     for (int e = 0; e < kMaxElemsPerLane; ++e) {
       const int d = lane + e * kWave;
-      if (d < D) Elem<T>::store(out + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d, num_scale * acc[e] / denom);
+      if (d < D) Elem<T>::store(out + (static_cast<size_t>(row) * p.num_q_heads + h) * D + d, num_scale * o_scale * acc[e] / denom);
     }
   }
 }

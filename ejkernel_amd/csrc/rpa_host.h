@@ -9,6 +9,8 @@ namespace rpa {
 
 // Each returns RPA_OK or a negative RPA_ERR_* code; all of them only enqueue on `stream`.
 int launch_generic(const RpaParams& p, hipStream_t stream);
+// Writes the new tokens' K/V rows into the paged cache (ragged_page_attention_v3, _kernel.py:207-218).
+int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream);
 
 // Tiled MFMA path (bf16, head_dim 128 or 256, page_size a multiple of 4).
 constexpr int kTiledMaxSeqs = 1024;        // schedule arrays live in LDS

@@ -1,0 +1,46 @@
+// Cache update of ragged_page_attention_v3: token t of sequence s (t in [q_start, q_start + q_len)) is the key /
+// value at position kv_len - q_len + (t - q_start) of that sequence, and its rows go to
+// cache[block_tables[s, pos / page], pos % page, 2j | 2j + 1, :] for every kv head j
+// (ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:44-57 merge_kv, :207-218 update).
+// One workgroup per token; the 16-byte pieces of its K and V rows are spread over the threads.  Pure copy: the
+// element type only sets the row length in bytes.
+#include "rpa_device.h"
+#include "rpa_host.h"
+
+namespace rpa {
+
+__global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const char* __restrict__ new_k,
+                                                              const char* __restrict__ new_v, int row_bytes) {
+  const int t = blockIdx.x;
+  int nseq = p.num_seqs[0];
+  nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
+  if (t >= p.query_start_loc[nseq]) return;
+  const int s = find_seq(p.query_start_loc, nseq, t);
+  const int q0 = p.query_start_loc[s], q_len = p.query_start_loc[s + 1] - q0;
+  const int kv_len = p.context_lens[s];
+  const int pos = kv_len - q_len + (t - q0);
+  if (pos < 0 || pos >= kv_len || pos >= p.pages_per_seq * p.page_size) return;
+  int page = p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + pos / p.page_size];
+  page = page < 0 ? 0 : (page >= p.num_pages ? p.num_pages - 1 : page);
+  const size_t tok = static_cast<size_t>(page) * p.page_size + pos % p.page_size;
+  char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * 2 * p.num_kv_heads * row_bytes;
+  const size_t src_off = static_cast<size_t>(t) * p.num_kv_heads * row_bytes;
+  const int pieces_per_row = row_bytes / 16, n = 2 * p.num_kv_heads * pieces_per_row;
+  for (int k = threadIdx.x; k < n; k += blockDim.x) {
+    const int row = k / pieces_per_row, piece = k - row * pieces_per_row;  // row = combined head 2j (K) or 2j + 1 (V)
+    const char* src = ((row & 1) ? new_v : new_k) + src_off + static_cast<size_t>(row >> 1) * row_bytes + 16 * piece;
+    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(row) * row_bytes + 16 * piece) = *reinterpret_cast<const uint4*>(src);
+  }
+}
+
+int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream) {
+  const RpaParams& p = v.attn;
+  if (p.total_tokens == 0) return RPA_OK;
+  const int row_bytes = p.head_dim * (p.dtype == RPA_DTYPE_BF16 ? 2 : 4);
+  if (row_bytes % 16 != 0) return RPA_ERR_UNSUPPORTED;
+  hipLaunchKernelGGL(kv_cache_update_kernel, dim3(p.total_tokens), dim3(256), 0, stream, p,
+                     static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes);
+  return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
+}
+
+}  // namespace rpa

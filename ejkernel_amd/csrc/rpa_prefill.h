@@ -84,6 +84,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   bool t_any[MRT];
   bf16x8_t qreg[MRT][C::NKS];
   const float scale = rbf(p.softmax_scale);
+  const float post_scale = logit_scale(p);
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
     const int R = w_row_lo + 16 * m + i;
@@ -103,7 +104,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
-        sc[e] = pack_bf16x2(__uint_as_float(raw[e] << 16) * scale, __uint_as_float(raw[e] & 0xffff0000u) * scale);
+        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
+                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
       qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
     }
   }
@@ -318,7 +320,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
           for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sv[u][r] = s_acc[m][u][r];
+            for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? s_acc[m][u][r] : s_acc[m][u][r] * post_scale;
           if (cap != 0.f) {
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -438,7 +440,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       num_scale = m_run[m] == -INFINITY ? 0.f : expf(m_run[m] - mt);
       denom = num_scale * l_run + ssum;
     }
-    const float inv = num_scale / fmaxf(denom, 1e-6f);
+    const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
     bf16_t* orow = out + q_off[m];
     if constexpr (C::TRV) {
       // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row

@@ -340,7 +340,7 @@ int launch_tiled(const RpaParams& p, hipStream_t stream) {
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
-  const bool mimic = env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
+  const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
   if (p.head_dim == 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);

@@ -30,6 +30,20 @@ struct TileArgs {
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
 };
 
+// How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the
+// bf16 scale and rounded to bf16 before the contraction.  Arithmetic of ragged_page_attention_v3 (!kMimic): q
+// enters as it is (divided by q_scale and rounded, if given) and the fp32 logits are multiplied by
+// softmax_scale * k_scale * q_scale.
+template <bool kMimic>
+__device__ __forceinline__ float q_operand(float x, const RpaParams& p, float mimic_scale) {
+  if (kMimic) return x * mimic_scale;
+  return p.q_scale > 0.f ? x / p.q_scale : x;
+}
+__device__ __forceinline__ float logit_scale(const RpaParams& p) {
+  return p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f);
+}
+__device__ __forceinline__ float out_scale(const RpaParams& p) { return p.v_scale > 0.f ? p.v_scale : 1.f; }
+
 // Split of the decode stream over the wavefronts of the grid, in two regions that are each cut evenly: workers
 // [0, h) share the first n_a tiles, workers [h, ...) the rest.  Within a region the first `rem` workers take
 // q + 1 tiles and the others q.  The caller chooses n_a so that every non-empty share lies in front of every

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define RPA_ABI_VERSION 1
+#define RPA_ABI_VERSION 2
 
 /* element type of queries / kv_pages / out */
 #define RPA_DTYPE_BF16 0
@@ -43,6 +43,9 @@ extern "C" {
 
 /* rpa_fwd_launch flags */
 #define RPA_FLAG_FORCE_GENERIC 1u /* route every sequence through the scalar fp32 kernel */
+#define RPA_FLAG_FP32_LOGITS 2u   /* the arithmetic of ragged_page_attention_v3 (_kernel.py:228-262): q enters the   */
+                                  /* contraction unscaled, logits stay fp32 and are scaled after it, probabilities  */
+                                  /* are rounded to the cache dtype before P V                                      */
 
 typedef struct RpaParams {
   /* ---- device buffers (argument names follow ragged_page_attention.py:540-547) ---- */
@@ -83,7 +86,27 @@ typedef struct RpaParams {
   int32_t num_warps;              /* wavefronts per workgroup                         */
   int32_t num_stages;             /* reserved                                         */
   uint32_t flags;                 /* RPA_FLAG_*                                       */
+
+  /* ---- quantisation scales of ragged_page_attention_v3 (_kernel.py:221-226,232-235,258-259); 0 = absent.   */
+  /*      q is divided by q_scale before the contraction, logits are multiplied by k_scale * q_scale, the      */
+  /*      output by v_scale.  Only v_scale is honoured without RPA_FLAG_FP32_LOGITS.                           */
+  float q_scale;
+  float k_scale;
+  float v_scale;
 } RpaParams;
+
+/*
+ * ragged_page_attention_v3: write the new tokens' K/V rows into the paged cache, then attend over it.
+ * Replaces ejkernel/kernels/_xla/ragged_page_attention_v3/_interface.py:25-96 (program: _kernel.py:127-318).
+ * The cache has the layout of kv_pages above, which is what merge_kv (_kernel.py:44-57) produces when head_dim
+ * is a multiple of 128: [num_pages, page_size, 2*num_kv_heads / packing, packing, head_dim].
+ */
+typedef struct RpaV3Params {
+  RpaParams attn;         /* kv_pages = the cache, updated in place; context_lens = kv_lens (they include the new  */
+                          /* tokens); num_seqs = &distribution[2]; RPA_FLAG_FP32_LOGITS is implied                 */
+  const void* new_keys;   /* [total_tokens, num_kv_heads, head_dim], dtype of the cache                            */
+  const void* new_values; /* [total_tokens, num_kv_heads, head_dim]                                                */
+} RpaV3Params;
 
 /* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */
 uint64_t rpa_workspace_bytes(const RpaParams* dims);
@@ -94,6 +117,11 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
 
 /* Enqueues the forward pass on `hip_stream` (a hipStream_t; NULL = default stream). */
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
+
+/* Enqueues the cache update (token t of sequence s goes to position kv_len - q_len + (t - q_start) of s) and then
+ * the forward pass, both on `hip_stream`.  Sequences whose block tables share a page that one of them writes see
+ * the written rows (the reference updates and attends sequence by sequence). */
+int rpa_v3_launch(const RpaV3Params* params, void* hip_stream);
 
 /* Message for the calling thread's most recent failure ("" if none). */
 const char* rpa_last_error(void);

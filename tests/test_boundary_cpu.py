@@ -21,7 +21,7 @@ ROOT = Path(__file__).resolve().parent.parent
 def _declared_functions():
     text = (ROOT / "include" / "rpa_mi355x.h").read_text()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(rpa_[a-z_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(rpa_[a-z0-9_]+)\s*\(", text)))
 
 
 def test_library_loads_and_exports_every_declared_symbol():
