@@ -377,16 +377,22 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         }  // active
         __builtin_amdgcn_sched_barrier(0);
         // ---- K operands of the next half.  At the end of a tile the next one is published first: this wavefront's
-        // own part of it has landed (wait_fetch), and after the barrier so has everybody's; by then every wavefront
-        // also holds its last V operands of the current tile in registers, so that stage can be refilled.
-        if (h + 1 < C::NH) {
-          load_k(kt, h + 1);
-        } else if (kt_i + 1 < n_tiles) {
-          wait_fetch(min(n_tiles - 2 - kt_i, C::NSTG - 2));
-          __syncthreads();
-          if (kt_i + C::NSTG < n_tiles) fetch_tile(tile + C::NSTG * C::TK, buf);
-          load_k(lds + ((kt_i + 1) % C::NSTG) * 2 * C::TILE_B, 0);
-        }
+        // own part of it has landed (wait_fetch), and after the barrier so has everybody's; the stage of the current
+        // tile is refilled right away, so every wavefront must hold its last V operands of that tile in registers
+        // by then.  With one slice (head_dim 128) that is the case before the P V MFMAs, which then hide the LDS
+        // latency and the barrier; with two slices the second slice's V operands are only read during P V, and the
+        // step comes after it.
+        auto next_k = [&]() {
+          if (h + 1 < C::NH) {
+            load_k(kt, h + 1);
+          } else if (kt_i + 1 < n_tiles) {
+            wait_fetch(min(n_tiles - 2 - kt_i, C::NSTG - 2));
+            __syncthreads();
+            if (kt_i + C::NSTG < n_tiles) fetch_tile(tile + C::NSTG * C::TK, buf);
+            load_k(lds + ((kt_i + 1) % C::NSTG) * 2 * C::TILE_B, 0);
+          }
+        };
+        if constexpr (C::NS == 1) next_k();
         __builtin_amdgcn_sched_barrier(0);
         // O^T += V^T P^T: one A operand per MFMA column block c, used by every row tile
         if (active) {
@@ -420,6 +426,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
             __builtin_amdgcn_sched_barrier(0);
           }
         }
+        if constexpr (C::NS > 1) next_k();
       }
     }
   }

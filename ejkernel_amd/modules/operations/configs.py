@@ -1,4 +1,4 @@
-"""Configuration dataclasses of the ragged paged attention op.
+"""Configuration dataclasses of the ragged paged attention ops.
 
 Field names, order and defaults are those of
 ``ejkernel/modules/operations/configs.py:29-34`` (``BaseOperationConfig``) and
@@ -45,3 +45,22 @@ class RaggedPageAttentionConfig(BaseOperationConfig):
             raise ValueError(f"num_kv_pages_per_block={self.num_kv_pages_per_block} must be positive.")
         if self.num_queries_per_block is not None and self.num_queries_per_block <= 0:
             raise ValueError(f"num_queries_per_block={self.num_queries_per_block} must be positive.")
+
+
+@dataclass
+class RaggedPageAttentionv3Config(BaseOperationConfig):
+    """Configuration for ragged paged attention v3 (ejkernel/modules/operations/configs.py:262-278)."""
+
+    chunk_prefill_size: int | None = None
+    num_kv_pages_per_block: int | None = None
+    num_queries_per_block: int | None = None
+    num_warps: int = 4
+    num_stages: int = 1
+
+    def validate(self) -> None:
+        if self.platform not in _PLATFORMS:
+            raise ValueError(f"platform={self.platform!r} must be one of {_PLATFORMS}")
+        for name in ("chunk_prefill_size", "num_kv_pages_per_block", "num_queries_per_block"):
+            v = getattr(self, name)
+            if v is not None and v <= 0:
+                raise ValueError(f"{name}={v} must be positive.")

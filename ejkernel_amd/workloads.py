@@ -53,6 +53,52 @@ class Batch:
                     logits_soft_cap=self.logits_soft_cap)
 
 
+@dataclass
+class V3Batch:
+    """Arguments of ``ragged_page_attention_v3`` built over a :class:`Batch` (same lengths, pages and queries)."""
+
+    queries: torch.Tensor
+    keys: torch.Tensor
+    values: torch.Tensor
+    kv_cache: torch.Tensor
+    kv_lens: torch.Tensor
+    block_tables: torch.Tensor
+    query_start_loc: torch.Tensor
+    distribution: torch.Tensor
+    base: Batch
+
+    def args(self):
+        return (self.queries, self.keys, self.values, self.kv_cache, self.kv_lens, self.block_tables,
+                self.query_start_loc, self.distribution)
+
+    def kwargs(self):
+        return dict(softmax_scale=self.base.softmax_scale, sliding_window=self.base.sliding_window,
+                    logits_soft_cap=self.base.logits_soft_cap)
+
+
+def to_v3(batch: Batch, seed: int = 0) -> V3Batch:
+    """New K/V rows for every query token; the cache shares ``batch.kv_pages``' memory, viewed in five dimensions.
+
+    The positions the new tokens will occupy hold random data beforehand, so a missed write shows in the output.
+    """
+    dev = batch.queries.device
+    dtype = batch.queries.dtype
+    t_alloc, _, head_dim = batch.queries.shape
+    num_pages, page_size, hx2, _ = batch.kv_pages.shape
+    pack = 32 // torch.finfo(dtype).bits
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(int(seed) + 7919)
+    keys = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype)
+    values = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype)
+    S = int(batch.num_seqs.reshape(-1)[0])
+    return V3Batch(
+        queries=batch.queries, keys=keys, values=values,
+        kv_cache=batch.kv_pages.view(num_pages, page_size, hx2 // pack, pack, head_dim),
+        kv_lens=batch.context_lens, block_tables=batch.block_tables.reshape(-1).contiguous(),
+        query_start_loc=batch.query_start_loc,
+        distribution=torch.tensor([0, 0, S], dtype=torch.int32, device=dev), base=batch)
+
+
 def _randn_chunked(shape, gen, device, dtype, chunk_elems=1 << 27):
     """N(0,1) in `dtype`, drawn in fp32 chunks so a large pool never needs 2x its size."""
     out = torch.empty(shape, dtype=dtype, device=device)

@@ -138,6 +138,18 @@ def test_bf16_head_dims(flags, D):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128)])
+@pytest.mark.parametrize("window", [None, 48])
+def test_bf16_prefill_tiles_over_many_key_tiles(flags, hq, hkv, D, window):
+    """Prefill chunks whose workgroup tiles walk three and more K/V tiles (the LDS stages are refilled while in
+    use), with and without earlier context, a partial last row tile, and decode sequences in the same batch."""
+    b = small([200, 1, 70, 130, 3], [200, 300, 100, 400, 90], num_q_heads=hq, num_kv_heads=hkv, head_dim=D,
+              pages_per_seq=32, sliding_window=window)
+    out = to_np(run_hip(b, flags))
+    assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, f"prefill tiles {hq}/{hkv} D={D} W={window}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
 def test_bf16_ragged_edge_cases(flags):
     """Empty sequences, kv_len not a page multiple, padding entries, garbage beyond the pages in use."""
     q_lens = [0, 1, 7, 0, 64, 1, 3, 130]

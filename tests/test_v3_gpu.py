@@ -1,0 +1,172 @@
+"""ragged_page_attention_v3 on the device (through ``rpa_v3_launch``) against its CPU oracle.
+
+The updated cache must match the oracle's bit for bit (it is a copy).  Outputs: bf16 within max-abs 2e-2 /
+mean-abs 2e-3 of the restatement of the reference program (``oracle/rpa_v3_oracle.py``); float32 within 1e-5 of the
+float64 dense evaluation on the updated cache.  Each case runs on the MFMA path and on the scalar path.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from ejkernel_amd import _native
+from ejkernel_amd.modules import RaggedPageAttentionv3Config, ragged_page_attention, ragged_page_attention_v3
+from ejkernel_amd.workloads import compact_for_host, make_batch, make_workload, to_v3
+from oracle import rpa_oracle
+from oracle.rpa_v3_oracle import rpa_v3
+from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PATHS = [pytest.param(0, id="tiled"), pytest.param(_native.RPA_FLAG_FORCE_GENERIC, id="generic")]
+
+
+def small(q_lens, kv_lens, **kw):
+    args = dict(num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=16, seed=3, device=DEV)
+    args.update(kw)
+    return to_v3(make_batch(q_lens, kv_lens, **args), seed=args["seed"])
+
+
+def oracle(v, **kw):
+    dt = "bfloat16" if v.queries.dtype == torch.bfloat16 else "float32"
+    k = dict(v.kwargs())
+    k.update(kw)
+    return rpa_v3(*[to_np(a) for a in v.args()], cache_dtype=dt, **k)
+
+
+def run_hip(v, flags=0, **kw):
+    k = dict(v.kwargs())
+    k.update(kw)
+    out, cache = ragged_page_attention_v3(*v.args(), _flags=flags, **k)
+    torch.cuda.synchronize()
+    assert cache.data_ptr() == v.kv_cache.data_ptr()  # updated in place and handed back
+    return out, cache
+
+
+CASES = {
+    "decode": ([1] * 9, [1, 16, 17, 33, 100, 255, 256, 64, 5], {}),
+    "mixed": ([9, 1, 0, 17, 2, 4], [40, 250, 8, 17, 133, 256], dict(max_num_seqs=8)),
+    "prefill": ([96, 130, 64], [96, 250, 200], dict(num_q_heads=8, num_kv_heads=2)),
+    "window_cap": ([5, 1, 40, 1], [90, 256, 120, 17], dict(sliding_window=24, logits_soft_cap=20.0)),
+    "gqa8_d256": ([3, 1, 70], [50, 200, 100], dict(num_q_heads=16, num_kv_heads=2, head_dim=256)),
+    "page4": ([2, 1, 33], [30, 64, 40], dict(page_size=4, pages_per_seq=16)),
+}
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("case", list(CASES))
+def test_bf16_parity_and_cache_update(case, flags):
+    q_lens, kv_lens, kw = CASES[case]
+    v = small(q_lens, kv_lens, **kw)
+    ref_out, ref_cache = oracle(v)          # before the device call: the cache is updated in place
+    out, cache = run_hip(v, flags)
+    assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
+    rows = int(sum(q_lens))
+    assert_bf16_parity(to_np(out), ref_out, rows, case)
+    assert not out[rows:].any()
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_scales(flags):
+    v = small([4, 1, 20], [60, 130, 20])
+    kw = dict(q_scale=4.0, k_scale=0.5, v_scale=2.0)
+    ref_out, ref_cache = oracle(v, **kw)
+    out, cache = run_hip(v, flags, **kw)
+    assert np.array_equal(to_np(cache), ref_cache)
+    mx, mean = err_stats(to_np(out), ref_out, 25)
+    assert mx <= 4e-2 and mean <= 4e-3, (mx, mean)   # outputs are doubled by v_scale, so is the tolerance
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_float32_against_float64_on_the_updated_cache(flags):
+    v = small([9, 1, 0, 17, 2, 4], [40, 250, 8, 17, 133, 256], dtype=torch.float32, max_num_seqs=8)
+    out, cache = run_hip(v, flags)
+    P, page, _, _, D = cache.shape
+    b = v.base
+    ref = rpa_oracle.rpa_exact(to_np(v.queries), to_np(cache).reshape(P, page, -1, D), to_np(v.kv_lens),
+                               to_np(b.block_tables), to_np(v.query_start_loc), to_np(b.num_seqs),
+                               softmax_scale=b.softmax_scale)
+    mx, _ = err_stats(to_np(out), ref, b.total_valid_tokens)
+    assert mx <= F32_MAX_ABS, mx
+
+
+def test_new_rows_land_where_the_block_table_says_and_nothing_else_changes():
+    v = small([3, 1, 0, 6], [19, 33, 7, 6], page_size=4, pages_per_seq=16)
+    before = v.kv_cache.clone()
+    _, cache = run_hip(v)
+    b = v.base
+    P, page, _, _, D = cache.shape
+    rows_after = cache.view(P, page, -1, D)
+    expect = before.view(P, page, -1, D).clone()
+    bt = b.block_tables.cpu().numpy()
+    qsl = v.query_start_loc.cpu().numpy()
+    for s, (ql, kl) in enumerate(zip(b.q_lens, b.kv_lens)):
+        for t in range(int(ql)):
+            pos = int(kl - ql + t)
+            expect[bt[s, pos // page], pos % page, 0::2] = v.keys[qsl[s] + t]
+            expect[bt[s, pos // page], pos % page, 1::2] = v.values[qsl[s] + t]
+    assert torch.equal(rows_after, expect)
+
+
+def test_same_result_as_the_v2_operation_on_the_updated_cache():
+    """The attention half is the v2 operation with fp32 logits: the two agree within the bf16 tolerance."""
+    v = small([9, 1, 0, 17, 2, 4], [40, 250, 8, 17, 133, 256], max_num_seqs=8)
+    out3, cache = run_hip(v)
+    b = v.base
+    out2 = ragged_page_attention(*b.args(), **b.kwargs())   # b.kv_pages shares the updated memory
+    rows = b.total_valid_tokens
+    assert_bf16_parity(to_np(out3), to_np(out2), rows, "v3 vs v2")
+
+
+def test_validation_errors_follow_the_reference():
+    v = small([2, 1], [20, 30])
+    a = list(v.args())
+    with pytest.raises(ValueError, match="distribution shape"):
+        ragged_page_attention_v3(*a[:7], torch.zeros(2, dtype=torch.int32, device=DEV))
+    with pytest.raises(ValueError, match="index arrays must be int32"):
+        ragged_page_attention_v3(*a[:4], a[4].long(), *a[5:])
+    with pytest.raises(ValueError, match="soft_cap"):
+        ragged_page_attention_v3(*a, logits_soft_cap=0.0)
+    with pytest.raises(ValueError, match="sliding_window"):
+        ragged_page_attention_v3(*a, sliding_window=0)
+    with pytest.raises(ValueError, match="packing mismatch"):
+        ragged_page_attention_v3(*a[:3], a[3].reshape(a[3].shape[0], a[3].shape[1], -1, 1, 128), *a[4:])
+    with pytest.raises(ValueError):
+        ragged_page_attention_v3(*a, cfg=RaggedPageAttentionv3Config(num_queries_per_block=0))
+    with pytest.raises(NotImplementedError):
+        ragged_page_attention_v3(*a, mesh=object())
+
+
+@pytest.mark.parametrize("name,n_sample", [("decode_llama3_8b", 10), ("mixed_prefill_decode", 12)])
+def test_full_size_workload(name, n_sample):
+    """Sampled parity against the oracle plus size-independent properties of the cache update."""
+    b = make_workload(name, device=DEV)
+    v = to_v3(b, seed=5)
+    rng = np.random.default_rng(1)
+    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:n_sample])
+    sub = compact_for_host(b, ids)                       # pages of the sampled sequences, before the update
+    rows_idx = sub.meta["rows"]
+    sub_v = to_v3(sub, seed=0)
+    sub_v.keys[: len(rows_idx)] = v.keys[rows_idx.to(DEV)].cpu()
+    sub_v.values[: len(rows_idx)] = v.values[rows_idx.to(DEV)].cpu()
+    ref_out, _ = oracle(sub_v)
+    checksum_before = b.kv_pages.view(torch.int16).sum(dtype=torch.int64).item()
+    out, cache = run_hip(v)
+    rows = sub.total_valid_tokens
+    got = to_np(out[rows_idx.to(DEV)])
+    assert_bf16_parity(got, ref_out, rows, name)
+    total = b.total_valid_tokens
+    assert torch.isfinite(out.float()).all() and not out[total:].any()
+    # every new row is in the cache at its position, and the cache changed by exactly those rows
+    P, page, _, _, D = cache.shape
+    rows_after = cache.view(P, page, -1, D)
+    qsl = b.query_start_loc.long()
+    S = len(b.q_lens)
+    seq_of_tok = torch.repeat_interleave(torch.arange(S, device=DEV), torch.as_tensor(b.q_lens, device=DEV))
+    t = torch.arange(total, device=DEV)
+    pos = b.context_lens.long()[seq_of_tok] - torch.as_tensor(b.q_lens, device=DEV)[seq_of_tok] + (t - qsl[seq_of_tok])
+    pg = b.block_tables.long()[seq_of_tok, pos // page]
+    assert torch.equal(rows_after[pg, pos % page, 0::2], v.keys[:total])
+    assert torch.equal(rows_after[pg, pos % page, 1::2], v.values[:total])
+    checksum_after = cache.view(torch.int16).sum(dtype=torch.int64).item()
+    assert checksum_after != checksum_before
