@@ -36,6 +36,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="decode_llama3_8b")
+    ap.add_argument("--op", default="rpa", choices=["rpa", "rpa_v3"],
+                    help="rpa = ragged_page_attention (the headline path); rpa_v3 = ragged_page_attention_v3 on the same "
+                         "workload: every query token also brings a new K/V row that is written into the cache first")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -108,6 +111,63 @@ def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs, budget
     return res
 
 
+def cpu_sample_and_parity_v3(batch, v3, out, want_baseline, want_parity, n_seqs, budget_s=12.0):
+    """The same for ragged_page_attention_v3: the NumPy restatement of the reference program (oracle/rpa_v3_oracle.py)
+    on a bounded sample of sequences, whose cache pages are taken as they were before the timed calls."""
+    import numpy as np
+
+    from ejkernel_amd.workloads import compact_for_host, to_v3
+    from oracle.rpa_v3_oracle import rpa_v3
+    from tests.helpers import err_stats, to_np
+
+    try:
+        from threadpoolctl import threadpool_info
+        threads = max([int(i.get("num_threads", 1)) for i in threadpool_info()] or [1])
+    except Exception:  # pragma: no cover
+        threads = 1
+    S = len(batch.q_lens)
+    rng = np.random.default_rng(0)
+    cand = [int(s) for s in rng.permutation(S) if batch.q_lens[s] > 0]
+
+    def run(ids):
+        sub = compact_for_host(batch, sorted(ids))
+        sv = to_v3(sub)
+        rows_idx = sub.meta["rows"]
+        sv.keys[: len(rows_idx)] = v3.keys[rows_idx.to(v3.keys.device)].cpu()
+        sv.values[: len(rows_idx)] = v3.values[rows_idx.to(v3.keys.device)].cpu()
+        a = [to_np(x) for x in sv.args()]
+        t0 = time.perf_counter()
+        ref, _ = rpa_v3(*a, **sv.kwargs())
+        return sub, ref, time.perf_counter() - t0
+
+    if n_seqs <= 0:
+        sub, _, dt = run(cand[:1])
+        work = lambda ids: float(sum(int(batch.q_lens[s]) * int(batch.kv_lens[s]) + int(batch.kv_lens[s]) for s in ids))  # noqa: E731
+        rate = work(cand[:1]) / max(dt, 1e-3)
+        n_seqs, acc = 0, 0.0
+        for s in cand:
+            acc += work([s])
+            n_seqs += 1
+            if acc / rate > budget_s:
+                break
+    ids = cand[:max(1, n_seqs)]
+    sub, ref, dt = run(ids)
+    rows = sub.total_valid_tokens
+    res = {}
+    if want_parity:
+        got = to_np(out[sub.meta["rows"].to(out.device)])
+        mx, mean = err_stats(got, ref, rows)
+        res["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": rows, "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
+    if want_baseline:
+        res["cpu_baseline"] = {
+            "value": rows / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
+            "sample": f"{len(ids)} of {S} sequences ({rows} query tokens, {int(sub.kv_lens.sum())} kv tokens), one run of "
+                      f"{dt:.2f} s; NumPy restatement of the reference's v3 program (cache update, float32 dense attention per "
+                      f"sequence on the visible keys), BLAS threads {threads}",
+        }
+    return res
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -143,7 +203,19 @@ def main():
                                 num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m["page_size"],
                                 sliding_window=batch.sliding_window)
 
+    v3 = None
+    if args.op == "rpa_v3":
+        from ejkernel_amd.modules import ragged_page_attention_v3
+        from ejkernel_amd.workloads import to_v3
+
+        v3 = to_v3(batch, seed=1)
+        # the new rows are read once and written once into the cache, on top of the attention traffic
+        row_bytes = 2 * m["num_kv_heads"] * m["head_dim"] * 2
+        counts["bytes"] += 2 * counts["tokens"] * row_bytes
+
     def step():
+        if v3 is not None:
+            return ragged_page_attention_v3(*v3.args(), **v3.kwargs())[0]
         return ragged_page_attention(*batch.args(), **batch.kwargs())
 
     for _ in range(args.warmup):
@@ -173,20 +245,27 @@ def main():
     else:
         roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
-    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.scale == 1.0 else None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
+    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.scale == 1.0 and v3 is None else None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
                  "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
                  "algorithmic_flops": counts["flops"], "tflops": tflops, "gbps": gbps})
 
     line = {
-        "metric": "ragged paged-attn tokens/s", "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "metric": "ragged paged-attn tokens/s" if v3 is None else "ragged paged-attn v3 (cache update + attention) tokens/s", "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": args.workload, "description": WORKLOADS[args.workload], "scale": args.scale,
+        "config": {"workload": args.workload, "op": args.op, "description": WORKLOADS[args.workload], "scale": args.scale,
                    "query_tokens": tokens, "num_seqs": len(batch.q_lens), "kv_tokens": int(batch.kv_lens.sum())},
         "roofline": roof,
     }
     if not (args.no_cpu_baseline and args.no_parity):
-        line.update(cpu_sample_and_parity(batch, out, not args.no_cpu_baseline, not args.no_parity, args.cpu_seqs))
+        if v3 is None:
+            line.update(cpu_sample_and_parity(batch, out, not args.no_cpu_baseline, not args.no_parity, args.cpu_seqs))
+        else:
+            # Repeating the call rewrites the same rows with the same values, so the cache after the timed steps is the
+            # cache after one update; the oracle starts from the pages with the new rows still holding their old content,
+            # which only differ at the positions it overwrites itself.
+            line.update(cpu_sample_and_parity_v3(batch, v3, out, not args.no_cpu_baseline, not args.no_parity,
+                                                 args.cpu_seqs))
     print(json.dumps(line))
 
 

@@ -85,6 +85,10 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   bf16x8_t qreg[MRT][C::NKS];
   const float scale = rbf(p.softmax_scale);
   const float post_scale = logit_scale(p);
+  // Without a soft cap the fp32 logit scale is not applied to every logit: maxima and the exp2 argument take it
+  // as a factor (it is positive), which costs nothing per key.
+  const bool fold_scale = !kMimic && cap == 0.f && post_scale > 0.f;
+  const float sf = fold_scale ? post_scale : 1.f, sf_log2e = sf * kLog2e;
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
     const int R = w_row_lo + 16 * m + i;
@@ -320,7 +324,13 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
           for (int u = 0; u < 2; ++u)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? s_acc[m][u][r] : s_acc[m][u][r] * post_scale;
+            for (int r = 0; r < 4; ++r) sv[u][r] = s_acc[m][u][r];
+          if (!kMimic && !fold_scale) {  // wave-uniform: only with a soft cap (or a non-positive scale)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) sv[u][r] *= post_scale;
+          }
           if (cap != 0.f) {
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -342,8 +352,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                 sv[u][r] = keep ? sv[u][r] : -INFINITY;
               }
           }
-          float tmax = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
-                             fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
+          float tmax = sf * fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
+                                  fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
           // Lazy rescale: the reference point m_run (the same in the four lanes of a row) only moves when some
           // logit exceeds it by more than kLazy; probabilities then stay below e^kLazy, far inside bf16 / fp32
           // range.  The common case needs no cross-lane step at all: a wave-wide vote on the lane-local maxima.
@@ -364,10 +374,10 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           const float neg = -m_use * kLog2e;
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
-            float e0 = __builtin_amdgcn_exp2f(fmaf(sv[u][0], kLog2e, neg));
-            float e1 = __builtin_amdgcn_exp2f(fmaf(sv[u][1], kLog2e, neg));
-            float e2 = __builtin_amdgcn_exp2f(fmaf(sv[u][2], kLog2e, neg));
-            float e3 = __builtin_amdgcn_exp2f(fmaf(sv[u][3], kLog2e, neg));
+            float e0 = __builtin_amdgcn_exp2f(fmaf(sv[u][0], sf_log2e, neg));
+            float e1 = __builtin_amdgcn_exp2f(fmaf(sv[u][1], sf_log2e, neg));
+            float e2 = __builtin_amdgcn_exp2f(fmaf(sv[u][2], sf_log2e, neg));
+            float e3 = __builtin_amdgcn_exp2f(fmaf(sv[u][3], sf_log2e, neg));
             pw[m][2 * u] = pack_bf16x2(e0, e1);
             pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
           }
