@@ -26,6 +26,8 @@ EXPORTED_SYMBOLS = (
     "rpa_workspace_init",
     "rpa_fwd_launch",
     "rpa_v3_launch",
+    "rpa_page_attention_workspace_bytes",
+    "rpa_page_attention_launch",
 )
 
 
@@ -78,6 +80,32 @@ class RpaV3Params(ctypes.Structure):
     ]
 
 
+class RpaPageAttnParams(ctypes.Structure):
+    """Field-for-field image of ``struct RpaPageAttnParams``."""
+
+    _fields_ = [
+        ("query", ctypes.c_void_p),
+        ("key_cache", ctypes.c_void_p),
+        ("value_cache", ctypes.c_void_p),
+        ("context_lens", ctypes.c_void_p),
+        ("block_tables", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("num_seqs", ctypes.c_int32),
+        ("num_q_heads", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("block_size", ctypes.c_int32),
+        ("num_blocks", ctypes.c_int32),
+        ("max_blocks", ctypes.c_int32),
+        ("attn_scale", ctypes.c_float),
+        ("dtype", ctypes.c_int32),
+        ("compute", ctypes.c_int32),
+        ("flags", ctypes.c_uint32),
+    ]
+
+
 class NativeLibraryError(RuntimeError):
     pass
 
@@ -114,6 +142,10 @@ def load() -> ctypes.CDLL:
     lib.rpa_fwd_launch.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
     lib.rpa_v3_launch.restype = ctypes.c_int
     lib.rpa_v3_launch.argtypes = [ctypes.POINTER(RpaV3Params), ctypes.c_void_p]
+    lib.rpa_page_attention_workspace_bytes.restype = ctypes.c_uint64
+    lib.rpa_page_attention_workspace_bytes.argtypes = [ctypes.POINTER(RpaPageAttnParams)]
+    lib.rpa_page_attention_launch.restype = ctypes.c_int
+    lib.rpa_page_attention_launch.argtypes = [ctypes.POINTER(RpaPageAttnParams), ctypes.c_void_p]
     if lib.rpa_abi_version() != RPA_ABI_VERSION:
         raise NativeLibraryError(
             f"{LIB_PATH} has ABI version {lib.rpa_abi_version()}, this package expects {RPA_ABI_VERSION}: rebuild it"

@@ -22,7 +22,7 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-static int validate(const RpaParams& p, bool need_pointers) {
+static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_seq = false) {
   if (p.total_tokens < 0 || p.num_q_heads <= 0 || p.num_kv_heads <= 0 || p.head_dim <= 0 || p.page_size <= 0 ||
       p.num_pages <= 0 || p.max_num_seqs <= 0 || p.pages_per_seq <= 0 || p.num_sinks < 0)
     return fail(RPA_ERR_INVALID_ARGUMENT, "non-positive dimension in RpaParams");
@@ -38,7 +38,8 @@ static int validate(const RpaParams& p, bool need_pointers) {
   if (!(p.q_scale >= 0.f) || !(p.k_scale >= 0.f) || !(p.v_scale >= 0.f))
     return fail(RPA_ERR_INVALID_ARGUMENT, "q_scale / k_scale / v_scale must be positive (0 = absent)");
   if (need_pointers) {
-    if (!p.queries || !p.kv_pages || !p.context_lens || !p.block_tables || !p.query_start_loc || !p.num_seqs || !p.out)
+    if (!p.queries || !p.kv_pages || !p.context_lens || !p.block_tables || !p.out ||
+        (!one_token_per_seq && (!p.query_start_loc || !p.num_seqs)))
       return fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaParams");
     if (p.num_sinks > 0 && !p.sinks) return fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d but sinks is null", p.num_sinks);
   }
@@ -93,25 +94,91 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
   return RPA_OK;
 }
 
+namespace rpa {
+static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream);
+}
+
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {
   if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
   const RpaParams& p = *params;
   int rc = rpa::validate(p, true);
   if (rc != RPA_OK) return rc;
-  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
-  if (rpa::tiled_supported(p)) {
-    rc = rpa::launch_tiled(p, stream);
+  return rpa::dispatch(p, rpa::interleaved_layout(p), rpa::tiled_supported(p), static_cast<hipStream_t>(hip_stream));
+}
+
+static RpaParams page_attention_params(const RpaPageAttnParams& a) {
+  RpaParams p = {};
+  p.queries = a.query;
+  p.kv_pages = a.key_cache;
+  p.context_lens = a.context_lens;
+  p.block_tables = a.block_tables;
+  p.query_start_loc = nullptr;  // sequence s owns row s
+  p.num_seqs = nullptr;         // all of them are present
+  p.out = a.out;
+  p.workspace = a.workspace;
+  p.workspace_bytes = a.workspace_bytes;
+  p.total_tokens = a.num_seqs;
+  p.max_num_seqs = a.num_seqs;
+  p.num_q_heads = a.num_q_heads;
+  p.num_kv_heads = a.num_kv_heads;
+  p.head_dim = a.head_dim;
+  p.page_size = a.block_size;
+  p.num_pages = a.num_blocks;
+  p.pages_per_seq = a.max_blocks;
+  p.softmax_scale = a.attn_scale;
+  p.dtype = a.dtype;
+  p.compute = a.compute;
+  p.flags = a.flags & (RPA_FLAG_FORCE_GENERIC | RPA_FLAG_FP32_LOGITS);
+  return p;
+}
+
+// The tiled decode loop handles up to four 16-row tiles per (sequence, kv head); larger query groups would need
+// the prefill tile, which assumes the interleaved cache.
+static bool page_attention_tiled(const RpaParams& p) {
+  return rpa::tiled_supported(p) && p.num_q_heads / p.num_kv_heads <= 64;
+}
+
+uint64_t rpa_page_attention_workspace_bytes(const RpaPageAttnParams* dims) {
+  if (dims == nullptr) return 0;
+  const RpaParams p = page_attention_params(*dims);
+  return rpa_workspace_bytes(&p);
+}
+
+int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream) {
+  if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
+  const RpaParams p = page_attention_params(*params);
+  int rc = rpa::validate(p, true, true);
+  if (rc != RPA_OK) return rc;
+  if (!params->value_cache) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaPageAttnParams");
+  const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
+  rpa::KvLayout kv;
+  kv.k_base = static_cast<const char*>(params->key_cache);
+  kv.v_base = static_cast<const char*>(params->value_cache);
+  kv.stride_b = p.head_dim * esize;
+  kv.head_b = static_cast<uint32_t>(p.page_size) * kv.stride_b;
+  kv.page_b = static_cast<uint64_t>(p.num_kv_heads) * kv.head_b;
+  if (static_cast<uint64_t>(p.page_size) * p.head_dim * esize > 0xffffffffull)
+    return rpa::fail(RPA_ERR_UNSUPPORTED, "a cache block of one head exceeds 4 GiB");
+  return rpa::dispatch(p, kv, page_attention_tiled(p), static_cast<hipStream_t>(hip_stream));
+}
+
+namespace rpa {
+static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream) {
+  int rc;
+  if (tiled) {
+    rc = rpa::launch_tiled(p, kv, stream);
     if (rc == RPA_ERR_WORKSPACE)
       return rpa::fail(rc, "workspace of %llu bytes is too small, rpa_workspace_bytes() asks for %llu",
                        (unsigned long long)p.workspace_bytes, (unsigned long long)rpa_workspace_bytes(&p));
     if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
     return RPA_OK;
   }
-  rc = rpa::launch_generic(p, stream);
+  rc = rpa::launch_generic(p, kv, stream);
   if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
   return RPA_OK;
 }
+}  // namespace rpa
 
 int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");

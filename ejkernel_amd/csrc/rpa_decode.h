@@ -68,7 +68,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
 
-  const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;  // elements between tokens
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
   // Same row through the constant address space: reads with a wave-uniform index become scalar loads, which
   // are counted apart from the vector loads of the K/V stream.  The block table is never written by this kernel.
@@ -88,10 +87,12 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   // the row address is a scalar base plus one per-lane byte offset that is constant for the whole item.
   // Slow path (last tile of a range, small pages): per-lane page lookup; tokens past the end of the range are
   // replaced by the last valid one (their scores are masked).
-  const char* kvb = reinterpret_cast<const char*>(kv);
-  const uint32_t stride_b = static_cast<uint32_t>(tok_stride) * 2u;  // bytes between tokens
-  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
-  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + static_cast<uint32_t>(2 * j * D * 2 + 16 * i);
+  const char* kvb = a.kv.k_base;
+  const int64_t v_delta = a.kv.v_base - a.kv.k_base;  // the V row of a (token, head) relative to its K row
+  const uint32_t stride_b = a.kv.stride_b;            // bytes between tokens
+  const uint64_t page_b = a.kv.page_b;
+  const uint32_t head_off = static_cast<uint32_t>(j) * a.kv.head_b;
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + static_cast<uint32_t>(16 * i);
   auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
     if (a.uniform_page && tile + C::TT <= range_hi) {
 #pragma unroll
@@ -104,10 +105,11 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const char* row = sbase + static_cast<uint64_t>(r) * stride_b;
+          const char* row_v = row + v_delta;
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN) {
             kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN));
-            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN + 2u * D));
+            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row_v + (lane_off + 256u * sN));
           }
         }
       }
@@ -120,14 +122,14 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       int page = bt[t4c >> a.page_shift];
       page = min(max(page, 0), p.num_pages - 1);
       const char* base = kvb + static_cast<uint64_t>(page) * page_b +
-                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (2 * j * D * 2 + 16 * i);
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + 16 * i);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
           kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN);
-          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN + 2 * D);
+          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + v_delta + 256 * sN);
         }
       }
     }

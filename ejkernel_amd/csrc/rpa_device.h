@@ -59,4 +59,17 @@ __device__ __forceinline__ int find_seq(const int32_t* __restrict__ cu, int n, i
   return lo;
 }
 
+// Ragged metadata with the one-token-per-sequence case folded in: a null query_start_loc means sequence s owns
+// exactly row s, a null num_seqs means every one of the max_num_seqs sequences is present (page_attention).
+__device__ __forceinline__ int seq_count(const RpaParams& p) {
+  int n = p.num_seqs != nullptr ? p.num_seqs[0] : p.max_num_seqs;
+  return n < 0 ? 0 : (n > p.max_num_seqs ? p.max_num_seqs : n);
+}
+__device__ __forceinline__ int q_start_of(const RpaParams& p, int s) {
+  return p.query_start_loc != nullptr ? p.query_start_loc[s] : s;
+}
+__device__ __forceinline__ int seq_of_row(const RpaParams& p, int nseq, int row) {
+  return p.query_start_loc != nullptr ? find_seq(p.query_start_loc, nseq, row) : row;
+}
+
 }  // namespace rpa

@@ -15,7 +15,7 @@ namespace rpa {
 constexpr int kMaxElemsPerLane = 8;  // head_dim <= 512
 
 template <typename T, bool kBf16Compute>
-__global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
+__global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayout kvl) {
   extern __shared__ float q_lds[];  // [head_dim] scaled query row of the current head
   const int row = blockIdx.x;
   const int j = blockIdx.y;
@@ -23,21 +23,19 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
   const int D = p.head_dim;
   const int G = p.num_q_heads / p.num_kv_heads;
   const T* __restrict__ q = static_cast<const T*>(p.queries);
-  const T* __restrict__ kv = static_cast<const T*>(p.kv_pages);
   T* __restrict__ out = static_cast<T*>(p.out);
 
-  int nseq = p.num_seqs[0];
-  nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
-  const int total = p.query_start_loc[nseq];
+  const int nseq = seq_count(p);
+  const int total = q_start_of(p, nseq);
   const size_t row_base = (static_cast<size_t>(row) * p.num_q_heads + static_cast<size_t>(j) * G) * D;
   if (row >= total) {  // rows past the ragged batch are defined as zero
     for (int i = lane; i < G * D; i += kWave) Elem<T>::store(out + row_base + i, 0.f);
     return;
   }
-  const int s = find_seq(p.query_start_loc, nseq, row);
-  const int q_len = p.query_start_loc[s + 1] - p.query_start_loc[s];
+  const int s = seq_of_row(p, nseq, row);
+  const int q_len = q_start_of(p, s + 1) - q_start_of(p, s);
   const int kv_len = p.context_lens[s];
-  const int pos = kv_len - q_len + (row - p.query_start_loc[s]);
+  const int pos = kv_len - q_len + (row - q_start_of(p, s));
   const int hi = min(pos + 1, kv_len);
   const int lo = p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0;
 
@@ -50,7 +48,6 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
   const float post = p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f);
   const float o_scale = p.v_scale > 0.f ? p.v_scale : 1.f;
   const float cap = p.logits_soft_cap;
-  const size_t tok_stride = static_cast<size_t>(2) * p.num_kv_heads * D;
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
 
   for (int g = 0; g < G; ++g) {
@@ -80,10 +77,10 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
       const int t = t0 + lane;
       const bool valid = t < hi;
       const int tc = valid ? t : hi - 1;
-      const int page = bt[tc / p.page_size];
-      const size_t tok = static_cast<size_t>(page) * p.page_size + (tc % p.page_size);
-      const size_t k_off = tok * tok_stride + static_cast<size_t>(2 * j) * D;
-      const T* __restrict__ kp = kv + k_off;
+      const int page = min(max(bt[tc / p.page_size], 0), p.num_pages - 1);
+      const size_t k_off = static_cast<size_t>(page) * kvl.page_b + static_cast<size_t>(tc % p.page_size) * kvl.stride_b +
+                           static_cast<size_t>(j) * kvl.head_b;  // bytes from the K (or V) base
+      const T* __restrict__ kp = reinterpret_cast<const T*>(kvl.k_base + k_off);
       float sc = 0.f;
       for (int d = 0; d < D; ++d) {
         float kvv = Elem<T>::load(kp + d);
@@ -120,7 +117,7 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
       for (int tt = 0; tt < n_in_tile; ++tt) {
         const float p_tt = __shfl(pr, tt, kWave);
         const size_t o = (static_cast<size_t>(__shfl(off_hi, tt, kWave)) << 32) | __shfl(off_lo, tt, kWave);
-        const T* __restrict__ vp = kv + o + D;  // V row follows the K row of the same kv head
+        const T* __restrict__ vp = reinterpret_cast<const T*>(kvl.v_base + o);
 #pragma unroll
         for (int e = 0; e < kMaxElemsPerLane; ++e) {
           const int d = lane + e * kWave;
@@ -153,18 +150,18 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p) {
   }
 }
 
-int launch_generic(const RpaParams& p, hipStream_t stream) {
+int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   if (p.head_dim > kMaxElemsPerLane * kWave) return RPA_ERR_UNSUPPORTED;
   if (p.total_tokens == 0) return RPA_OK;
   dim3 grid(p.total_tokens, p.num_kv_heads), block(kWave);
   const size_t lds = static_cast<size_t>(p.head_dim) * sizeof(float);
   const bool bf16c = p.compute == RPA_COMPUTE_BF16;
   if (p.dtype == RPA_DTYPE_BF16) {
-    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, true>), grid, block, lds, stream, p);
-    else hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, false>), grid, block, lds, stream, p);
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, true>), grid, block, lds, stream, p, kv);
+    else hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, false>), grid, block, lds, stream, p, kv);
   } else {
-    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<float, true>), grid, block, lds, stream, p);
-    else hipLaunchKernelGGL((rpa_generic_kernel<float, false>), grid, block, lds, stream, p);
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<float, true>), grid, block, lds, stream, p, kv);
+    else hipLaunchKernelGGL((rpa_generic_kernel<float, false>), grid, block, lds, stream, p, kv);
   }
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }

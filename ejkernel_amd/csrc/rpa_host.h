@@ -7,8 +7,28 @@
 
 namespace rpa {
 
+// Where the K and V rows of (page, slot, kv head) live, in bytes.  ragged_page_attention interleaves K and V of a
+// head inside one token record; page_attention keeps two caches of [blocks, kv heads, block, head_dim].
+struct KvLayout {
+  const char* k_base;
+  const char* v_base;
+  uint64_t page_b;    // between pages
+  uint32_t stride_b;  // between the tokens of a page
+  uint32_t head_b;    // between the kv heads of a token
+};
+inline KvLayout interleaved_layout(const RpaParams& p) {
+  const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
+  KvLayout l;
+  l.k_base = static_cast<const char*>(p.kv_pages);
+  l.v_base = l.k_base + static_cast<size_t>(p.head_dim) * esize;
+  l.stride_b = 2u * p.num_kv_heads * p.head_dim * esize;
+  l.page_b = static_cast<uint64_t>(p.page_size) * l.stride_b;
+  l.head_b = 2u * p.head_dim * esize;
+  return l;
+}
+
 // Each returns RPA_OK or a negative RPA_ERR_* code; all of them only enqueue on `stream`.
-int launch_generic(const RpaParams& p, hipStream_t stream);
+int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream);
 // Writes the new tokens' K/V rows into the paged cache (ragged_page_attention_v3, _kernel.py:207-218).
 int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream);
 
@@ -30,7 +50,7 @@ struct WorkspaceLayout {
 
 bool tiled_supported(const RpaParams& p);
 void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl);
-int launch_tiled(const RpaParams& p, hipStream_t stream);
+int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream);
 
 // Compute units of the current device (cached per device).
 int device_cu_count();

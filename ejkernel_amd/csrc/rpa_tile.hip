@@ -55,8 +55,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   char* lds_data = smem + sched_bytes(p.max_num_seqs);
   char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
-  int nseq = p.num_seqs[0];
-  nseq = min(max(nseq, 0), p.max_num_seqs);
+  const int nseq = seq_count(p);
 
   // ---- schedule.  Per sequence: tiles it adds to the decode stream (one row tile, has keys), workgroup tiles
   // (more than kWaveItemMaxRowTiles row tiles), or wave-level items (everything else).
@@ -102,7 +101,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 
   // ---- rows past the ragged batch are zero
   {
-    const int total_rows = p.query_start_loc[nseq];
+    const int total_rows = q_start_of(p, nseq);
     const int row_u4 = p.num_q_heads * D / 8;  // 16-byte pieces per row
     u32x4_t* o4 = static_cast<u32x4_t*>(p.out);
     for (int row = total_rows + blockIdx.x; row < p.total_tokens; row += gridDim.x)
@@ -324,12 +323,13 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
-int launch_tiled(const RpaParams& p, hipStream_t stream) {
+int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   WorkspaceLayout wl;
   tiled_workspace_layout(p, &wl);
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
   TileArgs a;
   a.p = p;
+  a.kv = kv;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);

@@ -19,6 +19,7 @@ constexpr float kLog2e = 1.4426950408889634f;
 
 struct TileArgs {
   RpaParams p;
+  KvLayout kv;        // K / V addressing of the decode loop (prefill tiles assume the interleaved layout)
   int page_shift;     // log2(page_size)
   int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
   int decode_grid;    // workgroups that take part when the batch has no prefill tiles
@@ -97,8 +98,8 @@ struct SeqInfo {
 template <int TT>
 __device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
   SeqInfo si;
-  si.q0 = p.query_start_loc[s];
-  si.q_len = p.query_start_loc[s + 1] - si.q0;
+  si.q0 = q_start_of(p, s);
+  si.q_len = q_start_of(p, s + 1) - si.q0;
   si.kv_len = p.context_lens[s];
   si.rows = si.q_len > 0 ? si.q_len * G : 0;
   si.n_rt = (si.rows + 15) >> 4;

@@ -3,13 +3,17 @@
 
 from .operations import (
     BaseOperationConfig,
+    PageAttention,
+    PageAttentionConfig,
     RaggedPageAttention,
     RaggedPageAttentionConfig,
     RaggedPageAttentionv3,
     RaggedPageAttentionv3Config,
+    page_attention,
     ragged_page_attention,
     ragged_page_attention_v3,
 )
 
-__all__ = ["BaseOperationConfig", "RaggedPageAttention", "RaggedPageAttentionConfig", "RaggedPageAttentionv3",
-           "RaggedPageAttentionv3Config", "ragged_page_attention", "ragged_page_attention_v3"]
+__all__ = ["BaseOperationConfig", "PageAttention", "PageAttentionConfig", "RaggedPageAttention",
+           "RaggedPageAttentionConfig", "RaggedPageAttentionv3", "RaggedPageAttentionv3Config", "page_attention",
+           "ragged_page_attention", "ragged_page_attention_v3"]

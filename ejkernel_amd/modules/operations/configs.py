@@ -64,3 +64,17 @@ class RaggedPageAttentionv3Config(BaseOperationConfig):
             v = getattr(self, name)
             if v is not None and v <= 0:
                 raise ValueError(f"{name}={v} must be positive.")
+
+
+@dataclass
+class PageAttentionConfig(BaseOperationConfig):
+    """Configuration for page attention (ejkernel/modules/operations/configs.py:147-162)."""
+
+    num_splits: int = 0
+    pages_per_compute_block: int | None = None
+    num_warps: int = 4
+    num_stages: int = 1
+
+    def validate(self) -> None:
+        if self.platform not in _PLATFORMS:
+            raise ValueError(f"platform={self.platform!r} must be one of {_PLATFORMS}")

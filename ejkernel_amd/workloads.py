@@ -99,6 +99,90 @@ def to_v3(batch: Batch, seed: int = 0) -> V3Batch:
         distribution=torch.tensor([0, 0, S], dtype=torch.int32, device=dev), base=batch)
 
 
+@dataclass
+class PageAttnBatch:
+    """Arguments of ``page_attention``: one query token per sequence over separate paged K and V caches."""
+
+    query: torch.Tensor
+    key_cache: torch.Tensor
+    value_cache: torch.Tensor
+    context_lens: torch.Tensor
+    block_tables: torch.Tensor
+    attn_scale: float
+    kv_lens: np.ndarray | None = None
+    name: str = ""
+    meta: dict = field(default_factory=dict)
+
+    def args(self):
+        return (self.query, self.key_cache, self.value_cache, self.context_lens, self.block_tables)
+
+
+def make_page_attention_batch(kv_lens, *, num_q_heads, num_kv_heads, head_dim, block_size, max_blocks, num_blocks=None,
+                              seed=0, device="cpu", dtype=torch.bfloat16, name="") -> PageAttnBatch:
+    """Random caches of [num_blocks, num_kv_heads, block_size, head_dim]; blocks of different sequences are distinct."""
+    kv_lens = np.asarray(kv_lens, dtype=np.int64)
+    S = len(kv_lens)
+    assert kv_lens.max(initial=0) <= max_blocks * block_size
+    num_blocks = num_blocks or S * max_blocks
+    assert num_blocks >= S * max_blocks
+    rng = np.random.Generator(np.random.PCG64(seed))
+    bt = rng.permutation(num_blocks)[: S * max_blocks].reshape(S, max_blocks).astype(np.int32)
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(int(seed))
+    shape = (num_blocks, num_kv_heads, block_size, head_dim)
+    return PageAttnBatch(
+        query=_randn_chunked((S, num_q_heads, head_dim), gen, dev, dtype),
+        key_cache=_randn_chunked(shape, gen, dev, dtype), value_cache=_randn_chunked(shape, gen, dev, dtype),
+        context_lens=torch.from_numpy(kv_lens.astype(np.int32)).to(dev), block_tables=torch.from_numpy(bt).to(dev),
+        attn_scale=float(head_dim**-0.5), kv_lens=kv_lens, name=name,
+        meta=dict(num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, page_size=block_size,
+                  pages_per_seq=max_blocks, num_pages=num_blocks, max_num_seqs=S, seed=seed))
+
+
+def page_attention_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bfloat16) -> PageAttnBatch:
+    """The decode workloads (one token per sequence) with the cache layout of ``page_attention``."""
+    seed = 1003
+    rng = np.random.Generator(np.random.PCG64(seed))
+
+    def n(x, lo=1):
+        return max(lo, int(round(x * scale)))
+
+    if name == "decode_small":
+        kv = rng.integers(64, 513, size=8)
+        return make_page_attention_batch(kv, num_q_heads=8, num_kv_heads=2, head_dim=128, block_size=16, max_blocks=32,
+                                         num_blocks=512, seed=seed, device=device, dtype=dtype, name=name)
+    if name == "decode_llama3_8b":
+        S = n(256)
+        kv = rng.integers(n(512), n(8192) + 1, size=S)
+        mb = -(-n(8192) // 16)
+        return make_page_attention_batch(kv, num_q_heads=32, num_kv_heads=8, head_dim=128, block_size=16, max_blocks=mb,
+                                         num_blocks=max(S * mb, n(160000)), seed=seed, device=device, dtype=dtype,
+                                         name=name)
+    raise KeyError(name)
+
+
+def page_attention_subset(batch: PageAttnBatch, seq_ids) -> PageAttnBatch:
+    """Sub-batch of ``seq_ids`` with their blocks renumbered densely, on the CPU (for a host-side checker)."""
+    seq_ids = list(seq_ids)
+    bs = batch.key_cache.shape[2]
+    bt = batch.block_tables.cpu().numpy()
+    new_bt = np.zeros((len(seq_ids), bt.shape[1]), np.int32)
+    phys = []
+    for i, s in enumerate(seq_ids):
+        nb = -(-int(batch.kv_lens[s]) // bs)
+        new_bt[i, :nb] = np.arange(len(phys), len(phys) + nb)
+        phys.extend(bt[s, :nb].tolist())
+    phys = phys or [0]
+    idx = torch.tensor(phys, dtype=torch.long, device=batch.key_cache.device)
+    ids = torch.tensor(seq_ids, dtype=torch.long, device=batch.query.device)
+    return PageAttnBatch(query=batch.query[ids].cpu(), key_cache=batch.key_cache[idx].cpu(),
+                         value_cache=batch.value_cache[idx].cpu(),
+                         context_lens=torch.from_numpy(batch.kv_lens[seq_ids].astype(np.int32)),
+                         block_tables=torch.from_numpy(new_bt), attn_scale=batch.attn_scale,
+                         kv_lens=batch.kv_lens[seq_ids], name=batch.name + "/sub", meta=dict(batch.meta, rows=ids.cpu()))
+
+
 def _randn_chunked(shape, gen, device, dtype, chunk_elems=1 << 27):
     """N(0,1) in `dtype`, drawn in fp32 chunks so a large pool never needs 2x its size."""
     out = torch.empty(shape, dtype=dtype, device=device)

@@ -123,6 +123,38 @@ int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
  * the written rows (the reference updates and attends sequence by sequence). */
 int rpa_v3_launch(const RpaV3Params* params, void* hip_stream);
 
+/*
+ * page_attention: one query token per sequence over a key cache and a value cache of
+ * [num_blocks, num_kv_heads, block_size, head_dim].  Replaces the backend entry
+ * ejkernel/kernels/_xla/page_attention/_interface.py:25-115 (program: _xla_impl_fwd.py:22-101), reached from
+ * ejkernel/modules/operations/page_attention.py:364-383.  A key at position k of sequence s is kept iff
+ * k < context_lens[s]; a sequence without keys yields zeros.
+ */
+typedef struct RpaPageAttnParams {
+  const void* query;           /* [num_seqs, num_q_heads, head_dim]                          */
+  const void* key_cache;       /* [num_blocks, num_kv_heads, block_size, head_dim]           */
+  const void* value_cache;     /* [num_blocks, num_kv_heads, block_size, head_dim]           */
+  const int32_t* context_lens; /* [num_seqs]                                                 */
+  const int32_t* block_tables; /* [num_seqs, max_blocks]                                     */
+  void* out;                   /* [num_seqs, num_q_heads, head_dim], dtype of query          */
+  void* workspace;             /* >= rpa_page_attention_workspace_bytes() bytes, cleared once with rpa_workspace_init */
+  uint64_t workspace_bytes;
+  int32_t num_seqs;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t block_size;
+  int32_t num_blocks;
+  int32_t max_blocks;
+  float attn_scale;            /* multiplies q (rounded to the query dtype, as `query * attn_scale` is) */
+  int32_t dtype;               /* RPA_DTYPE_*                                                */
+  int32_t compute;             /* RPA_COMPUTE_*                                              */
+  uint32_t flags;              /* RPA_FLAG_FORCE_GENERIC, RPA_FLAG_FP32_LOGITS               */
+} RpaPageAttnParams;
+
+uint64_t rpa_page_attention_workspace_bytes(const RpaPageAttnParams* dims);
+int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream);
+
 /* Message for the calling thread's most recent failure ("" if none). */
 const char* rpa_last_error(void);
 
