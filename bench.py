@@ -36,9 +36,11 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="decode_llama3_8b")
-    ap.add_argument("--op", default="rpa", choices=["rpa", "rpa_v3"],
+    ap.add_argument("--op", default="rpa", choices=["rpa", "rpa_v3", "page_attention"],
                     help="rpa = ragged_page_attention (the headline path); rpa_v3 = ragged_page_attention_v3 on the same "
-                         "workload: every query token also brings a new K/V row that is written into the cache first")
+                         "workload: every query token also brings a new K/V row that is written into the cache first; "
+                         "page_attention = the decode workloads (decode_small, decode_llama3_8b) with separate K and V "
+                         "caches of [blocks, kv heads, block, head_dim]")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -168,6 +170,82 @@ def cpu_sample_and_parity_v3(batch, v3, out, want_baseline, want_parity, n_seqs,
     return res
 
 
+def page_attention_main(args):
+    """bench.py --op page_attention: the same contract as the default path, for the page_attention operation."""
+    import numpy as np
+    import torch
+
+    from ejkernel_amd.modules import page_attention
+    from ejkernel_amd.roofline import HBM_PEAK_GBPS, algorithmic_counts
+    from ejkernel_amd.workloads import WORKLOADS, page_attention_subset, page_attention_workload
+
+    dev = "cuda:0"
+    b = page_attention_workload(args.workload, device=dev, scale=args.scale)
+    m = b.meta
+    S = len(b.kv_lens)
+    counts = algorithmic_counts(np.ones(S, np.int64), b.kv_lens, num_q_heads=m["num_q_heads"],
+                                num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m["page_size"])
+
+    def step():
+        return page_attention(*b.args(), attn_scale=b.attn_scale)
+
+    for _ in range(args.warmup):
+        out = step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        starts[i].record()
+        out = step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ev_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    kernel_ms = sum(ev_ms) / len(ev_ms)
+    ms_per_step = wall * 1e3 / args.steps
+    gbps = counts["bytes"] / (kernel_ms * 1e-3) / 1e9
+    line = {
+        "metric": "page-attn tokens/s", "value": S / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": args.workload, "op": args.op, "description": WORKLOADS[args.workload], "scale": args.scale,
+                   "query_tokens": S, "num_seqs": S, "kv_tokens": int(b.kv_lens.sum())},
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
+                     "traffic": None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
+                     "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
+                     "algorithmic_flops": counts["flops"], "gbps": gbps},
+    }
+    if not (args.no_cpu_baseline and args.no_parity):
+        from oracle.page_attention_oracle import page_attention_strict
+        from tests.helpers import err_stats, to_np
+
+        try:
+            from threadpoolctl import threadpool_info
+            threads = max([int(i.get("num_threads", 1)) for i in threadpool_info()] or [1])
+        except Exception:  # pragma: no cover
+            threads = 1
+        rng = np.random.default_rng(0)
+        cand = [int(s) for s in rng.permutation(S)]
+        n = args.cpu_seqs or min(S, 48)
+        sub = page_attention_subset(b, sorted(cand[:n]))
+        a = [to_np(t) for t in sub.args()]
+        t0 = time.perf_counter()
+        ref = page_attention_strict(*a, attn_scale=b.attn_scale)
+        dt = time.perf_counter() - t0
+        if not args.no_parity:
+            mx, mean = err_stats(to_np(out[sub.meta["rows"].to(dev)]), ref, n)
+            line["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": n, "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
+        if not args.no_cpu_baseline:
+            line["cpu_baseline"] = {
+                "value": n / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
+                "sample": f"{n} of {S} sequences ({int(sub.kv_lens.sum())} kv tokens), one run of {dt:.2f} s; NumPy "
+                          f"restatement of the reference's XLA program (every block-table entry gathered, one dense bf16 "
+                          f"softmax per sequence), BLAS threads {threads}",
+            }
+    print(json.dumps(line))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -184,6 +262,8 @@ def main():
     _native.load()  # fail loudly before any timing if the HIP library is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
+    if args.op == "page_attention":
+        return page_attention_main(args)
     if args.copy_probe:
         n = args.copy_probe << 20
         src = torch.full((n,), 7, dtype=torch.uint8, device=dev)
