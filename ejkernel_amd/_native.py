@@ -13,7 +13,7 @@ from pathlib import Path
 # RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
-RPA_ABI_VERSION = 2
+RPA_ABI_VERSION = 3
 RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
@@ -28,6 +28,8 @@ EXPORTED_SYMBOLS = (
     "rpa_v3_launch",
     "rpa_page_attention_workspace_bytes",
     "rpa_page_attention_launch",
+    "rpa_ragged_decode_workspace_bytes",
+    "rpa_ragged_decode_launch",
 )
 
 
@@ -67,6 +69,7 @@ class RpaParams(ctypes.Structure):
         ("q_scale", ctypes.c_float),
         ("k_scale", ctypes.c_float),
         ("v_scale", ctypes.c_float),
+        ("kv_start", ctypes.c_void_p),
     ]
 
 
@@ -100,6 +103,32 @@ class RpaPageAttnParams(ctypes.Structure):
         ("num_blocks", ctypes.c_int32),
         ("max_blocks", ctypes.c_int32),
         ("attn_scale", ctypes.c_float),
+        ("dtype", ctypes.c_int32),
+        ("compute", ctypes.c_int32),
+        ("flags", ctypes.c_uint32),
+    ]
+
+
+class RpaRaggedDecodeParams(ctypes.Structure):
+    """Field-for-field image of ``struct RpaRaggedDecodeParams``."""
+
+    _fields_ = [
+        ("query", ctypes.c_void_p),
+        ("key", ctypes.c_void_p),
+        ("value", ctypes.c_void_p),
+        ("sequence_start", ctypes.c_void_p),
+        ("sequence_end", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p),
+        ("workspace_bytes", ctypes.c_uint64),
+        ("batch", ctypes.c_int32),
+        ("num_q_heads", ctypes.c_int32),
+        ("num_kv_heads", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32),
+        ("seq_len", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float),
+        ("logits_soft_cap", ctypes.c_float),
+        ("window_left", ctypes.c_int32),
         ("dtype", ctypes.c_int32),
         ("compute", ctypes.c_int32),
         ("flags", ctypes.c_uint32),
@@ -146,6 +175,10 @@ def load() -> ctypes.CDLL:
     lib.rpa_page_attention_workspace_bytes.argtypes = [ctypes.POINTER(RpaPageAttnParams)]
     lib.rpa_page_attention_launch.restype = ctypes.c_int
     lib.rpa_page_attention_launch.argtypes = [ctypes.POINTER(RpaPageAttnParams), ctypes.c_void_p]
+    lib.rpa_ragged_decode_workspace_bytes.restype = ctypes.c_uint64
+    lib.rpa_ragged_decode_workspace_bytes.argtypes = [ctypes.POINTER(RpaRaggedDecodeParams)]
+    lib.rpa_ragged_decode_launch.restype = ctypes.c_int
+    lib.rpa_ragged_decode_launch.argtypes = [ctypes.POINTER(RpaRaggedDecodeParams), ctypes.c_void_p]
     if lib.rpa_abi_version() != RPA_ABI_VERSION:
         raise NativeLibraryError(
             f"{LIB_PATH} has ABI version {lib.rpa_abi_version()}, this package expects {RPA_ABI_VERSION}: rebuild it"

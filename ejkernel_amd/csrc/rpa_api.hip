@@ -22,7 +22,7 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
-static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_seq = false) {
+static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_seq = false, bool contiguous = false) {
   if (p.total_tokens < 0 || p.num_q_heads <= 0 || p.num_kv_heads <= 0 || p.head_dim <= 0 || p.page_size <= 0 ||
       p.num_pages <= 0 || p.max_num_seqs <= 0 || p.pages_per_seq <= 0 || p.num_sinks < 0)
     return fail(RPA_ERR_INVALID_ARGUMENT, "non-positive dimension in RpaParams");
@@ -38,7 +38,7 @@ static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_s
   if (!(p.q_scale >= 0.f) || !(p.k_scale >= 0.f) || !(p.v_scale >= 0.f))
     return fail(RPA_ERR_INVALID_ARGUMENT, "q_scale / k_scale / v_scale must be positive (0 = absent)");
   if (need_pointers) {
-    if (!p.queries || !p.kv_pages || !p.context_lens || !p.block_tables || !p.out ||
+    if (!p.queries || !p.kv_pages || !p.context_lens || (!contiguous && !p.block_tables) || !p.out ||
         (!one_token_per_seq && (!p.query_start_loc || !p.num_seqs)))
       return fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaParams");
     if (p.num_sinks > 0 && !p.sinks) return fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d but sinks is null", p.num_sinks);
@@ -157,8 +157,65 @@ int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream)
   kv.stride_b = p.head_dim * esize;
   kv.head_b = static_cast<uint32_t>(p.page_size) * kv.stride_b;
   kv.page_b = static_cast<uint64_t>(p.num_kv_heads) * kv.head_b;
+  kv.contiguous = 0;
   if (static_cast<uint64_t>(p.page_size) * p.head_dim * esize > 0xffffffffull)
     return rpa::fail(RPA_ERR_UNSUPPORTED, "a cache block of one head exceeds 4 GiB");
+  return rpa::dispatch(p, kv, page_attention_tiled(p), static_cast<hipStream_t>(hip_stream));
+}
+
+static RpaParams ragged_decode_params(const RpaRaggedDecodeParams& a) {
+  RpaParams p = {};
+  p.queries = a.query;
+  p.kv_pages = a.key;
+  p.context_lens = a.sequence_end;  // the query sits at sequence_end - 1 and sees keys below sequence_end
+  p.kv_start = a.sequence_start;
+  p.block_tables = nullptr;         // contiguous caches: sequence b is "page" b
+  p.query_start_loc = nullptr;
+  p.num_seqs = nullptr;
+  p.out = a.out;
+  p.workspace = a.workspace;
+  p.workspace_bytes = a.workspace_bytes;
+  p.total_tokens = a.batch;
+  p.max_num_seqs = a.batch;
+  p.num_q_heads = a.num_q_heads;
+  p.num_kv_heads = a.num_kv_heads;
+  p.head_dim = a.head_dim;
+  int page = 4;  // a power of two that holds a whole sequence, so the slot inside the "page" is the position
+  while (page < a.seq_len && page < (1 << 30)) page <<= 1;
+  p.page_size = page;
+  p.num_pages = a.batch;
+  p.pages_per_seq = 1;
+  p.softmax_scale = a.softmax_scale;
+  p.logits_soft_cap = a.logits_soft_cap;
+  p.sliding_window = a.window_left >= 0 ? a.window_left + 1 : 0;  // k >= pos - left  <=>  k > pos - (left + 1)
+  p.dtype = a.dtype;
+  p.compute = a.compute;
+  p.flags = a.flags & RPA_FLAG_FORCE_GENERIC;
+  return p;
+}
+
+uint64_t rpa_ragged_decode_workspace_bytes(const RpaRaggedDecodeParams* dims) {
+  if (dims == nullptr || dims->seq_len <= 0) return 0;
+  const RpaParams p = ragged_decode_params(*dims);
+  return rpa_workspace_bytes(&p);
+}
+
+int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stream) {
+  if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
+  if (params->seq_len <= 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "seq_len=%d must be positive", params->seq_len);
+  const RpaParams p = ragged_decode_params(*params);
+  int rc = rpa::validate(p, true, true, true);
+  if (rc != RPA_OK) return rc;
+  if (!params->value || !params->sequence_start)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaRaggedDecodeParams");
+  const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
+  rpa::KvLayout kv;
+  kv.k_base = static_cast<const char*>(params->key);
+  kv.v_base = static_cast<const char*>(params->value);
+  kv.head_b = p.head_dim * esize;
+  kv.stride_b = static_cast<uint32_t>(p.num_kv_heads) * kv.head_b;
+  kv.page_b = static_cast<uint64_t>(params->seq_len) * kv.stride_b;
+  kv.contiguous = 1;
   return rpa::dispatch(p, kv, page_attention_tiled(p), static_cast<hipStream_t>(hip_stream));
 }
 

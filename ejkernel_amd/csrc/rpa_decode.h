@@ -98,7 +98,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
         const int t16 = tile + 16 * u;
-        int page = bt_c[t16 >> a.page_shift];
+        int page = a.kv.contiguous ? s : bt_c[t16 >> a.page_shift];
         page = min(max(page, 0), p.num_pages - 1);
         const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
                             static_cast<uint64_t>(t16 & (p.page_size - 1)) * stride_b;
@@ -119,7 +119,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     for (int u = 0; u < NT; ++u) {
       const int t4c = min(tile + 16 * u + 4 * g, t_last & ~3);
       const int rlim = min(3, t_last - t4c);
-      int page = bt[t4c >> a.page_shift];
+      int page = a.kv.contiguous ? s : bt[t4c >> a.page_shift];
       page = min(max(page, 0), p.num_pages - 1);
       const char* base = kvb + static_cast<uint64_t>(page) * page_b +
                          static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + 16 * i);
@@ -159,7 +159,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     }
     // 4. online softmax; this lane: query row i, tokens tile + 16u + 4g + r
     float sv[NT][4];
-    const bool need_mask = (tile + C::TT > range_hi) || (tile + C::TT - 1 > pos_min) || (W > 0 && tile <= pos_max - W);
+    const bool need_mask = (tile + C::TT > range_hi) || (tile + C::TT - 1 > pos_min) || (W > 0 && tile <= pos_max - W) ||
+                           tile < si.start;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
@@ -177,7 +178,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const int tok = tile + 16 * u + 4 * g + r;
-          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W);
+          const bool keep = tok <= pos_n && tok < range_hi && (W <= 0 || tok > pos_n - W) && tok >= si.start;
           sv[u][r] = keep ? sv[u][r] : -INFINITY;
         }
     }

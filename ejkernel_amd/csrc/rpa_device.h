@@ -68,6 +68,9 @@ __device__ __forceinline__ int seq_count(const RpaParams& p) {
 __device__ __forceinline__ int q_start_of(const RpaParams& p, int s) {
   return p.query_start_loc != nullptr ? p.query_start_loc[s] : s;
 }
+__device__ __forceinline__ int kv_start_of(const RpaParams& p, int s) {
+  return p.kv_start != nullptr ? max(p.kv_start[s], 0) : 0;
+}
 __device__ __forceinline__ int seq_of_row(const RpaParams& p, int nseq, int row) {
   return p.query_start_loc != nullptr ? find_seq(p.query_start_loc, nseq, row) : row;
 }

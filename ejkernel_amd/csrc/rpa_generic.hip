@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
   const int kv_len = p.context_lens[s];
   const int pos = kv_len - q_len + (row - q_start_of(p, s));
   const int hi = min(pos + 1, kv_len);
-  const int lo = p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0;
+  const int lo = max(p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0, kv_start_of(p, s));
 
   const bool t_is_bf16 = sizeof(T) == 2;
   // RPA_FLAG_FP32_LOGITS: q enters the dot product unscaled (divided by q_scale and rounded to the storage type, if
@@ -77,7 +77,7 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
       const int t = t0 + lane;
       const bool valid = t < hi;
       const int tc = valid ? t : hi - 1;
-      const int page = min(max(bt[tc / p.page_size], 0), p.num_pages - 1);
+      const int page = min(max(kvl.contiguous ? s : bt[tc / p.page_size], 0), p.num_pages - 1);
       const size_t k_off = static_cast<size_t>(page) * kvl.page_b + static_cast<size_t>(tc % p.page_size) * kvl.stride_b +
                            static_cast<size_t>(j) * kvl.head_b;  // bytes from the K (or V) base
       const T* __restrict__ kp = reinterpret_cast<const T*>(kvl.k_base + k_off);

@@ -15,6 +15,7 @@ struct KvLayout {
   uint64_t page_b;    // between pages
   uint32_t stride_b;  // between the tokens of a page
   uint32_t head_b;    // between the kv heads of a token
+  int32_t contiguous; // 1: no block table, sequence s is page s (page_b = bytes between sequences, slot = position)
 };
 inline KvLayout interleaved_layout(const RpaParams& p) {
   const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
@@ -24,6 +25,7 @@ inline KvLayout interleaved_layout(const RpaParams& p) {
   l.stride_b = 2u * p.num_kv_heads * p.head_dim * esize;
   l.page_b = static_cast<uint64_t>(p.page_size) * l.stride_b;
   l.head_b = 2u * p.head_dim * esize;
+  l.contiguous = 0;
   return l;
 }
 

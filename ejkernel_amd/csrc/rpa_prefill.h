@@ -71,7 +71,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
   const int wg_pos_min = pos0 + wg_row_lo / G, wg_pos_max = pos0 + (wg_row_hi - 1) / G;
   const int range_hi = min(si.kv_len, wg_pos_max + 1);
-  const int range_lo = (W > 0 ? max(0, wg_pos_min - W + 1) : 0) & ~(C::TK - 1);
+  const int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
   const int t_last = range_hi - 1;
 
   // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
@@ -120,9 +120,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
     act_hi[m] = t_any[m] ? t_pos_hi[m] : -0x7fffffff;
-    act_lo[m] = W > 0 ? t_pos_lo[m] - W - 31 : -0x7fffffff;
+    act_lo[m] = max(W > 0 ? t_pos_lo[m] - W - 31 : -0x7fffffff, si.start - 32);
     nomask_hi[m] = min(t_pos_lo[m] - 31, range_hi - 32);
-    nomask_lo[m] = W > 0 ? t_pos_hi[m] - W : -0x7fffffff;
+    nomask_lo[m] = max(W > 0 ? t_pos_hi[m] - W : -0x7fffffff, si.start - 1);
   }
   const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;  // < w_pos_lo when the wave has no rows
   const int w_pos_lo = pos0 + w_row_lo / G;
@@ -348,7 +348,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
               for (int r = 0; r < 4; ++r) {
                 const int tok = tok0 + 16 * u + r;
-                const bool keep = tok <= pos_n[m] && tok < range_hi && (W <= 0 || tok > pos_n[m] - W);
+                const bool keep = tok <= pos_n[m] && tok < range_hi && (W <= 0 || tok > pos_n[m] - W) && tok >= si.start;
                 sv[u][r] = keep ? sv[u][r] : -INFINITY;
               }
           }

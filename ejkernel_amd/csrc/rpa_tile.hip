@@ -224,7 +224,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         const int row_hi = min(rt * 16 + 16, si.rows);
         const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
         const int range_hi = min(si.kv_len, pos_max + 1);
-        const int range_lo = (p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0) & ~(C::TT - 1);
+        const int range_lo = max(p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0, si.start) & ~(C::TT - 1);
         Part part;
         part.partial = false;
         process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);

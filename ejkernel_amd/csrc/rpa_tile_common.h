@@ -92,6 +92,7 @@ __device__ __forceinline__ int part_slot(int k, int stream_a, const Shares& sh) 
 struct SeqInfo {
   int q0, q_len, kv_len, rows, n_rt;
   int lo_al, hi;  // key range of the whole sequence, start aligned down to the tile
+  int start;      // first key position the sequence may attend to
   bool eligible;  // single row tile with keys: part of the decode stream
 };
 
@@ -104,7 +105,9 @@ __device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
   si.rows = si.q_len > 0 ? si.q_len * G : 0;
   si.n_rt = (si.rows + 15) >> 4;
   const int pos_min = si.kv_len - si.q_len;
+  si.start = kv_start_of(p, s);
   int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
+  lo = max(lo, si.start);
   si.lo_al = lo & ~(TT - 1);
   si.hi = max(si.kv_len, 0);
   si.eligible = si.n_rt == 1 && si.hi > si.lo_al;  // a sequence without keys stays an item: its rows become zero

@@ -3,17 +3,19 @@
 
 from .operations import (
     BaseOperationConfig,
+    FwdParams,
     PageAttention,
     PageAttentionConfig,
+    RaggedDecodeAttention,
+    RaggedDecodeAttentionConfig,
     RaggedPageAttention,
     RaggedPageAttentionConfig,
     RaggedPageAttentionv3,
     RaggedPageAttentionv3Config,
     page_attention,
+    ragged_decode_attention,
     ragged_page_attention,
     ragged_page_attention_v3,
 )
 
-__all__ = ["BaseOperationConfig", "PageAttention", "PageAttentionConfig", "RaggedPageAttention",
-           "RaggedPageAttentionConfig", "RaggedPageAttentionv3", "RaggedPageAttentionv3Config", "page_attention",
-           "ragged_page_attention", "ragged_page_attention_v3"]
+__all__ = ['BaseOperationConfig', 'FwdParams', 'PageAttention', 'PageAttentionConfig', 'RaggedDecodeAttention', 'RaggedDecodeAttentionConfig', 'RaggedPageAttention', 'RaggedPageAttentionConfig', 'RaggedPageAttentionv3', 'RaggedPageAttentionv3Config', 'page_attention', 'ragged_decode_attention', 'ragged_page_attention', 'ragged_page_attention_v3']

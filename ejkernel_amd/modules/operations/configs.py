@@ -78,3 +78,34 @@ class PageAttentionConfig(BaseOperationConfig):
     def validate(self) -> None:
         if self.platform not in _PLATFORMS:
             raise ValueError(f"platform={self.platform!r} must be one of {_PLATFORMS}")
+
+
+@dataclass
+class FwdParams:
+    """Forward block sizes a config may carry (ejkernel/ops/utils/datacarrier.py:58-95); accepted, not used here."""
+
+    blocksize_m: int | None = None
+    blocksize_k: int | None = None
+    blocksize_n: int | None = None
+    q_blocksize: int | None = None
+    kv_blocksize: int | None = None
+    blocksize_heads: int | None = None
+    blocksize_keys: int | None = None
+    num_key_splits: int | None = None
+    num_warps: int | None = None
+    num_stages: int | None = None
+
+
+@dataclass
+class RaggedDecodeAttentionConfig(BaseOperationConfig):
+    """Configuration for ragged decode attention (ejkernel/modules/operations/configs.py:224-239)."""
+
+    fwd_params: FwdParams | None = None
+
+    def __post_init__(self):
+        if isinstance(self.fwd_params, dict):
+            self.fwd_params = FwdParams(**self.fwd_params)
+
+    def validate(self) -> None:
+        if self.platform not in _PLATFORMS:
+            raise ValueError(f"platform={self.platform!r} must be one of {_PLATFORMS}")

@@ -136,7 +136,8 @@ def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tens
 
 
 def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *, softmax_scale,
-            logits_soft_cap, compute_dtype, sliding_window, softmax_aux, cfg, flags: int = 0) -> torch.Tensor:
+            logits_soft_cap, compute_dtype, sliding_window, softmax_aux, cfg, flags: int = 0,
+            kv_start=None) -> torch.Tensor:
     lib = _native.load()
     if not queries.is_cuda:
         raise RuntimeError(
@@ -194,6 +195,9 @@ def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_
     p.num_warps = cfg.num_warps or 0
     p.num_stages = cfg.num_stages or 0
     p.flags = flags
+    if kv_start is not None:  # first visible key per sequence (RpaParams.kv_start); not a parameter of the reference op
+        kv_start = kv_start.to(device=dev, dtype=torch.int32).contiguous()
+        p.kv_start = kv_start.data_ptr()
 
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream
@@ -243,6 +247,7 @@ class RaggedPageAttention:
         *,
         cfg: RaggedPageAttentionConfig,
         _flags: int = 0,
+        _kv_start=None,
     ):
         """Same parameters as the reference's ``run`` (``:225-318``).
 
@@ -258,7 +263,8 @@ class RaggedPageAttention:
                          vmem_limit_bytes=vmem_limit_bytes)
         return _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs,
                        softmax_scale=softmax_scale, logits_soft_cap=logits_soft_cap, compute_dtype=compute_dtype,
-                       sliding_window=sliding_window, softmax_aux=softmax_aux, cfg=cfg, flags=_flags)
+                       sliding_window=sliding_window, softmax_aux=softmax_aux, cfg=cfg, flags=_flags,
+                       kv_start=_kv_start)
 
     def heuristic_cfg(self, inv=None) -> RaggedPageAttentionConfig:
         """Default configuration (``:320-337``)."""

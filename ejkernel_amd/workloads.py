@@ -183,6 +183,64 @@ def page_attention_subset(batch: PageAttnBatch, seq_ids) -> PageAttnBatch:
                          kv_lens=batch.kv_lens[seq_ids], name=batch.name + "/sub", meta=dict(batch.meta, rows=ids.cpu()))
 
 
+@dataclass
+class RaggedDecodeBatch:
+    """Arguments of ``ragged_decode_attention``: one query token per sequence, contiguous K and V."""
+
+    query: torch.Tensor
+    key: torch.Tensor
+    value: torch.Tensor
+    sequence_start: torch.Tensor
+    sequence_end: torch.Tensor
+    softmax_scale: float
+    starts: np.ndarray | None = None
+    ends: np.ndarray | None = None
+    name: str = ""
+    meta: dict = field(default_factory=dict)
+
+    def args(self):
+        return (self.query, self.key, self.value, self.sequence_start, self.sequence_end)
+
+
+def make_ragged_decode_batch(starts, ends, *, seq_len, num_q_heads, num_kv_heads, head_dim, seed=0, device="cpu",
+                             dtype=torch.bfloat16, name="") -> RaggedDecodeBatch:
+    starts = np.asarray(starts, dtype=np.int64)
+    ends = np.asarray(ends, dtype=np.int64)
+    B = len(ends)
+    assert ends.max(initial=0) <= seq_len
+    dev = torch.device(device)
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(int(seed))
+    shape = (B, seq_len, num_kv_heads, head_dim)
+    return RaggedDecodeBatch(
+        query=_randn_chunked((B, num_q_heads, head_dim), gen, dev, dtype), key=_randn_chunked(shape, gen, dev, dtype),
+        value=_randn_chunked(shape, gen, dev, dtype),
+        sequence_start=torch.from_numpy(starts.astype(np.int32)).to(dev),
+        sequence_end=torch.from_numpy(ends.astype(np.int32)).to(dev), softmax_scale=float(head_dim**-0.5),
+        starts=starts, ends=ends, name=name,
+        meta=dict(num_q_heads=num_q_heads, num_kv_heads=num_kv_heads, head_dim=head_dim, seq_len=seq_len, seed=seed))
+
+
+def ragged_decode_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bfloat16) -> RaggedDecodeBatch:
+    """The decode lengths of the named workloads in the contiguous layout (every sequence owns ``seq_len`` slots)."""
+    seed = 1003
+    rng = np.random.Generator(np.random.PCG64(seed))
+
+    def n(x, lo=1):
+        return max(lo, int(round(x * scale)))
+
+    if name == "decode_small":
+        ends = rng.integers(64, 513, size=8)
+        return make_ragged_decode_batch(np.zeros(8, int), ends, seq_len=512, num_q_heads=8, num_kv_heads=2,
+                                        head_dim=128, seed=seed, device=device, dtype=dtype, name=name)
+    if name == "decode_llama3_8b":
+        S = n(256)
+        ends = rng.integers(n(512), n(8192) + 1, size=S)
+        return make_ragged_decode_batch(np.zeros(S, int), ends, seq_len=n(8192), num_q_heads=32, num_kv_heads=8,
+                                        head_dim=128, seed=seed, device=device, dtype=dtype, name=name)
+    raise KeyError(name)
+
+
 def _randn_chunked(shape, gen, device, dtype, chunk_elems=1 << 27):
     """N(0,1) in `dtype`, drawn in fp32 chunks so a large pool never needs 2x its size."""
     out = torch.empty(shape, dtype=dtype, device=device)

@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define RPA_ABI_VERSION 2
+#define RPA_ABI_VERSION 3
 
 /* element type of queries / kv_pages / out */
 #define RPA_DTYPE_BF16 0
@@ -93,6 +93,10 @@ typedef struct RpaParams {
   float q_scale;
   float k_scale;
   float v_scale;
+
+  /* ---- [max_num_seqs] first key position a sequence may attend to (sequence_start of ragged_decode_attention,   */
+  /*      _xla/ragged_decode_attention/_xla_impl_fwd.py:55-58), or NULL for 0.                                   */
+  const int32_t* kv_start;
 } RpaParams;
 
 /*
@@ -154,6 +158,39 @@ typedef struct RpaPageAttnParams {
 
 uint64_t rpa_page_attention_workspace_bytes(const RpaPageAttnParams* dims);
 int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream);
+
+/*
+ * ragged_decode_attention: one query token per sequence over contiguous caches key / value
+ * [batch, seq_len, num_kv_heads, head_dim]; sequence b attends to positions [sequence_start[b], sequence_end[b])
+ * from the query position sequence_end[b] - 1, optionally only to the last window_left + 1 of them.  Replaces the
+ * backend entry ejkernel/kernels/_xla/ragged_decode_attention/_interface.py:26-121 (program:
+ * _xla_impl_fwd.py:25-364), reached from ejkernel/modules/operations/ragged_decode_attention.py.  Attention sinks
+ * (softmax_aux) are not part of this entry point.
+ */
+typedef struct RpaRaggedDecodeParams {
+  const void* query;             /* [batch, num_q_heads, head_dim]                */
+  const void* key;               /* [batch, seq_len, num_kv_heads, head_dim]      */
+  const void* value;             /* [batch, seq_len, num_kv_heads, head_dim]      */
+  const int32_t* sequence_start; /* [batch]                                       */
+  const int32_t* sequence_end;   /* [batch]                                       */
+  void* out;                     /* [batch, num_q_heads, head_dim]                */
+  void* workspace;               /* >= rpa_ragged_decode_workspace_bytes() bytes, cleared once with rpa_workspace_init */
+  uint64_t workspace_bytes;
+  int32_t batch;
+  int32_t num_q_heads;
+  int32_t num_kv_heads;
+  int32_t head_dim;
+  int32_t seq_len;
+  float softmax_scale;
+  float logits_soft_cap;         /* 0 = disabled                                  */
+  int32_t window_left;           /* keys at positions >= query position - window_left are kept; < 0 = no window */
+  int32_t dtype;                 /* RPA_DTYPE_*                                   */
+  int32_t compute;               /* RPA_COMPUTE_*                                 */
+  uint32_t flags;                /* RPA_FLAG_FORCE_GENERIC                        */
+} RpaRaggedDecodeParams;
+
+uint64_t rpa_ragged_decode_workspace_bytes(const RpaRaggedDecodeParams* dims);
+int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stream);
 
 /* Message for the calling thread's most recent failure ("" if none). */
 const char* rpa_last_error(void);

@@ -257,8 +257,12 @@ def rpa_exact(
     sliding_window=None,
     softmax_aux=None,
     dtype=np.float64,
+    kv_start=None,
 ):
     """Dense per-sequence evaluation of the intended semantics in ``dtype`` (float64).
+
+    ``kv_start`` (optional, one entry per sequence) drops the keys before that position: the extension of the
+    operation that ragged_decode_attention's ``sequence_start`` needs; the reference operation has no such input.
 
     Follows ``ref_ragged_page_attention`` (_pallas_impl_fwd.py:62-121): gather the
     sequence's pages, split K/V by even/odd combined head, repeat KV heads over the
@@ -302,6 +306,8 @@ def rpa_exact(
         keep = k_pos[None, :] <= q_pos[:, None]
         if sliding_window is not None:
             keep &= k_pos[None, :] > (q_pos[:, None] - int(sliding_window))
+        if kv_start is not None:
+            keep &= (k_pos >= int(kv_start[s]))[None, :]
         logits = np.where(keep[None, None], logits, -np.inf)
         m = logits.max(axis=3)  # [j,g,q]
         if sinks is not None:

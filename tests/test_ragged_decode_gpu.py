@@ -1,0 +1,113 @@
+"""ragged_decode_attention on the device (through ``rpa_ragged_decode_launch``) against its CPU oracle.
+
+Where the reference's XLA program is attention -- sequences inside one KV block whose first block has a visible
+key -- bf16 outputs are within max-abs 2e-2 / mean-abs 2e-3 of its op-by-op restatement.  Everywhere (several
+blocks, starts past the first block, windows: the program is off or NaN there) they are held to the same bound
+against the float64 dense evaluation.  float32 inputs: <= 1e-5 against float64.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from ejkernel_amd import _native
+from ejkernel_amd.modules import RaggedDecodeAttentionConfig, ragged_decode_attention
+from ejkernel_amd.workloads import make_ragged_decode_batch, ragged_decode_workload
+from oracle.ragged_decode_oracle import ragged_decode_exact, ragged_decode_strict
+from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, to_np
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PATHS = [pytest.param(0, id="tiled"), pytest.param(_native.RPA_FLAG_FORCE_GENERIC, id="generic")]
+
+
+def small(starts, ends, **kw):
+    args = dict(seq_len=320, num_q_heads=8, num_kv_heads=2, head_dim=128, seed=13, device=DEV)
+    args.update(kw)
+    return make_ragged_decode_batch(starts, ends, **args)
+
+
+def np_args(b):
+    return [to_np(t) for t in b.args()]
+
+
+def run_hip(b, flags=0, **kw):
+    out = ragged_decode_attention(*b.args(), softmax_scale=b.softmax_scale, _flags=flags, **kw)
+    torch.cuda.synchronize()
+    return to_np(out)
+
+
+ENDS = [1, 15, 16, 17, 100, 255, 256, 300, 64]
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("kw", [dict(), dict(num_q_heads=8, num_kv_heads=8), dict(num_q_heads=32, num_kv_heads=1),
+                                dict(head_dim=256, num_q_heads=16, num_kv_heads=8), dict(head_dim=64), dict(seq_len=301)],
+                         ids=["gqa4", "mha", "mqa32", "d256", "d64", "odd_seq_len"])
+def test_bf16_against_the_reference_program_on_one_block(kw, flags):
+    b = small(np.zeros(len(ENDS), int), ENDS, **kw)
+    ref = ragged_decode_strict(*np_args(b), softmax_scale=b.softmax_scale, block_size=512)
+    assert_bf16_parity(run_hip(b, flags), ref, len(ENDS), str(kw))
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("window,cap", [(None, None), ((40, 0), None), ((7, 3), None), (None, 20.0), ((100, 0), 5.0)])
+def test_bf16_starts_windows_and_caps_against_float64(flags, window, cap):
+    starts = [0, 3, 16, 0, 99, 200, 31, 290, 64]       # the last one is empty (start == end)
+    b = small(starts, ENDS[:-1] + [64])
+    b.sequence_start[:] = torch.tensor(np.minimum(starts, b.ends), dtype=torch.int32)
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=window, logits_soft_cap=cap)
+    out = run_hip(b, flags, sliding_window=window, logits_soft_cap=cap)
+    assert_bf16_parity(out, ref, len(ENDS), f"window {window} cap {cap}")
+    assert not out[8].any()                           # nothing visible: zeros
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_float32_against_float64(flags):
+    b = small([0, 5, 100, 0], [300, 64, 101, 17], dtype=torch.float32)
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=(150, 0))
+    mx, _ = err_stats(run_hip(b, flags, sliding_window=(150, 0)), ref, 4)
+    assert mx <= F32_MAX_ABS, mx
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_single_visible_key_is_bit_exact(flags):
+    b = small([9, 0, 255], [10, 1, 256])
+    out = ragged_decode_attention(*b.args(), softmax_scale=0.1, _flags=flags)
+    for s, pos in enumerate([9, 0, 255]):
+        assert torch.equal(out[s], b.value[s, pos].repeat_interleave(4, dim=0))
+    out = ragged_decode_attention(*small([0, 0], [200, 33]).args(), sliding_window=(0, 0), _flags=flags)
+    b2 = small([0, 0], [200, 33])
+    assert torch.equal(out[0], b2.value[0, 199].repeat_interleave(4, dim=0))
+    assert torch.equal(out[1], b2.value[1, 32].repeat_interleave(4, dim=0))
+
+
+def test_query_with_a_singleton_axis_and_rejected_arguments():
+    b = small([0, 4], [50, 20])
+    out = ragged_decode_attention(*b.args())
+    out4 = ragged_decode_attention(b.query[:, None], *b.args()[1:])
+    assert out4.shape == (2, 1, 8, 128) and torch.equal(out4[:, 0], out)
+    with pytest.raises(NotImplementedError, match="softmax_aux"):
+        ragged_decode_attention(*b.args(), torch.zeros(4, device=DEV))
+    with pytest.raises(ValueError):
+        ragged_decode_attention(*b.args(), sliding_window=(-1, 0))
+    with pytest.raises(ValueError):
+        ragged_decode_attention(*b.args()[:4], b.sequence_end.long())
+    with pytest.raises(ValueError):
+        ragged_decode_attention(*b.args(), cfg=RaggedDecodeAttentionConfig(platform="tpu"))
+    with pytest.raises(NotImplementedError):
+        ragged_decode_attention(*b.args(), mesh=object())
+
+
+@pytest.mark.parametrize("name,n_sample", [("decode_small", 8), ("decode_llama3_8b", 10)])
+def test_full_size_workload(name, n_sample):
+    b = ragged_decode_workload(name, device=DEV)
+    out = ragged_decode_attention(*b.args(), softmax_scale=b.softmax_scale)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out, ragged_decode_attention(*b.args(), softmax_scale=b.softmax_scale))
+    rng = np.random.default_rng(0)
+    ids = torch.tensor(sorted(int(s) for s in rng.permutation(len(b.ends))[:n_sample]))
+    sub = [to_np(t[ids.to(DEV)]) for t in b.args()]
+    ref = ragged_decode_exact(*sub, softmax_scale=b.softmax_scale)
+    assert_bf16_parity(to_np(out[ids.to(DEV)]), ref, len(ids), name)

@@ -150,6 +150,25 @@ def test_bf16_prefill_tiles_over_many_key_tiles(flags, hq, hkv, D, window):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("window", [None, 48])
+def test_bf16_first_visible_key_per_sequence(flags, window):
+    """``RpaParams.kv_start`` (what ragged_decode_attention's ``sequence_start`` maps to) on every kind of work item:
+    decode stream, few-row items and prefill tiles, with starts inside, at the edge of and past the visible range."""
+    b = small([200, 1, 70, 130, 3, 1, 40], [200, 300, 100, 400, 90, 64, 40], pages_per_seq=32, sliding_window=window)
+    starts = np.array([37, 250, 0, 399, 88, 64, 16], np.int32)   # 64 of 64: nothing visible for that sequence
+    aux = torch.as_tensor(starts, device=DEV)
+    out = RaggedPageAttention().run(*b.args(), softmax_scale=b.softmax_scale, sliding_window=b.sliding_window,
+                                    cfg=RaggedPageAttentionConfig(), _flags=flags, _kv_start=aux)
+    torch.cuda.synchronize()
+    from oracle import rpa_oracle
+    from tests.helpers import oracle_args
+
+    ref = rpa_oracle.rpa_exact(*oracle_args(b), softmax_scale=b.softmax_scale, sliding_window=b.sliding_window,
+                               kv_start=starts)
+    assert_bf16_parity(to_np(out), ref, b.total_valid_tokens, f"kv_start W={window}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
 def test_bf16_ragged_edge_cases(flags):
     """Empty sequences, kv_len not a page multiple, padding entries, garbage beyond the pages in use."""
     q_lens = [0, 1, 7, 0, 64, 1, 3, 130]
