@@ -36,11 +36,12 @@ def parse():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="decode_llama3_8b")
-    ap.add_argument("--op", default="rpa", choices=["rpa", "rpa_v3", "page_attention"],
+    ap.add_argument("--op", default="rpa", choices=["rpa", "rpa_v3", "page_attention", "ragged_decode"],
                     help="rpa = ragged_page_attention (the headline path); rpa_v3 = ragged_page_attention_v3 on the same "
                          "workload: every query token also brings a new K/V row that is written into the cache first; "
                          "page_attention = the decode workloads (decode_small, decode_llama3_8b) with separate K and V "
-                         "caches of [blocks, kv heads, block, head_dim]")
+                         "caches of [blocks, kv heads, block, head_dim]; ragged_decode = ragged_decode_attention on the "
+                         "same lengths with contiguous K and V of [batch, seq_len, kv heads, head_dim]")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -175,18 +176,26 @@ def page_attention_main(args):
     import numpy as np
     import torch
 
-    from ejkernel_amd.modules import page_attention
+    from ejkernel_amd.modules import page_attention, ragged_decode_attention
     from ejkernel_amd.roofline import HBM_PEAK_GBPS, algorithmic_counts
-    from ejkernel_amd.workloads import WORKLOADS, page_attention_subset, page_attention_workload
+    from ejkernel_amd.workloads import (WORKLOADS, page_attention_subset, page_attention_workload,
+                                        ragged_decode_workload)
 
     dev = "cuda:0"
-    b = page_attention_workload(args.workload, device=dev, scale=args.scale)
+    contiguous = args.op == "ragged_decode"
+    if contiguous:
+        b = ragged_decode_workload(args.workload, device=dev, scale=args.scale)
+        b.kv_lens = b.ends - b.starts
+    else:
+        b = page_attention_workload(args.workload, device=dev, scale=args.scale)
     m = b.meta
     S = len(b.kv_lens)
     counts = algorithmic_counts(np.ones(S, np.int64), b.kv_lens, num_q_heads=m["num_q_heads"],
-                                num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m["page_size"])
+                                num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m.get("page_size", 16))
 
     def step():
+        if contiguous:
+            return ragged_decode_attention(*b.args(), softmax_scale=b.softmax_scale)
         return page_attention(*b.args(), attn_scale=b.attn_scale)
 
     for _ in range(args.warmup):
@@ -206,7 +215,7 @@ def page_attention_main(args):
     ms_per_step = wall * 1e3 / args.steps
     gbps = counts["bytes"] / (kernel_ms * 1e-3) / 1e9
     line = {
-        "metric": "page-attn tokens/s", "value": S / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
+        "metric": "ragged-decode-attn tokens/s" if contiguous else "page-attn tokens/s", "value": S / (ms_per_step * 1e-3), "unit": "tokens/s", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "op": args.op, "description": WORKLOADS[args.workload], "scale": args.scale,
@@ -228,20 +237,35 @@ def page_attention_main(args):
         rng = np.random.default_rng(0)
         cand = [int(s) for s in rng.permutation(S)]
         n = args.cpu_seqs or min(S, 48)
-        sub = page_attention_subset(b, sorted(cand[:n]))
-        a = [to_np(t) for t in sub.args()]
-        t0 = time.perf_counter()
-        ref = page_attention_strict(*a, attn_scale=b.attn_scale)
-        dt = time.perf_counter() - t0
+        if contiguous:
+            # The reference program is attention only for sequences inside one KV block, so it is timed and used as the
+            # checker with a block that covers the sequence (fwd_params.kv_blocksize >= seq_len).
+            from oracle.ragged_decode_oracle import ragged_decode_strict
+
+            ids = torch.tensor(sorted(cand[:n]))
+            a = [to_np(t[ids.to(dev)]) for t in b.args()]
+            t0 = time.perf_counter()
+            ref = ragged_decode_strict(*a, softmax_scale=b.softmax_scale, block_size=int(m["seq_len"]))
+            dt = time.perf_counter() - t0
+            rows_idx, kv_tokens = ids, int(b.kv_lens[ids.numpy()].sum())
+            what = ("NumPy restatement of the reference's XLA scan with one KV block per sequence (bf16 op by op)")
+        else:
+            sub = page_attention_subset(b, sorted(cand[:n]))
+            a = [to_np(t) for t in sub.args()]
+            t0 = time.perf_counter()
+            ref = page_attention_strict(*a, attn_scale=b.attn_scale)
+            dt = time.perf_counter() - t0
+            rows_idx, kv_tokens = sub.meta["rows"], int(sub.kv_lens.sum())
+            what = ("NumPy restatement of the reference's XLA program (every block-table entry gathered, one dense bf16 "
+                    "softmax per sequence)")
         if not args.no_parity:
-            mx, mean = err_stats(to_np(out[sub.meta["rows"].to(dev)]), ref, n)
+            mx, mean = err_stats(to_np(out[rows_idx.to(dev)]), ref, n)
             line["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": n, "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
         if not args.no_cpu_baseline:
             line["cpu_baseline"] = {
                 "value": n / dt, "unit": "tokens/s", "cores": int(threads), "kind": "port",
-                "sample": f"{n} of {S} sequences ({int(sub.kv_lens.sum())} kv tokens), one run of {dt:.2f} s; NumPy "
-                          f"restatement of the reference's XLA program (every block-table entry gathered, one dense bf16 "
-                          f"softmax per sequence), BLAS threads {threads}",
+                "sample": f"{n} of {S} sequences ({kv_tokens} kv tokens), one run of {dt:.2f} s; {what}, BLAS threads "
+                          f"{threads}",
             }
     print(json.dumps(line))
 
@@ -262,7 +286,7 @@ def main():
     _native.load()  # fail loudly before any timing if the HIP library is missing
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = "cuda:0"
-    if args.op == "page_attention":
+    if args.op in ("page_attention", "ragged_decode"):
         return page_attention_main(args)
     if args.copy_probe:
         n = args.copy_probe << 20
