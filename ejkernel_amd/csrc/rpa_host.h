@@ -35,7 +35,13 @@ int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream);
 int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream);
 
 // Tiled MFMA path (bf16, head_dim 128 or 256, page_size a multiple of 4).
-constexpr int kTiledMaxSeqs = 1024;        // schedule arrays live in LDS
+constexpr int kTiledMaxSeqs = 1024;        // entries of a schedule array in LDS; larger batches keep every 2nd, 4th, ...
+constexpr int kTiledMaxSchedShift = 4;     // sequence's start there: up to 16384 sequences
+inline int sched_shift_for(int max_num_seqs) {
+  int k = 0;
+  while (((max_num_seqs + (1 << k) - 1) >> k) > kTiledMaxSeqs) ++k;
+  return k;
+}
 constexpr int kTiledMaxWgsPerCu = 4;        // persistent grid = compute units x this, at most
 
 constexpr uint64_t kWorkspaceTicketBytes = 1u << 20;  // head of the workspace, cleared by rpa_workspace_init

@@ -48,11 +48,15 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   const RpaParams& p = a.p;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int G = p.num_q_heads / p.num_kv_heads;
-  int* item_start = reinterpret_cast<int*>(smem);            // wave-level items
-  int* tile_start = item_start + (p.max_num_seqs + 1);       // decode stream tiles
-  int* wg_start = tile_start + (p.max_num_seqs + 1);         // workgroup-level prefill tiles
-  int* scratch = wg_start + (p.max_num_seqs + 1);
-  char* lds_data = smem + sched_bytes(p.max_num_seqs);
+  // Schedule arrays: exclusive prefix sums over the sequences, kept for every K-th sequence (K = 1 for batches of up
+  // to kTiledMaxSeqs sequences); the sequences in between are walked when an entry is looked up.
+  const int shift = a.sched_shift, K = 1 << shift;
+  const int sched_n = (p.max_num_seqs + K - 1) >> shift;
+  int* item_start = reinterpret_cast<int*>(smem);   // wave-level items
+  int* tile_start = item_start + (sched_n + 1);     // decode stream tiles
+  int* wg_start = tile_start + (sched_n + 1);       // workgroup-level prefill tiles
+  int* scratch = wg_start + (sched_n + 1);
+  char* lds_data = smem + sched_bytes(sched_n);
   char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
   const int nseq = seq_count(p);
@@ -65,7 +69,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     else if (si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
     else items = p.num_kv_heads * si.n_rt;
   };
-  const int per = (nseq + kWgThreads - 1) / kWgThreads;
+  const int per = (((nseq + kWgThreads - 1) / kWgThreads + K - 1) >> shift) << shift;  // a multiple of K per thread
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
   int my_items = 0, my_tiles = 0, my_wg = 0;
   for (int s = s_begin; s < s_end; ++s) {
@@ -82,9 +86,11 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
     classify(seq_info<C::TT>(p, s, G), t, it, wg);
-    item_start[s] = item_base;
-    tile_start[s] = tile_base;
-    wg_start[s] = wg_base;
+    if ((s & (K - 1)) == 0) {
+      item_start[s >> shift] = item_base;
+      tile_start[s >> shift] = tile_base;
+      wg_start[s >> shift] = wg_base;
+    }
     item_base += it;
     tile_base += t;
     wg_base += wg;
@@ -92,10 +98,11 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   total_items = __builtin_amdgcn_readfirstlane(total_items);
   total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
   total_wg = __builtin_amdgcn_readfirstlane(total_wg);
+  const int nc = (nseq + K - 1) >> shift;  // entries in use
   if (tid == 0) {
-    item_start[nseq] = total_items;
-    tile_start[nseq] = total_tiles;
-    wg_start[nseq] = total_wg;
+    item_start[nc] = total_items;
+    tile_start[nc] = total_tiles;
+    wg_start[nc] = total_wg;
   }
   __syncthreads();
 
@@ -115,13 +122,28 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   if (static_cast<int>(blockIdx.x) >= grid_wgs) return;
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
-  auto find = [&](const int* start, int x) {
-    int lo = 0, hi = nseq;
+  // `kind` says which count the array sums (0 items, 1 stream tiles, 2 prefill tiles); `base` receives start[s].
+  auto find = [&](const int* start, int kind, int x, int& base) {
+    int lo = 0, hi = nc;
     while (hi - lo > 1) {
       const int mid = (lo + hi) >> 1;
       if (start[mid] <= x) lo = mid; else hi = mid;
     }
-    return __builtin_amdgcn_readfirstlane(lo);
+    lo = __builtin_amdgcn_readfirstlane(lo);
+    int s = lo << shift;
+    int b = __builtin_amdgcn_readfirstlane(start[lo]);
+    if (shift > 0) {
+      const int s_last = min(s + K, nseq) - 1;
+      for (; s < s_last; ++s) {
+        int t, it, wg;
+        classify(seq_info<C::TT>(p, s, G), t, it, wg);
+        const int cnt = __builtin_amdgcn_readfirstlane(kind == 0 ? it : kind == 1 ? t : wg);
+        if (x < b + cnt) break;
+        b += cnt;
+      }
+    }
+    base = b;
+    return s;
   };
 
   // Prefill tiles are compute-bound and the decode stream is bandwidth-bound, and one workgroup per compute unit
@@ -180,10 +202,11 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
             ++probe;
           }
           if (w < 0) break;
-          const int s = find(wg_start, w);
+          int s_base;
+          const int s = find(wg_start, 2, w, s_base);
           const SeqInfo si = seq_info<C::TT>(p, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
-          const int local = w - __builtin_amdgcn_readfirstlane(wg_start[s]);
+          const int local = w - s_base;
           const int j = local / n_qt, member = local - j * n_qt;
           prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, n_qt - 1 - member);
         }
@@ -199,10 +222,10 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         const int n_xcd = gridDim.x % 8 == 0 ? 8 : 1;
         const int vwg = (blockIdx.x % n_xcd) * (gridDim.x / n_xcd) + blockIdx.x / n_xcd;
         for (int w = vwg; w < total_wg; w += gridDim.x) {
-          const int s = find(wg_start, w);
+          int base;
+          const int s = find(wg_start, 2, w, base);
           const SeqInfo si = seq_info<C::TT>(p, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
-          const int base = __builtin_amdgcn_readfirstlane(wg_start[s]);
           const int local = w - base;
           const int j = local / n_qt, member = local - j * n_qt;
           const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
@@ -217,9 +240,10 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     } else if (do_stream) {
       // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
       for (int w = worker; w < total_items; w += n_workers) {
-        const int s = find(item_start, w);
+        int s_base;
+        const int s = find(item_start, 0, w, s_base);
         const SeqInfo si = seq_info<C::TT>(p, s, G);
-        const int local = __builtin_amdgcn_readfirstlane(w - item_start[s]);
+        const int local = w - s_base;
         const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
         const int row_hi = min(rt * 16 + 16, si.rows);
         const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
@@ -245,10 +269,11 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         int x = sh.begin(worker);
         const int x_end = sh.begin(worker + 1);
         while (x < x_end) {
-          const int s = find(tile_start, x);
+          int s_base;
+          const int s = find(tile_start, 1, x, s_base);
           const SeqInfo si = seq_info<C::TT>(p, s, G);
           const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
-          const int local = __builtin_amdgcn_readfirstlane(x - tile_start[s]);
+          const int local = x - s_base;
           const int j = local / per_head, t0 = local - j * per_head;
           const int t1 = min(per_head, t0 + (x_end - x));
           Part part;
@@ -286,7 +311,7 @@ bool tiled_supported(const RpaParams& p) {
   if (p.dtype != RPA_DTYPE_BF16 || p.compute != RPA_COMPUTE_BF16) return false;
   if (p.head_dim != 128 && p.head_dim != 256) return false;
   if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
-  if (p.max_num_seqs > kTiledMaxSeqs) return false;
+  if (p.max_num_seqs > (kTiledMaxSeqs << kTiledMaxSchedShift)) return false;
   if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kQueueCounterIndex * 4ull) return false;
   return true;
 }
@@ -308,7 +333,7 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
   const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE, static_cast<size_t>(PC::LDS));
-  const size_t lds = sched_bytes(a.p.max_num_seqs) + data;
+  const size_t lds = sched_bytes((a.p.max_num_seqs + (1 << a.sched_shift) - 1) >> a.sched_shift) + data;
   // More than 64 KiB of dynamic LDS has to be allowed once per kernel (and device); the call is idempotent.
   static std::atomic<uint64_t> allowed[64];
   int dev = 0;
@@ -330,6 +355,7 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   TileArgs a;
   a.p = p;
   a.kv = kv;
+  a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);

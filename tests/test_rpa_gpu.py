@@ -168,6 +168,28 @@ def test_bf16_first_visible_key_per_sequence(flags, window):
     assert_bf16_parity(to_np(out), ref, b.total_valid_tokens, f"kv_start W={window}")
 
 
+@pytest.mark.parametrize("n_seqs,max_seqs", [(1500, 1500), (3000, 4096), (1025, 16384)])
+def test_bf16_batches_of_more_than_1024_sequences(n_seqs, max_seqs):
+    """Above 1024 sequences the schedule arrays keep every 2nd / 4th / 16th sequence's start: decode sequences, a few
+    prefill chunks and empty sequences spread over the batch must all be found."""
+    from oracle import rpa_oracle_c
+    from tests.helpers import oracle_args
+
+    rng = np.random.default_rng(n_seqs)
+    q_lens = np.ones(n_seqs, int)
+    kv_lens = rng.integers(1, 200, size=n_seqs)
+    for s in rng.choice(n_seqs, size=12, replace=False):
+        q_lens[s] = int(rng.integers(20, 90))
+        kv_lens[s] = q_lens[s] + int(rng.integers(0, 100))
+    for s in rng.choice(n_seqs, size=40, replace=False):
+        q_lens[s] = 0
+    b = small(q_lens, kv_lens, max_num_seqs=max_seqs, pages_per_seq=13)
+    out = to_np(run_hip(b))
+    ref = rpa_oracle_c.rpa_strict_c(*oracle_args(b), softmax_scale=b.softmax_scale)
+    assert_bf16_parity(out, ref, b.total_valid_tokens, f"{n_seqs} sequences")
+    assert not out[b.total_valid_tokens:].any()
+
+
 @pytest.mark.parametrize("flags", PATHS)
 def test_bf16_ragged_edge_cases(flags):
     """Empty sequences, kv_len not a page multiple, padding entries, garbage beyond the pages in use."""
