@@ -284,13 +284,22 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     ticket = __shfl(ticket, 0, kWave);
     if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    // The parts are read kMergeChunk at a time: all loads of a chunk are issued before the first is used, so the
+    // merge costs one memory latency per chunk instead of two per part.
+    constexpr int kMergeChunk = C::NS == 1 ? 4 : 1;
     const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
     float M = -INFINITY;
     if (row_valid)
-      for (int k = part.first_w; k <= part.last_w; ++k) {
-        const size_t sl = part_slot(k, part.stream_a, part.sh);
-        const uint64_t v = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v)));
+      for (int k0 = part.first_w; k0 <= part.last_w; k0 += 2 * kMergeChunk) {
+        uint64_t v[2 * kMergeChunk];
+#pragma unroll
+        for (int c = 0; c < 2 * kMergeChunk; ++c) {
+          const int k = min(k0 + c, part.last_w);
+          v[c] = __hip_atomic_load(ml + static_cast<size_t>(part_slot(k, part.stream_a, part.sh)) * 16, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int c = 0; c < 2 * kMergeChunk; ++c) M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v[c])));
       }
     const float M_use = M == -INFINITY ? 0.f : M;
     float L = 0.f;
@@ -299,24 +308,40 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
     if (row_valid) {
-      for (int k = part.first_w; k <= part.last_w; ++k) {
-        const size_t sl = part_slot(k, part.stream_a, part.sh);
-        const uint64_t mlv = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const float mk = __uint_as_float(static_cast<uint32_t>(mlv)), lk = __uint_as_float(static_cast<uint32_t>(mlv >> 32));
-        const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
-        L += w * lk;
-        const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
+      for (int k0 = part.first_w; k0 <= part.last_w; k0 += kMergeChunk) {
+        uint64_t mlv[kMergeChunk];
+        uint64_t ov[kMergeChunk][C::NS][4][4];
 #pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN)
+        for (int c = 0; c < kMergeChunk; ++c) {
+          const size_t sl = part_slot(min(k0 + c, part.last_w), part.stream_a, part.sh);
+          mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
 #pragma unroll
-          for (int r = 0; r < 4; ++r)
+          for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const uint64_t v = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
-                                                   __HIP_MEMORY_SCOPE_AGENT);
-              o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(v));
-              o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(v >> 32));
-            }
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                ov[c][sN][r][e] = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
+                                                    __HIP_MEMORY_SCOPE_AGENT);
+        }
+#pragma unroll
+        for (int c = 0; c < kMergeChunk; ++c) {
+          if (k0 + c > part.last_w) break;  // the tail of the last chunk repeats the last part: not added again
+          const float mk = __uint_as_float(static_cast<uint32_t>(mlv[c]));
+          const float lk = __uint_as_float(static_cast<uint32_t>(mlv[c] >> 32));
+          const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
+          L += w * lk;
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e]));
+                o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e] >> 32));
+              }
+        }
       }
     }
     m_run = M;

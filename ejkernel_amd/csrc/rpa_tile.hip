@@ -32,6 +32,7 @@
 namespace rpa {
 
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
+constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
 
 // Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints and 8 ints of scratch, then the data region
@@ -258,13 +259,20 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       if (total_tiles > 0) {
         Shares sh;
         {
-          // Equal shares when there are only a few tiles per wavefront (every non-empty share must stay in front
-          // of every empty one), weighted regions otherwise.
-          const int q = total_tiles / n_workers, rem = total_tiles - q * n_workers, half = n_workers / 2;
-          int first_tiles = half * q + min(half, rem);
-          if (by_xcd && q >= 4)
-            first_tiles = static_cast<int>(static_cast<long long>(total_tiles) * a.even_xcd_permille / 1000);
-          sh.set(total_tiles, n_workers, half, first_tiles);
+          // Weighted regions when every wavefront gets a few tiles at least.  Small batches use fewer wavefronts
+          // instead, kMinShareTiles tiles each: a (sequence, kv head) cut into many one-tile parts would spend its
+          // time in the merge, which reads the parts one after the other.
+          const int q = total_tiles / n_workers, half = n_workers / 2;
+          const int min_share = a.min_share_tiles;
+          if (q >= min_share) {
+            const int rem = total_tiles - q * n_workers;
+            int first_tiles = half * q + min(half, rem);
+            if (by_xcd) first_tiles = static_cast<int>(static_cast<long long>(total_tiles) * a.even_xcd_permille / 1000);
+            sh.set(total_tiles, n_workers, half, first_tiles);
+          } else {
+            const int n_active = max(1, total_tiles / min_share);
+            sh.set(total_tiles, n_active, n_active, total_tiles);  // one evenly cut region; the other wavefronts get nothing
+          }
         }
         int x = sh.begin(worker);
         const int x_end = sh.begin(worker + 1);
@@ -356,6 +364,7 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   a.p = p;
   a.kv = kv;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
+  a.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
