@@ -284,9 +284,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     ticket = __shfl(ticket, 0, kWave);
     if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
-    // The parts are read kMergeChunk at a time: all loads of a chunk are issued before the first is used, so the
+    // The parts are read kMergeChunk at a time (more would take registers from the prefill tile, which shares this
+    // kernel): all loads of a chunk are issued before the first is used, so the
     // merge costs one memory latency per chunk instead of two per part.
-    constexpr int kMergeChunk = C::NS == 1 ? 4 : 1;
+    constexpr int kMergeChunk = C::NS == 1 ? 2 : 1;
     const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
     float M = -INFINITY;
     if (row_valid)
