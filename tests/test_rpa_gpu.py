@@ -303,3 +303,29 @@ def test_non_default_stream():
         out = ragged_page_attention(*b.args(), softmax_scale=b.softmax_scale)
     st.synchronize()
     assert torch.equal(out, base)
+
+
+def test_launch_recorded_in_a_hip_graph_replays_correctly():
+    """The launch only enqueues (no allocation, no synchronisation, tickets and queue counters left at zero), so it can
+    be captured; every replay on new input values must equal the eager result bit for bit."""
+    b = make_workload("mixed_prefill_decode", device=DEV, scale=0.05)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            ragged_page_attention(*b.args(), **b.kwargs())
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = ragged_page_attention(*b.args(), **b.kwargs())
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for rep in range(4):
+        b.queries.copy_(torch.randn(b.queries.shape, generator=gen, device=DEV).to(b.queries.dtype))
+        if rep == 2:  # other K/V values too
+            b.kv_pages.mul_(-1)
+        want = ragged_page_attention(*b.args(), **b.kwargs())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), rep
