@@ -40,7 +40,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const int hg = row_valid ? R - qi * G : 0;
   const int pos_n = row_valid ? si.kv_len - si.q_len + qi : -1;
   const int head = j * G + hg;
-  const size_t q_row_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * D;
+  // head_dim 64 runs on the 128-wide instantiation: q is padded with zeros, the upper eight 16-byte pieces of a K / V
+  // row repeat the lower eight (K: multiplied by zero; V: output elements that are not stored).
+  const int hd = p.head_dim;
+  const size_t q_row_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * hd;
 
   // ---- Q^T operands: lane (row i, group g) holds q[row][32 ks + 8 g .. +8], pre-scaled and rounded to bf16
   bf16x8_t qreg[C::NKS];
@@ -49,7 +52,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (row_valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
+      if (row_valid && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -92,7 +95,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const uint32_t stride_b = a.kv.stride_b;            // bytes between tokens
   const uint64_t page_b = a.kv.page_b;
   const uint32_t head_off = static_cast<uint32_t>(j) * a.kv.head_b;
-  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + static_cast<uint32_t>(16 * i);
+  const int piece = i & (hd / 8 - 1);  // i itself from head_dim 128 up
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + static_cast<uint32_t>(16 * piece);
   auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
     if (a.uniform_page && tile + C::TT <= range_hi) {
 #pragma unroll
@@ -122,7 +126,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       int page = a.kv.contiguous ? s : bt[t4c >> a.page_shift];
       page = min(max(page, 0), p.num_pages - 1);
       const char* base = kvb + static_cast<uint64_t>(page) * page_b +
-                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + 16 * i);
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + 16 * piece);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
@@ -372,7 +376,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       u32x4_t w;
 #pragma unroll
       for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[sN][2 * e][r] * inv, o_acc[sN][2 * e + 1][r] * inv);
-      *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+      if (128 * sN + 32 * g + 8 * r < hd) *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
     }
 }
 

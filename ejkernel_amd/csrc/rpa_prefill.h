@@ -66,6 +66,10 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const float cap = p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
   const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
+  // head_dim 64 runs on the 128-wide instantiation: q is padded with zeros and the upper half of every K / V row in
+  // LDS repeats the lower half (K: multiplied by zero; V: output elements that are not stored).
+  const int hd = p.head_dim;
+  const uint32_t pmask = static_cast<uint32_t>(hd / 8 - 1);  // 16-byte pieces of a row that exist in memory
 
   // ---- key range of the workgroup's rows
   const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
@@ -96,7 +100,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     const int qi = row_valid[m] ? R / G : 0;
     head[m] = j * G + (row_valid[m] ? R - qi * G : 0);
     pos_n[m] = row_valid[m] ? pos0 + qi : -1;
-    q_off[m] = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head[m]) * D;
+    q_off[m] = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head[m]) * hd;
     const int tr_lo = w_row_lo + 16 * m, tr_hi = min(tr_lo + 16, si.rows);
     t_any[m] = tr_hi > tr_lo;
     t_pos_lo[m] = pos0 + tr_lo / G;
@@ -104,7 +108,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (row_valid[m]) raw = *reinterpret_cast<const u32x4_t*>(q + q_off[m] + 32 * ks + 8 * g);
+      if (row_valid[m] && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off[m] + 32 * ks + 8 * g);
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -144,7 +148,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // ---- cooperative fetch.  One wave-wide direct-to-LDS load moves a block of RB rows: the LDS side is 1 KiB in
   // lane order, so lane l fills piece slot l % PR of row l / PR and fetches the piece that the swizzle assigns
   // to that slot.  Block-table entries are scalar loads (the rows of a block always share a page).
-  const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * D) * 2u;
+  const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * hd) * 2u;
   const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
       reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
@@ -153,18 +157,18 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
   // (Without the transposing read the V tile is laid out like the K tile.)
   const int v_row = C::TRV ? (lane >> 1) % C::RB : l_row;
-  const uint32_t v_src = 16u * static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1));  // byte offset in the row
+  const uint32_t v_src = 16u * (static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)) & pmask);  // byte offset in the row
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
   uint32_t pre_off[HB];  // per-lane byte offset of K block n inside the group: row part + swizzled piece
 #pragma unroll
   for (int n = 0; n < HB; ++n) {
     const int t_local = GROUP * wave + C::RB * n + l_row;
-    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
   }
-  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + D * 2;  // V block 0; block n adds RB rows
+  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + hd * 2;  // V block 0; block n adds RB rows
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
-    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + D * 2;
+    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + hd * 2;
   };
   const bool group_in_page = p.page_size >= GROUP;
   auto fetch_tile = [&](int tile, int buf) {
@@ -174,7 +178,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       // the whole group lies in one page and inside the range: one block-table entry, one base address
       const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * D * 2;
+                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
 #pragma unroll
       for (int n = 0; n < HB; ++n) {
         __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n]),
@@ -190,16 +194,16 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
       const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * D * 2;
+                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
       const int tok = min(t_c + l_row, t_last);
       const int t_local = GROUP * wave + C::RB * n + l_row;
-      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
+      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
                                        (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
       const int v_tok = min(t_c + v_row, t_last);
-      const uint32_t v_piece = C::TRV ? v_src : 16u * static_cast<uint32_t>(l_slot ^ (t_local & 15));
+      const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
       __builtin_amdgcn_global_load_lds(
-          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + D * 2),
+          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + hd * 2),
           (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
     }
   };
@@ -468,7 +472,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           u32x2_t w;
           w[0] = pack_bf16x2(o_acc[m][sN][c][0] * inv, o_acc[m][sN][c][1] * inv);
           w[1] = pack_bf16x2(o_acc[m][sN][c][2] * inv, o_acc[m][sN][c][3] * inv);
-          *reinterpret_cast<u32x2_t*>(orow + 128 * sN + 16 * c + 4 * g) = w;
+          if (128 * sN + 16 * c < hd) *reinterpret_cast<u32x2_t*>(orow + 128 * sN + 16 * c + 4 * g) = w;
         }
     } else {
       // MFMA c of a slice holds head_dim elements 8 (4 g + r) + c of this lane's row

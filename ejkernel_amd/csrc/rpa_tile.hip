@@ -110,7 +110,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   // ---- rows past the ragged batch are zero
   {
     const int total_rows = q_start_of(p, nseq);
-    const int row_u4 = p.num_q_heads * D / 8;  // 16-byte pieces per row
+    const int row_u4 = p.num_q_heads * p.head_dim / 8;  // 16-byte pieces per row
     u32x4_t* o4 = static_cast<u32x4_t*>(p.out);
     for (int row = total_rows + blockIdx.x; row < p.total_tokens; row += gridDim.x)
       for (int k = tid; k < row_u4; k += kWgThreads) o4[static_cast<size_t>(row) * row_u4 + k] = u32x4_t{0u, 0u, 0u, 0u};
@@ -317,7 +317,7 @@ static int tiled_grid() {
 bool tiled_supported(const RpaParams& p) {
   if (p.flags & RPA_FLAG_FORCE_GENERIC) return false;
   if (p.dtype != RPA_DTYPE_BF16 || p.compute != RPA_COMPUTE_BF16) return false;
-  if (p.head_dim != 128 && p.head_dim != 256) return false;
+  if (p.head_dim != 64 && p.head_dim != 128 && p.head_dim != 256) return false;  // 64 runs on the 128-wide kernel
   if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
   if (p.max_num_seqs > (kTiledMaxSeqs << kTiledMaxSchedShift)) return false;
   if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kQueueCounterIndex * 4ull) return false;
@@ -330,7 +330,8 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   // partial results where another shape keeps its tickets.
   wl->counters_bytes = kWorkspaceTicketBytes;
   wl->partial_o_off = wl->counters_bytes;
-  wl->partial_o_bytes = (slots * 16 * p.head_dim * 4 + 255) & ~static_cast<uint64_t>(255);
+  const uint64_t tile_d = p.head_dim <= 128 ? 128 : 256;  // width the kernel works in
+  wl->partial_o_bytes = (slots * 16 * tile_d * 4 + 255) & ~static_cast<uint64_t>(255);
   wl->partial_ml_off = wl->partial_o_off + wl->partial_o_bytes;
   wl->partial_ml_bytes = (slots * 16 * 2 * 4 + 255) & ~static_cast<uint64_t>(255);
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
@@ -376,7 +377,7 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
-  if (p.head_dim == 128)
+  if (p.head_dim <= 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);
 }

@@ -138,7 +138,7 @@ def test_bf16_head_dims(flags, D):
 
 
 @pytest.mark.parametrize("flags", PATHS)
-@pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128)])
+@pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128), (8, 2, 64), (4, 4, 64)])
 @pytest.mark.parametrize("window", [None, 48])
 def test_bf16_prefill_tiles_over_many_key_tiles(flags, hq, hkv, D, window):
     """Prefill chunks whose workgroup tiles walk three and more K/V tiles (the LDS stages are refilled while in
