@@ -1,19 +1,25 @@
 // Workgroup-level attention tile for sequences with many rows (prefill chunks).
 //
-// One workgroup (4 wavefronts) owns WGROWS = 4 * 16 * MRT consecutive rows of one sequence and
-// one kv head -- (query token, group head) pairs, so 64 tokens x 4 heads at MRT = 4, G = 4 --
-// and walks the keys those rows can see once.  K and V tiles of TK tokens go from HBM straight
-// into a double-buffered LDS tile with 16-byte direct-to-LDS loads (global_load_lds_dwordx4: no
-// staging registers; 16 consecutive lanes read one contiguous 256-byte row), issued one step
-// ahead: one barrier per step.  Rows are stored unpadded with their 16-byte pieces XOR-swizzled
-// by the row number, which keeps both MFMA operand read patterns free of bank conflicts.  Each
-// wavefront then computes S^T = K Q^T and O^T += V^T P^T for its own 16 * MRT rows: every K and V operand read from LDS feeds MRT MFMAs, Q stays in registers, and
-// each lane owns one row per row tile, so the online softmax is lane-local as in the decode loop.
-// The row sums come from one extra MFMA against a vector of ones (they add exactly the bf16
-// probabilities that enter P V).  Logits stay in fp32 here (the decode loop rounds them to bf16 as
-// the reference does; on prefill tiles that rounding only costs VALU time: measured against the
-// reference restatement the mean error moves from 4e-4 to 5.5e-4 of a 2e-3 budget).  Halves of a step that lie entirely in a wavefront's causal
-// future or left of its window are skipped.
+// One workgroup (4 wavefronts) owns WGROWS = 4 * 16 * MRT consecutive rows of one sequence and one
+// kv head -- (query token, group head) pairs, so 32 tokens x 4 heads at MRT = 2, G = 4 -- and walks
+// the keys those rows can see once.  K and V tiles of TK tokens go from HBM / L2 straight into a
+// double-buffered LDS stage with 16-byte direct-to-LDS loads (global_load_lds_dwordx4: no staging
+// registers), issued one step ahead.  K rows are stored unpadded with their 16-byte pieces
+// XOR-swizzled by the row number (conflict-free ds_read_b128 of the MFMA operand).  The V tile is
+// stored by 32-byte column units, the layout the transposing LDS read (ds_read_b64_tr_b16) turns
+// into V^T operands directly; at head_dim 256, where a wavefront has 16 rows and the tile is
+// LDS-bound, V keeps the row-major layout and is transposed with byte permutes instead.
+// Each wavefront computes S^T = K Q^T and O^T += V^T P^T for its own 16 * MRT rows: every K and V
+// operand read from LDS feeds MRT MFMAs, Q stays in registers, and each lane owns one row per row
+// tile, so the online softmax is lane-local as in the decode loop.  The row sums come from one
+// extra MFMA against a vector of ones (they add exactly the bf16 probabilities that enter P V).
+// Logits stay in fp32 here (the decode loop rounds them to bf16 as the reference does; on prefill
+// tiles that rounding only costs vector instructions: against the reference restatement the mean
+// error moves from 4e-4 to 5.5e-4 of a 2e-3 budget).  The K operands of a half are requested one
+// half ahead and the barrier that publishes the next tile sits before the last P V of a tile, so
+// LDS latency and barrier skew hide behind matrix work.  Halves of a step that lie entirely in a
+// wavefront's causal future, left of its window or before the sequence's first visible key are
+// skipped.
 #pragma once
 
 #include "rpa_tile_common.h"

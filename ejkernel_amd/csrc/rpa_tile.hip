@@ -1,28 +1,29 @@
-// Ragged paged attention on MFMA, one wavefront per work item, one launch per batch.
+// Ragged paged attention on MFMA: one persistent launch per batch, two workgroups per compute unit.
 //
-// Rows of a sequence are its (query token, group head) pairs, handled 16 at a time (one
-// MFMA tile) per kv head.  A decode sequence (1-4 query tokens) has a single row tile.
-// All decode sequences of the batch form one stream of 32-key tiles ordered by
-// (sequence, kv head, position); every wavefront of the grid takes an equal contiguous
-// share of that stream, whatever the individual lengths are.  A wavefront whose share
-// covers only part of a (sequence, kv head) writes its partial (m, l, O) to the workspace
-// and takes a ticket; the last part to arrive merges all parts in stream order, so the
-// result does not depend on timing.  Sequences with more rows (prefill chunks) are
-// handled as (sequence, kv head, row tile) items over the full key range of the tile.
-// Work is discovered on the device from query_start_loc / context_lens / num_seqs; the
-// host never reads them.
+// Rows of a sequence are its (query token, group head) pairs, handled 16 at a time (one MFMA
+// tile) per kv head.  Work is discovered on the device from query_start_loc / context_lens /
+// num_seqs (the host never reads them) and comes in three kinds:
+//   * the decode stream: all sequences with a single row tile form one stream of key tiles
+//     ordered by (sequence, kv head, position); every streaming wavefront takes a contiguous
+//     share of it, whatever the individual lengths are.  A wavefront whose share covers only
+//     part of a (sequence, kv head) writes its partial (m, l, O) to the workspace and takes a
+//     ticket; the last part to arrive merges all parts in stream order, so the result does
+//     not depend on timing (rpa_decode.h);
+//   * wave items: sequences with two to four row tiles, one (sequence, row tile, kv head) per
+//     wavefront over the full key range, through the same loop;
+//   * prefill tiles: sequences with more rows, one workgroup per tile of 64 * MRT rows, K/V
+//     tiles staged through LDS, handed out from per-XCD queues (rpa_prefill.h).
+// In a mixed batch the upper half of the grid streams while the lower half starts on the
+// prefill tiles; a batch without prefill tiles uses one workgroup per compute unit.
 //
-// Per iteration a wavefront streams TT = 16*NT tokens of its kv head: K and V rows are
-// fetched with 16-byte loads in which each quarter-wave reads one whole contiguous row
-// (256 B at head_dim 128), one iteration ahead of their use.  K goes through a
-// wave-private LDS tile to reach the MFMA operand layout; V is transposed in registers
-// (byte permutes).  Scores are S^T = K Q^T, outputs O^T = V^T P^T, so every lane owns one
-// query row: the online-softmax state and the O rescale are lane-local, and the row
-// maximum needs only two cross-lane steps per iteration.
+// Scores are S^T = K Q^T, outputs O^T = V^T P^T, so every lane owns one query row: the
+// online-softmax state and the O rescale are lane-local.
 //
-// Numerics follow ejkernel/kernels/_xla/ragged_page_attention/_xla_impl_fwd.py:49,119-149:
-// q is pre-multiplied by the bf16 scale and rounded to bf16, logits are rounded to bf16,
-// probabilities are bf16, accumulation is fp32.
+// Numerics follow ejkernel/kernels/_xla/ragged_page_attention/_xla_impl_fwd.py:49,119-149
+// (template argument kMimic): q is pre-multiplied by the bf16 scale and rounded to bf16,
+// decode-loop logits are rounded to bf16, probabilities are bf16, accumulation is fp32.
+// With kMimic = false q enters unscaled and the fp32 logits are scaled afterwards
+// (ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:228-262).
 #include "rpa_device.h"
 #include <atomic>
 
