@@ -13,7 +13,7 @@ from pathlib import Path
 # RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
-RPA_ABI_VERSION = 3
+RPA_ABI_VERSION = 4
 RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
@@ -132,7 +132,13 @@ class RpaRaggedDecodeParams(ctypes.Structure):
         ("dtype", ctypes.c_int32),
         ("compute", ctypes.c_int32),
         ("flags", ctypes.c_uint32),
+        ("softmax_aux", ctypes.c_void_p),
+        ("num_sinks", ctypes.c_int32),
+        ("aux_rows", ctypes.c_int32),
     ]
+
+
+RPA_MAX_SINK_KEYS = 64
 
 
 class NativeLibraryError(RuntimeError):

@@ -20,7 +20,7 @@ LIB_DIR = PKG_DIR / "lib"
 LIB_PATH = LIB_DIR / "librpa_mi355x.so"
 OBJ_DIR = PKG_DIR / "build"
 
-SOURCES = ["rpa_api.hip", "rpa_generic.hip", "rpa_kv_update.hip", "rpa_tile.hip"]
+SOURCES = ["rpa_api.hip", "rpa_generic.hip", "rpa_kv_update.hip", "rpa_sink_keys.hip", "rpa_tile.hip"]
 
 # -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32.
 HIPCC_FLAGS = [

@@ -95,7 +95,7 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
 }
 
 namespace rpa {
-static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream);
+static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream, const PreState& pre = PreState());
 }
 
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {
@@ -132,11 +132,8 @@ static RpaParams page_attention_params(const RpaPageAttnParams& a) {
   return p;
 }
 
-// The tiled decode loop handles up to four 16-row tiles per (sequence, kv head); larger query groups would need
-// the prefill tile, which assumes the interleaved cache.
-static bool page_attention_tiled(const RpaParams& p) {
-  return rpa::tiled_supported(p) && p.num_q_heads / p.num_kv_heads <= 64;
-}
+// One query token per sequence: the tiled kernel runs without prefill tiles (which assume the interleaved cache).
+static bool page_attention_tiled(const RpaParams& p) { return rpa::tiled_supported(p); }
 
 uint64_t rpa_page_attention_workspace_bytes(const RpaPageAttnParams* dims) {
   if (dims == nullptr) return 0;
@@ -194,16 +191,33 @@ static RpaParams ragged_decode_params(const RpaRaggedDecodeParams& a) {
   return p;
 }
 
+// With sinks the workspace continues behind the attention kernels' part: the sink keys' attention state per
+// (sequence, query head) and the first position left for the attention kernels per sequence.
+struct SinkWorkspace {
+  uint64_t base, pre_o_off, pre_ml_off, start_off, total;
+};
+static SinkWorkspace sink_workspace(const RpaRaggedDecodeParams& a, const RpaParams& p) {
+  SinkWorkspace w;
+  const uint64_t rows = static_cast<uint64_t>(a.batch) * a.num_q_heads;
+  w.base = (rpa_workspace_bytes(&p) + 255) & ~255ull;
+  w.pre_o_off = w.base;
+  w.pre_ml_off = w.pre_o_off + ((rows * a.head_dim * 4 + 255) & ~255ull);
+  w.start_off = w.pre_ml_off + ((rows * 8 + 255) & ~255ull);
+  w.total = w.start_off + ((static_cast<uint64_t>(a.batch) * 4 + 255) & ~255ull);
+  return w;
+}
+
 uint64_t rpa_ragged_decode_workspace_bytes(const RpaRaggedDecodeParams* dims) {
-  if (dims == nullptr || dims->seq_len <= 0) return 0;
+  if (dims == nullptr || dims->seq_len <= 0 || dims->batch <= 0 || dims->num_q_heads <= 0 || dims->head_dim <= 0) return 0;
   const RpaParams p = ragged_decode_params(*dims);
+  if (dims->num_sinks > 0) return sink_workspace(*dims, p).total;
   return rpa_workspace_bytes(&p);
 }
 
 int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stream) {
   if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
   if (params->seq_len <= 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "seq_len=%d must be positive", params->seq_len);
-  const RpaParams p = ragged_decode_params(*params);
+  RpaParams p = ragged_decode_params(*params);
   int rc = rpa::validate(p, true, true, true);
   if (rc != RPA_OK) return rc;
   if (!params->value || !params->sequence_start)
@@ -216,21 +230,52 @@ int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stre
   kv.stride_b = static_cast<uint32_t>(p.num_kv_heads) * kv.head_b;
   kv.page_b = static_cast<uint64_t>(params->seq_len) * kv.stride_b;
   kv.contiguous = 1;
-  return rpa::dispatch(p, kv, page_attention_tiled(p), static_cast<hipStream_t>(hip_stream));
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const bool tiled = page_attention_tiled(p);
+  if (params->num_sinks == 0) return rpa::dispatch(p, kv, tiled, stream);
+
+  const int G = p.num_q_heads / p.num_kv_heads;
+  if (params->num_sinks < 0 || params->num_sinks > RPA_MAX_SINK_KEYS)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d must lie in [0, %d]", params->num_sinks, RPA_MAX_SINK_KEYS);
+  if (!params->softmax_aux) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d but softmax_aux is null", params->num_sinks);
+  if (params->aux_rows != 1 && params->aux_rows != G)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "aux_rows=%d must be 1 or num_q_heads / num_kv_heads = %d", params->aux_rows, G);
+  const SinkWorkspace w = sink_workspace(*params, p);
+  if (p.workspace == nullptr || p.workspace_bytes < w.total)
+    return rpa::fail(RPA_ERR_WORKSPACE, "workspace of %llu bytes is too small, rpa_ragged_decode_workspace_bytes() asks for %llu",
+                     (unsigned long long)p.workspace_bytes, (unsigned long long)w.total);
+  char* ws = static_cast<char*>(p.workspace);
+  rpa::SinkKeyArgs sk;
+  sk.aux = params->softmax_aux;
+  sk.num_sinks = params->num_sinks;
+  sk.aux_rows = params->aux_rows;
+  sk.seq_len = params->seq_len;
+  sk.pre_o = reinterpret_cast<float*>(ws + w.pre_o_off);
+  sk.pre_ml = reinterpret_cast<float*>(ws + w.pre_ml_off);
+  sk.main_start = reinterpret_cast<int32_t*>(ws + w.start_off);
+  rc = rpa::launch_sink_keys(p, kv, sk, stream);
+  if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
+  if (rc != RPA_OK) return rpa::fail(rc, "sink key launch failed: %s", hipGetErrorString(hipGetLastError()));
+  p.kv_start = sk.main_start;
+  p.workspace_bytes = w.base;
+  rpa::PreState pre;
+  pre.o = sk.pre_o;
+  pre.ml = sk.pre_ml;
+  return rpa::dispatch(p, kv, tiled, stream, pre);
 }
 
 namespace rpa {
-static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream) {
+static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream, const PreState& pre) {
   int rc;
   if (tiled) {
-    rc = rpa::launch_tiled(p, kv, stream);
+    rc = rpa::launch_tiled(p, kv, stream, pre);
     if (rc == RPA_ERR_WORKSPACE)
       return rpa::fail(rc, "workspace of %llu bytes is too small, rpa_workspace_bytes() asks for %llu",
                        (unsigned long long)p.workspace_bytes, (unsigned long long)rpa_workspace_bytes(&p));
     if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
     return RPA_OK;
   }
-  rc = rpa::launch_generic(p, kv, stream);
+  rc = rpa::launch_generic(p, kv, stream, pre);
   if (rc == RPA_ERR_UNSUPPORTED) return rpa::fail(rc, "head_dim=%d exceeds the supported maximum of 512", p.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
   return RPA_OK;

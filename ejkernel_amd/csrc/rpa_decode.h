@@ -15,8 +15,10 @@ struct Cfg {
   static constexpr int LDS_PER_WAVE = TT * ROWB;
 };
 
-// Everything one wavefront needs for one work item.
-template <int D, int NT, bool kMimic>
+// Everything one wavefront needs for one work item.  kWaveOnly: the state in TileArgs::pre, if any, is merged into
+// every row (only in the kernel instantiation without prefill tiles, so that the common one keeps its register
+// allocation).
+template <int D, int NT, bool kMimic, bool kWaveOnly = false>
 __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
                                              int j, int rt, int range_lo, int range_hi, const Part& part) {
   using C = Cfg<D, NT, kMimic>;
@@ -356,6 +358,31 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 
   // ---- normalise (with optional sinks) and store
   if (!row_valid) return;
+  if (kWaveOnly && a.pre.ml != nullptr) {
+    // keys an earlier kernel accumulated for this (token, head): one more part
+    const size_t idx = static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head;
+    const float ms = a.pre.ml[2 * idx], ls = a.pre.ml[2 * idx + 1];
+    const float M = fmaxf(m_run, ms);
+    const float M_use = M == -INFINITY ? 0.f : M;
+    const float w0 = __builtin_amdgcn_exp2f((m_run - M_use) * kLog2e), w1 = __builtin_amdgcn_exp2f((ms - M_use) * kLog2e);
+    const float* po = a.pre.o + idx * hd;
+#pragma unroll
+    for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int d0 = 128 * sN + 32 * g + 8 * r;  // this lane holds d0 .. d0 + 7 of its row in o_acc[sN][0..7][r]
+        if (d0 < hd) {
+          const f32x4_t x0 = *reinterpret_cast<const f32x4_t*>(po + d0), x1 = *reinterpret_cast<const f32x4_t*>(po + d0 + 4);
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            o_acc[sN][c][r] = w0 * o_acc[sN][c][r] + w1 * x0[c];
+            o_acc[sN][c + 4][r] = w0 * o_acc[sN][c + 4][r] + w1 * x1[c];
+          }
+        }
+      }
+    l_run = w0 * l_run + w1 * ls;
+    m_run = M;
+  }
   float num_scale = 1.f, denom = l_run;
   if (p.sinks != nullptr && p.num_sinks > 0) {
     const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;

@@ -15,7 +15,7 @@ namespace rpa {
 constexpr int kMaxElemsPerLane = 8;  // head_dim <= 512
 
 template <typename T, bool kBf16Compute>
-__global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayout kvl) {
+__global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayout kvl, PreState pre) {
   extern __shared__ float q_lds[];  // [head_dim] scaled query row of the current head
   const int row = blockIdx.x;
   const int j = blockIdx.y;
@@ -130,6 +130,19 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
       }
     }
 
+    if (pre.ml != nullptr) {  // keys an earlier kernel accumulated for this (token, head): one more part
+      const size_t idx = static_cast<size_t>(row) * p.num_q_heads + h;
+      const float ms = pre.ml[2 * idx], ls = pre.ml[2 * idx + 1];
+      const float M = fmaxf(m, ms);
+      const float w0 = m == -INFINITY ? 0.f : expf(m - M), w1 = ms == -INFINITY ? 0.f : expf(ms - M);
+#pragma unroll
+      for (int e = 0; e < kMaxElemsPerLane; ++e) {
+        const int d = lane + e * kWave;
+        if (d < D) acc[e] = w0 * acc[e] + w1 * pre.o[idx * D + d];
+      }
+      l = w0 * l + w1 * ls;
+      m = M;
+    }
     float num_scale = 1.f, denom = l;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(h) * p.num_sinks;
@@ -150,18 +163,18 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
   }
 }
 
-int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
+int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
   if (p.head_dim > kMaxElemsPerLane * kWave) return RPA_ERR_UNSUPPORTED;
   if (p.total_tokens == 0) return RPA_OK;
   dim3 grid(p.total_tokens, p.num_kv_heads), block(kWave);
   const size_t lds = static_cast<size_t>(p.head_dim) * sizeof(float);
   const bool bf16c = p.compute == RPA_COMPUTE_BF16;
   if (p.dtype == RPA_DTYPE_BF16) {
-    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, true>), grid, block, lds, stream, p, kv);
-    else hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, false>), grid, block, lds, stream, p, kv);
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, true>), grid, block, lds, stream, p, kv, pre);
+    else hipLaunchKernelGGL((rpa_generic_kernel<bf16_t, false>), grid, block, lds, stream, p, kv, pre);
   } else {
-    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<float, true>), grid, block, lds, stream, p, kv);
-    else hipLaunchKernelGGL((rpa_generic_kernel<float, false>), grid, block, lds, stream, p, kv);
+    if (bf16c) hipLaunchKernelGGL((rpa_generic_kernel<float, true>), grid, block, lds, stream, p, kv, pre);
+    else hipLaunchKernelGGL((rpa_generic_kernel<float, false>), grid, block, lds, stream, p, kv, pre);
   }
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }

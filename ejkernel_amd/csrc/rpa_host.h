@@ -29,8 +29,30 @@ inline KvLayout interleaved_layout(const RpaParams& p) {
   return l;
 }
 
+// Attention state -- row maximum, row sum, unnormalised output -- that an earlier kernel accumulated over keys
+// outside the range the attention kernels walk.  It is merged into a row like one more part of a split key range,
+// before the row is normalised.  Honoured where a sequence has one query token: the wave-level decode loop and the
+// scalar kernel, not the prefill tiles.
+struct PreState {
+  const float* o = nullptr;   // [tokens, num_q_heads, head_dim]
+  const float* ml = nullptr;  // [tokens, num_q_heads, 2]: maximum (-inf if no key), sum
+};
+
+// Sink keys of ragged_decode_attention (_xla_impl_fwd.py:71-75, :98-134): accumulates, per (sequence, query head),
+// the keys at positions [kv_start[s], kv_start[s] + num_sinks) below seq_len into `pre_o` / `pre_ml`, with
+// softmax_aux[row][t] added to the logit of absolute position t < num_sinks, and writes kv_start[s] + num_sinks to
+// `main_start`, the first position left for the attention kernels.
+struct SinkKeyArgs {
+  const float* aux;
+  int32_t num_sinks, aux_rows, seq_len;
+  float* pre_o;
+  float* pre_ml;
+  int32_t* main_start;
+};
+int launch_sink_keys(const RpaParams& p, const KvLayout& kv, const SinkKeyArgs& sk, hipStream_t stream);
+
 // Each returns RPA_OK or a negative RPA_ERR_* code; all of them only enqueue on `stream`.
-int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream);
+int launch_generic(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre = PreState());
 // Writes the new tokens' K/V rows into the paged cache (ragged_page_attention_v3, _kernel.py:207-218).
 int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream);
 
@@ -58,7 +80,7 @@ struct WorkspaceLayout {
 
 bool tiled_supported(const RpaParams& p);
 void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl);
-int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream);
+int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre = PreState());
 
 // Compute units of the current device (cached per device).
 int device_cu_count();

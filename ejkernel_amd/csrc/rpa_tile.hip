@@ -35,6 +35,7 @@ namespace rpa {
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
 constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
+constexpr int kDecodeShapedPadRows = 16; // token rows beyond one per sequence slot that still count as a decode batch
 
 // Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints and 8 ints of scratch, then the data region
 // shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
@@ -42,7 +43,11 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
   return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 8) * sizeof(int) + 15) & ~static_cast<size_t>(15);
 }
 
-template <int D, int NT, int MRT, bool kMimic>
+// kWaveOnly: the prefill tiles are compiled out and sequences with many row tiles run as wave-level items too (right
+// for every batch, slow for long prefill chunks).  That leaves the decode loop a register allocation of its own, about
+// 2 % faster on decode batches, which is why the host picks this instantiation for batches shaped like decode; it is
+// also the one that merges an attention state in a.pre into every row.
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -68,7 +73,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   auto classify = [&](const SeqInfo& si, int& tiles, int& items, int& wg_items) {
     tiles = items = wg_items = 0;
     if (si.eligible) tiles = p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
-    else if (si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
+    else if (!kWaveOnly && si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
     else items = p.num_kv_heads * si.n_rt;
   };
   const int per = (((nseq + kWgThreads - 1) / kWgThreads + K - 1) >> shift) << shift;  // a multiple of K per thread
@@ -175,6 +180,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 #pragma unroll 1
   for (int phase = 0; phase < 2; ++phase) {
     if ((phase == 0) != stream_first) {
+      if constexpr (!kWaveOnly) {
       // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)
       // adjacent in the item order.  Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2:
       // row tiles that share one K/V stream should run at the same time on the same XCD, so that all but the first
@@ -238,7 +244,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
       // workgroup has finished reading them.
       __syncthreads();
-
+      }
     } else if (do_stream) {
       // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
       for (int w = worker; w < total_items; w += n_workers) {
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         const int range_lo = max(p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0, si.start) & ~(C::TT - 1);
         Part part;
         part.partial = false;
-        process_item<D, NT, kMimic>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+        process_item<D, NT, kMimic, kWaveOnly>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
       }
 
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
@@ -292,7 +298,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           part.last_w = sh.owner(part.stream_a + per_head - 1);
           part.partial = part.first_w != part.last_w;
           part.slot = part_slot(worker, part.stream_a, sh);
-          process_item<D, NT, kMimic>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+          process_item<D, NT, kMimic, kWaveOnly>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
           x += t1 - t0;
         }
       }
@@ -338,7 +344,7 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
 }
 
-template <int D, int NT, int MRT, bool kMimic>
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -349,22 +355,23 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
   if (allowed[dev].load(std::memory_order_acquire) < lds) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
       return RPA_ERR_LAUNCH;
     allowed[dev].store(lds, std::memory_order_release);
   }
-  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic>), dim3(grid), dim3(kWgThreads), lds, stream, a);
+  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly>), dim3(grid), dim3(kWgThreads), lds, stream, a);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
-int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
+int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
   WorkspaceLayout wl;
   tiled_workspace_layout(p, &wl);
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
   TileArgs a;
   a.p = p;
   a.kv = kv;
+  a.pre = pre;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
   a.page_shift = __builtin_ctz(p.page_size);
@@ -378,6 +385,15 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream) {
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
+  // Decode-shaped batches -- one query token per sequence by construction, or a token buffer with no more rows than
+  // sequence slots plus the padding such buffers carry -- take the instantiation without prefill tiles.
+  const bool decode_shaped = p.query_start_loc == nullptr || p.total_tokens <= p.max_num_seqs + kDecodeShapedPadRows;
+  const bool wave_only = pre.ml != nullptr || (decode_shaped && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
+  if (wave_only) {
+    if (p.head_dim <= 128)
+      return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);
+    return mimic ? launch_cfg<256, 1, 1, true, true>(a, grid, stream) : launch_cfg<256, 1, 1, false, true>(a, grid, stream);
+  }
   if (p.head_dim <= 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);

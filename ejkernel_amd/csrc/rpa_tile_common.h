@@ -31,6 +31,7 @@ struct TileArgs {
   uint32_t* counters; // split tickets [max_num_seqs * num_kv_heads], then the queue counters; zero between launches
   float* partial_o;   // [2 * wavefronts of the grid][16][D]
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
+  PreState pre;       // state accumulated by an earlier kernel, merged by the wave-level loop (null: none)
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the

@@ -16,8 +16,15 @@ Differences from the reference's XLA program, all in its disfavour: it returns N
 sequence's first KV block holds no visible key, and its block recurrence only equals attention
 for sequences that fit one KV block (``oracle/ragged_decode_oracle.py`` restates both); this
 implementation computes attention in every case and zeros when nothing is visible.
-``softmax_aux`` (attention sinks) raises ``NotImplementedError``, as the reference's Triton
-backend would for options it lacks.
+
+``softmax_aux`` (attention sinks) follows that program too (``_xla_impl_fwd.py:71-75, :98-134``):
+with ``num_sinks`` entries per row, the keys ``[sequence_start[b], sequence_start[b] + num_sinks)``
+are visible whatever ``sequence_end`` and the window say, and a key at absolute position
+``t < num_sinks`` has ``softmax_aux[row, t]`` added to its logit after the soft cap.  A
+one-dimensional ``softmax_aux`` serves every head; a two-dimensional one needs 1 row or
+``num_q_heads // num_kv_heads`` rows (row ``g`` for the ``g``-th query head of every kv head),
+the only shapes the program's broadcast accepts -- any other row count raises ``ValueError`` here,
+where the reference fails while tracing.
 """
 
 from __future__ import annotations
@@ -57,8 +64,28 @@ def _static_validate(query, key, value, sequence_start, sequence_end, sliding_wi
         raise ValueError("logits_soft_cap must not be 0")
 
 
+def _validate_aux(softmax_aux, group: int):
+    """``softmax_aux`` as float32 ``[rows, num_sinks]`` with rows in (1, group) (``_xla_impl_fwd.py:118-134``)."""
+    if softmax_aux.dim() == 1:
+        aux = softmax_aux[None, :]
+    elif softmax_aux.dim() == 2:
+        aux = softmax_aux
+    else:
+        raise ValueError(f"softmax_aux must be [num_sinks] or [rows, num_sinks], got {tuple(softmax_aux.shape)}")
+    if aux.shape[1] == 0:
+        return None
+    if aux.shape[0] not in (1, group):
+        raise ValueError(
+            f"softmax_aux of shape {tuple(softmax_aux.shape)} does not broadcast against the {group} query heads of a "
+            "kv head: it needs 1 row or that many"
+        )
+    if aux.shape[1] > _native.RPA_MAX_SINK_KEYS:
+        raise ValueError(f"softmax_aux has {aux.shape[1]} sinks, at most {_native.RPA_MAX_SINK_KEYS} are supported")
+    return aux.to(torch.float32).contiguous()
+
+
 def _launch(query, key, value, sequence_start, sequence_end, *, softmax_scale, sliding_window, logits_soft_cap, cfg,
-            flags: int = 0):
+            flags: int = 0, softmax_aux=None):
     lib = _native.load()
     if not query.is_cuda:
         raise RuntimeError(
@@ -87,6 +114,13 @@ def _launch(query, key, value, sequence_start, sequence_end, *, softmax_scale, s
     p.dtype = _native.RPA_DTYPE_BF16 if bf16 else _native.RPA_DTYPE_F32
     p.compute = _native.RPA_COMPUTE_BF16 if bf16 else _native.RPA_COMPUTE_F32
     p.flags = flags
+    aux = None
+    if softmax_aux is not None:
+        if softmax_aux.device != dev:
+            raise ValueError(f"softmax_aux is on {softmax_aux.device}, query on {dev}")
+        aux = _validate_aux(softmax_aux, num_q_heads // num_kv_heads)
+    if aux is not None:
+        p.softmax_aux, p.aux_rows, p.num_sinks = aux.data_ptr(), aux.shape[0], aux.shape[1]
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream
         nbytes = int(lib.rpa_ragged_decode_workspace_bytes(ctypes.byref(p)))
@@ -134,15 +168,14 @@ class RaggedDecodeAttention:
         if platform is not None and platform not in _PLATFORMS:
             raise ValueError(f"platform={platform!r} must be one of {_PLATFORMS}")
         cfg.validate()
-        if softmax_aux is not None:
-            raise NotImplementedError("softmax_aux (attention sinks) is not implemented for ragged_decode_attention here")
         squeeze = query.dim() == 4 and query.shape[1] == 1
         q3 = query[:, 0] if squeeze else query
         _static_validate(q3, key, value, sequence_start, sequence_end, sliding_window, logits_soft_cap)
         if softmax_scale is None:  # _xla_impl_fwd.py:333-334
             softmax_scale = 1.0 / (q3.shape[-1] ** 0.5)
         out = _launch(q3, key, value, sequence_start, sequence_end, softmax_scale=softmax_scale,
-                      sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, cfg=cfg, flags=_flags)
+                      sliding_window=sliding_window, logits_soft_cap=logits_soft_cap, cfg=cfg, flags=_flags,
+                      softmax_aux=softmax_aux)
         return out[:, None] if squeeze else out
 
     def heuristic_cfg(self, inv=None) -> RaggedDecodeAttentionConfig:

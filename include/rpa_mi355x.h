@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define RPA_ABI_VERSION 3
+#define RPA_ABI_VERSION 4
 
 /* element type of queries / kv_pages / out */
 #define RPA_DTYPE_BF16 0
@@ -40,6 +40,8 @@ extern "C" {
 #define RPA_ERR_UNSUPPORTED (-2)
 #define RPA_ERR_WORKSPACE (-3)
 #define RPA_ERR_LAUNCH (-4)
+
+#define RPA_MAX_SINK_KEYS 64 /* most sink positions rpa_ragged_decode_launch accepts (num_sinks) */
 
 /* rpa_fwd_launch flags */
 #define RPA_FLAG_FORCE_GENERIC 1u /* route every sequence through the scalar fp32 kernel */
@@ -164,8 +166,13 @@ int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream)
  * [batch, seq_len, num_kv_heads, head_dim]; sequence b attends to positions [sequence_start[b], sequence_end[b])
  * from the query position sequence_end[b] - 1, optionally only to the last window_left + 1 of them.  Replaces the
  * backend entry ejkernel/kernels/_xla/ragged_decode_attention/_interface.py:26-121 (program:
- * _xla_impl_fwd.py:25-364), reached from ejkernel/modules/operations/ragged_decode_attention.py.  Attention sinks
- * (softmax_aux) are not part of this entry point.
+ * _xla_impl_fwd.py:25-364), reached from ejkernel/modules/operations/ragged_decode_attention.py.
+ *
+ * Attention sinks as that program defines them (softmax_aux, _xla_impl_fwd.py:71-75 and :98-134): with num_sinks > 0
+ * the keys at positions [sequence_start[b], sequence_start[b] + num_sinks) below seq_len are always visible, whatever
+ * sequence_end and the window say, and a key at absolute position t < num_sinks has softmax_aux[row][t] added to its
+ * logit (after the soft cap).  aux_rows is 1 (one vector for every head) or num_q_heads / num_kv_heads (row g for
+ * the g-th query head of every kv head, which is how the program broadcasts a two-dimensional softmax_aux).
  */
 typedef struct RpaRaggedDecodeParams {
   const void* query;             /* [batch, num_q_heads, head_dim]                */
@@ -187,6 +194,9 @@ typedef struct RpaRaggedDecodeParams {
   int32_t dtype;                 /* RPA_DTYPE_*                                   */
   int32_t compute;               /* RPA_COMPUTE_*                                 */
   uint32_t flags;                /* RPA_FLAG_FORCE_GENERIC                        */
+  const float* softmax_aux;      /* [aux_rows, num_sinks] fp32, or null           */
+  int32_t num_sinks;             /* 0 = no sinks; at most RPA_MAX_SINK_KEYS       */
+  int32_t aux_rows;              /* 1 or num_q_heads / num_kv_heads               */
 } RpaRaggedDecodeParams;
 
 uint64_t rpa_ragged_decode_workspace_bytes(const RpaRaggedDecodeParams* dims);

@@ -1,4 +1,4 @@
-"""NumPy restatement of the reference's ``ragged_decode_attention`` (XLA backend), without attention sinks.
+"""NumPy restatement of the reference's ``ragged_decode_attention`` (XLA backend), attention sinks included.
 
 TEST INFRASTRUCTURE ONLY (see ``oracle/__init__.py``).
 
@@ -23,8 +23,19 @@ under-weights every block after the first.  Only sequences that fit one KV block
 attention for all of them and is compared with this function on those cases only.
 ``ragged_decode_exact`` is the dense masked softmax in float64 (zeros when nothing is visible).
 
-Attention sinks (``softmax_aux``, ``:98-134`` and the sink part of the mask) are not restated:
-the build does not implement them.
+Attention sinks (``softmax_aux`` of ``num_sinks`` entries per row).  The program defines them
+through the keys: the positions ``[start, start + num_sinks)`` are visible whatever ``end`` and
+the window say (``:71-75``; the range is not cut at ``end``), and a key at absolute position
+``t < num_sinks`` gets ``softmax_aux[row, t]`` added to its logit after the soft cap and before
+the mask (``apply_attention_sinks_block``, ``:98-134``, called at ``:175-176``).  A one-dimensional
+``softmax_aux`` serves every head.  A two-dimensional one is added as ``[1, 1, rows, block]`` to
+scores of ``[batch, 1, G, block]`` inside the per-kv-head ``vmap`` (``:336-362``; ``softmax_aux``
+is closed over, not mapped), so it only broadcasts with ``rows in (1, G)``, ``G`` the query heads
+per kv head, and row ``g`` then belongs to the ``g``-th query head of every kv head; any other row
+count -- the ``[num_kv_heads, num_sinks]`` of the docstring included, unless it happens to equal
+``G`` -- fails to broadcast (``sink_rows`` raises ``ValueError`` for it).  A float32
+``softmax_aux`` promotes the biased scores of a bfloat16 call, and with them every later op of
+the block, to float32; the carry is cast back at the end of the block (``:198-200``).
 
 Parity status: no golden vectors in the reference, no jax here.  Pins
 (``tests/test_ragged_decode_oracle_pins.py``): brute force on tiny inputs, closed forms,
@@ -40,19 +51,42 @@ import numpy as np
 from .rpa_oracle import _rounder
 
 
-def visible(start, end, seq_len, sliding_window):
+def visible(start, end, seq_len, sliding_window, num_sinks=0):
+    """create_attention_mask (:25-82) for one sequence and one query position."""
     k = np.arange(seq_len)
     m = (k >= start) & (k < end)
     if sliding_window is not None:
         left, right = sliding_window
         qp = end - 1
         m &= (k >= qp - left) & (k <= qp + right)
+    if num_sinks > 0:
+        m |= (k >= start) & (k < start + num_sinks)
     return m
 
 
+def sink_rows(softmax_aux, group):
+    """``[G, num_sinks]`` float32 biases as the program broadcasts them (:118-134), or None."""
+    if softmax_aux is None:
+        return None
+    aux = np.asarray(softmax_aux, dtype=np.float32)
+    if aux.ndim == 1:
+        aux = aux[None, :]
+    if aux.ndim != 2 or aux.shape[0] not in (1, group):
+        raise ValueError(f"softmax_aux of shape {aux.shape} does not broadcast against {group} query heads per kv head")
+    return np.broadcast_to(aux, (group, aux.shape[1]))
+
+
+def _bias(aux, positions):
+    """Bias per (query head of the group, position): softmax_aux[:, t] for t < num_sinks, else 0 (:123-130)."""
+    ns = aux.shape[1]
+    b = aux[:, np.minimum(positions, ns - 1)]
+    return np.where(positions[None, :] < ns, b, np.float32(0.0)).astype(np.float32)
+
+
 def ragged_decode_strict(query, key, value, sequence_start, sequence_end, softmax_scale=None, block_size=128,
-                         sliding_window=None, logits_soft_cap=None, io_dtype="bfloat16"):
-    R = _rounder(io_dtype)
+                         sliding_window=None, logits_soft_cap=None, io_dtype="bfloat16", softmax_aux=None,
+                         aux_dtype="float32"):
+    R = _rounder(io_dtype)  # carries and everything up to the bias
     q = np.asarray(query, dtype=np.float32)
     kk = np.asarray(key, dtype=np.float32)
     vv = np.asarray(value, dtype=np.float32)
@@ -60,6 +94,10 @@ def ragged_decode_strict(query, key, value, sequence_start, sequence_end, softma
     _, S, Hkv, _ = kk.shape
     G = Hq // Hkv
     scale = R(np.float32(1.0 / np.sqrt(D) if softmax_scale is None else softmax_scale))
+    aux = sink_rows(softmax_aux, G)
+    ns = 0 if aux is None else aux.shape[1]
+    # ops after the bias run in the promoted dtype
+    Rm = R if (aux is None or aux_dtype == io_dtype) else _rounder("float32")
     nblk = -(-S // block_size)
     pad = nblk * block_size - S
     if pad:
@@ -68,7 +106,7 @@ def ragged_decode_strict(query, key, value, sequence_start, sequence_end, softma
     out = np.zeros((B, Hq, D), np.float32)
     with np.errstate(invalid="ignore", over="ignore"):
         for b in range(B):
-            mask = np.pad(visible(int(sequence_start[b]), int(sequence_end[b]), S, sliding_window), (0, pad))
+            mask = np.pad(visible(int(sequence_start[b]), int(sequence_end[b]), S, sliding_window, ns), (0, pad))
             qs = R(q[b].reshape(Hkv, G, D) * scale)
             o = np.zeros((Hkv, G, D), np.float32)
             m = np.full((Hkv, G, 1), -np.inf, np.float32)
@@ -82,24 +120,26 @@ def ragged_decode_strict(query, key, value, sequence_start, sequence_end, softma
                 if logits_soft_cap is not None:
                     cap = np.float32(logits_soft_cap)
                     sc = R(R(np.tanh(R(sc / cap))) * cap)
+                if aux is not None:
+                    sc = Rm(sc + _bias(aux, np.arange(i * block_size, (i + 1) * block_size))[None, :, :])
                 sc = np.where(mb, sc, -np.inf).astype(np.float32)
                 m_new = np.maximum(m, sc.max(axis=-1, keepdims=True))
-                e = R(np.exp(R(sc - m_new)))
+                e = Rm(np.exp(Rm(sc - m_new)))
                 e = np.where(mb, e, np.float32(0.0))
-                l_curr = R(e.sum(axis=-1, keepdims=True, dtype=np.float32))
-                corr = R(np.exp(R(m - m_new)))
-                l_new = R(R(corr * l) + l_curr)
+                l_curr = Rm(e.sum(axis=-1, keepdims=True, dtype=np.float32))
+                corr = Rm(np.exp(Rm(m - m_new)))
+                l_new = Rm(Rm(corr * l) + l_curr)
                 safe = np.where(l_new == 0, np.float32(1.0), l_new)
-                w = R(e / safe)
-                o_curr = R(np.einsum("jgk,jkd->jgd", w, vb, dtype=np.float32))
-                o = R(R(R(R(corr * l) * o) + R(l_curr * o_curr)) / safe)
-                m, l = m_new, l_new
+                w = Rm(e / safe)
+                o_curr = Rm(np.einsum("jgk,jkd->jgd", w, vb, dtype=np.float32))
+                o = R(Rm(Rm(Rm(Rm(corr * l) * o) + Rm(l_curr * o_curr)) / safe))
+                m, l = R(m_new), R(l_new)
             out[b] = o.reshape(Hq, D)
     return out
 
 
 def ragged_decode_exact(query, key, value, sequence_start, sequence_end, softmax_scale=None, sliding_window=None,
-                        logits_soft_cap=None):
+                        logits_soft_cap=None, softmax_aux=None):
     q = np.asarray(query, dtype=np.float64)
     kk = np.asarray(key, dtype=np.float64)
     vv = np.asarray(value, dtype=np.float64)
@@ -107,9 +147,11 @@ def ragged_decode_exact(query, key, value, sequence_start, sequence_end, softmax
     _, S, Hkv, _ = kk.shape
     G = Hq // Hkv
     scale = 1.0 / np.sqrt(D) if softmax_scale is None else float(softmax_scale)
+    aux = sink_rows(softmax_aux, G)
+    ns = 0 if aux is None else aux.shape[1]
     out = np.zeros((B, Hq, D))
     for b in range(B):
-        vis = visible(int(sequence_start[b]), int(sequence_end[b]), S, sliding_window)
+        vis = visible(int(sequence_start[b]), int(sequence_end[b]), S, sliding_window, ns)
         if not vis.any():
             continue
         k = kk[b, vis].transpose(1, 0, 2)
@@ -117,6 +159,8 @@ def ragged_decode_exact(query, key, value, sequence_start, sequence_end, softmax
         sc = np.einsum("jgd,jkd->jgk", q[b].reshape(Hkv, G, D) * scale, k)
         if logits_soft_cap is not None:
             sc = logits_soft_cap * np.tanh(sc / logits_soft_cap)
+        if aux is not None:
+            sc = sc + _bias(aux, np.flatnonzero(vis)).astype(np.float64)[None, :, :]
         w = np.exp(sc - sc.max(axis=-1, keepdims=True))
         w /= w.sum(axis=-1, keepdims=True)
         out[b] = np.einsum("jgk,jkd->jgd", w, v).reshape(Hq, D)

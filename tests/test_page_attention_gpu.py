@@ -43,8 +43,9 @@ KV = [1, 15, 16, 17, 100, 255, 256, 300, 64]
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("kw", [dict(), dict(num_q_heads=8, num_kv_heads=8), dict(num_q_heads=32, num_kv_heads=1),
                                 dict(head_dim=256, num_q_heads=16, num_kv_heads=8), dict(block_size=4, max_blocks=80),
-                                dict(block_size=64, max_blocks=5), dict(head_dim=64)],
-                         ids=["gqa4", "mha", "mqa32", "d256", "block4", "block64", "d64"])
+                                dict(block_size=64, max_blocks=5), dict(head_dim=64),
+                                dict(num_q_heads=80, num_kv_heads=1)],
+                         ids=["gqa4", "mha", "mqa32", "d256", "block4", "block64", "d64", "mqa80"])
 def test_bf16_explicit_scale(kw, flags):
     b = small(KV, **kw)
     ref = page_attention_strict(*np_args(b), attn_scale=b.attn_scale)

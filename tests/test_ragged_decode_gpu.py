@@ -42,8 +42,9 @@ ENDS = [1, 15, 16, 17, 100, 255, 256, 300, 64]
 
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("kw", [dict(), dict(num_q_heads=8, num_kv_heads=8), dict(num_q_heads=32, num_kv_heads=1),
-                                dict(head_dim=256, num_q_heads=16, num_kv_heads=8), dict(head_dim=64), dict(seq_len=301)],
-                         ids=["gqa4", "mha", "mqa32", "d256", "d64", "odd_seq_len"])
+                                dict(head_dim=256, num_q_heads=16, num_kv_heads=8), dict(head_dim=64), dict(seq_len=301),
+                                dict(num_q_heads=80, num_kv_heads=1)],
+                         ids=["gqa4", "mha", "mqa32", "d256", "d64", "odd_seq_len", "mqa80"])
 def test_bf16_against_the_reference_program_on_one_block(kw, flags):
     b = small(np.zeros(len(ENDS), int), ENDS, **kw)
     ref = ragged_decode_strict(*np_args(b), softmax_scale=b.softmax_scale, block_size=512)
@@ -87,8 +88,11 @@ def test_query_with_a_singleton_axis_and_rejected_arguments():
     out = ragged_decode_attention(*b.args())
     out4 = ragged_decode_attention(b.query[:, None], *b.args()[1:])
     assert out4.shape == (2, 1, 8, 128) and torch.equal(out4[:, 0], out)
-    with pytest.raises(NotImplementedError, match="softmax_aux"):
-        ragged_decode_attention(*b.args(), torch.zeros(4, device=DEV))
+    with pytest.raises(ValueError, match="broadcast"):   # [num_kv_heads, num_sinks] with 4 query heads per kv head
+        ragged_decode_attention(*b.args(), torch.zeros(2, 4, device=DEV))
+    with pytest.raises(ValueError, match="at most"):
+        ragged_decode_attention(*b.args(), torch.zeros(65, device=DEV))
+    assert torch.equal(ragged_decode_attention(*b.args(), torch.zeros(0, device=DEV)), out)
     with pytest.raises(ValueError):
         ragged_decode_attention(*b.args(), sliding_window=(-1, 0))
     with pytest.raises(ValueError):
@@ -97,6 +101,88 @@ def test_query_with_a_singleton_axis_and_rejected_arguments():
         ragged_decode_attention(*b.args(), cfg=RaggedDecodeAttentionConfig(platform="tpu"))
     with pytest.raises(NotImplementedError):
         ragged_decode_attention(*b.args(), mesh=object())
+
+
+# ---- attention sinks (softmax_aux): keys [start, start + num_sinks) always visible, bias on absolute t < num_sinks
+
+SINK_STARTS = [0, 2, 16, 0, 99, 200, 31, 290, 64, 318]
+SINK_ENDS = [1, 15, 16, 300, 100, 255, 256, 300, 64, 320]   # 2: empty, 8: empty, 9: sink range cut by seq_len
+
+
+def sink_batch(**kw):
+    return small(SINK_STARTS, SINK_ENDS, **kw)
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("window,cap", [(None, None), ((40, 0), None), ((0, 0), None), ((100, 0), 5.0)])
+@pytest.mark.parametrize("aux_kind", ["vector", "per_group_head"])
+def test_bf16_sinks_against_float64(flags, window, cap, aux_kind):
+    b = sink_batch()
+    g = torch.Generator().manual_seed(3)
+    aux = (torch.randn(5, generator=g) if aux_kind == "vector" else torch.randn(4, 5, generator=g)) * 2.0
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=window, logits_soft_cap=cap,
+                              softmax_aux=aux.numpy())
+    out = to_np(ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, sliding_window=window,
+                                        logits_soft_cap=cap, _flags=flags))
+    assert_bf16_parity(out, ref, len(SINK_ENDS), f"sinks {aux_kind} window {window} cap {cap}")
+    assert out[2].any() and out[8].any()               # an empty sequence still attends to its sink range
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("kw", [dict(num_q_heads=8, num_kv_heads=8), dict(num_q_heads=32, num_kv_heads=1),
+                                dict(head_dim=256, num_q_heads=16, num_kv_heads=8), dict(head_dim=64)],
+                         ids=["mha", "mqa32", "d256", "d64"])
+def test_bf16_sinks_against_the_reference_program_on_one_block(kw, flags):
+    b = small(np.zeros(len(ENDS), int), ENDS, **kw)
+    aux = torch.tensor([1.5, -0.5, 3.0, 0.25])
+    ref = ragged_decode_strict(*np_args(b), softmax_scale=b.softmax_scale, block_size=512, softmax_aux=aux.numpy())
+    out = to_np(ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, _flags=flags))
+    assert_bf16_parity(out, ref, len(ENDS), f"sinks {kw}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_float32_sinks_against_float64(flags):
+    b = sink_batch(dtype=torch.float32)
+    aux = torch.tensor([[0.5, -1.0, 2.0]])
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=(30, 0), softmax_aux=aux.numpy())
+    out = to_np(ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, sliding_window=(30, 0),
+                                        _flags=flags))
+    mx, _ = err_stats(out, ref, len(SINK_ENDS))
+    assert mx <= F32_MAX_ABS, mx
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_sink_closed_forms_on_the_device(flags):
+    # q = 0 and a window that keeps the query position only: weights e^{a_t} on the sink range, 1 on the query position
+    b = small([0, 5], [200, 200], dtype=torch.float32)
+    b.query.zero_()
+    aux = torch.tensor([0.75, -0.5])
+    out = ragged_decode_attention(*b.args(), aux.to(DEV), sliding_window=(0, 0), _flags=flags).double()
+    v = b.value.double()
+    w0, w1 = float(np.exp(0.75)), float(np.exp(-0.5))
+    want0 = (w0 * v[0, 0] + w1 * v[0, 1] + v[0, 199]) / (w0 + w1 + 1.0)
+    want1 = (v[1, 5] + v[1, 6] + v[1, 199]) / 3.0     # the sink range {5, 6} lies past the biased positions
+    assert (out[0] - want0.repeat_interleave(4, dim=0)).abs().max() <= 1e-6
+    assert (out[1] - want1.repeat_interleave(4, dim=0)).abs().max() <= 1e-6
+    # biases of zero on keys that are visible anyway change nothing at all
+    b = small([0, 3], [300, 77])
+    plain = ragged_decode_attention(*b.args(), _flags=flags)
+    zeros = ragged_decode_attention(*b.args(), torch.zeros(4, device=DEV), _flags=flags)
+    assert (plain.float() - zeros.float()).abs().max() <= 8e-3   # same keys, split at another point: one bf16 ulp
+
+
+def test_sinks_full_size_workload():
+    b = ragged_decode_workload("decode_llama3_8b", device=DEV)
+    aux = torch.linspace(-1.0, 2.0, 4)
+    out = ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, sliding_window=(1023, 0))
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    assert torch.equal(out, ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale,
+                                                    sliding_window=(1023, 0)))
+    ids = torch.tensor(sorted(int(s) for s in np.random.default_rng(1).permutation(len(b.ends))[:8]))
+    sub = [to_np(t[ids.to(DEV)]) for t in b.args()]
+    ref = ragged_decode_exact(*sub, softmax_scale=b.softmax_scale, sliding_window=(1023, 0), softmax_aux=aux.numpy())
+    assert_bf16_parity(to_np(out[ids.to(DEV)]), ref, len(ids), "decode_llama3_8b with sinks")
 
 
 @pytest.mark.parametrize("name,n_sample", [("decode_small", 8), ("decode_llama3_8b", 10)])

@@ -149,6 +149,18 @@ def test_bf16_prefill_tiles_over_many_key_tiles(flags, hq, hkv, D, window):
     assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, f"prefill tiles {hq}/{hkv} D={D} W={window}")
 
 
+@pytest.mark.parametrize("hq,hkv,D", [(8, 2, 128), (16, 2, 256), (8, 2, 64)])
+@pytest.mark.parametrize("window", [None, 48])
+def test_bf16_long_chunks_in_a_decode_shaped_batch(hq, hkv, D, window):
+    """A token buffer no larger than the number of sequence slots runs on the kernel without prefill tiles: chunks with
+    many row tiles are then walked as wave-level items."""
+    b = small([40, 1, 1, 23, 1], [300, 300, 17, 23, 90], num_q_heads=hq, num_kv_heads=hkv, head_dim=D,
+              pages_per_seq=32, sliding_window=window, max_num_seqs=96)
+    assert b.queries.shape[0] <= 96 + 16
+    out = to_np(run_hip(b, 0))
+    assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, f"decode-shaped {hq}/{hkv} D={D} W={window}")
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("window", [None, 48])
 def test_bf16_first_visible_key_per_sequence(flags, window):
