@@ -89,6 +89,20 @@ def main():
                         softmax_scale=np.float32(128 ** -0.5), block_size=np.int32(128),
                         expected=rpa_oracle.bf16_bits(out))
 
+    # attention sinks: three biased positions, a window that leaves the sink range outside, starts inside and past
+    # the biased positions, an empty sequence
+    rng = np.random.default_rng(6)
+    q = bf(rng.standard_normal((4, 4, 128)))
+    k, v = (bf(rng.standard_normal((4, 96, 2, 128))) for _ in range(2))
+    start, end = np.array([0, 1, 40, 90], np.int32), np.array([96, 50, 40, 96], np.int32)
+    aux = np.array([[1.5, -0.75, 0.5], [0.0, 2.0, -1.0]], np.float32)
+    out = ragged_decode_strict(q, k, v, start, end, softmax_scale=128 ** -0.5, block_size=128, sliding_window=(9, 0),
+                               softmax_aux=aux)
+    np.savez_compressed(os.path.join(HERE, "ragged_decode_sinks.npz"), query=rpa_oracle.bf16_bits(q),
+                        key=rpa_oracle.bf16_bits(k), value=rpa_oracle.bf16_bits(v), sequence_start=start,
+                        sequence_end=end, softmax_scale=np.float32(128 ** -0.5), block_size=np.int32(128),
+                        window_left=np.int32(9), softmax_aux=aux, expected=rpa_oracle.bf16_bits(out))
+
 
 if __name__ == "__main__":
     main()

@@ -51,6 +51,11 @@ def test_other_oracles_reproduce_their_fixtures():
     out = ragged_decode_strict(*[bf16_from_bits(f[k]) for k in ("query", "key", "value")], f["sequence_start"],
                                f["sequence_end"], softmax_scale=float(f["softmax_scale"]), block_size=int(f["block_size"]))
     assert np.array_equal(bf16_bits(out), f["expected"])
+    f = load("ragged_decode_sinks.npz")
+    out = ragged_decode_strict(*[bf16_from_bits(f[k]) for k in ("query", "key", "value")], f["sequence_start"],
+                               f["sequence_end"], softmax_scale=float(f["softmax_scale"]), block_size=int(f["block_size"]),
+                               sliding_window=(int(f["window_left"]), 0), softmax_aux=f["softmax_aux"])
+    assert np.array_equal(bf16_bits(out), f["expected"])
 
 
 # ----------------------------------------------------------------------------- device side
@@ -101,4 +106,9 @@ def test_device_kernels_against_the_frozen_outputs(flags):
     f = load("ragged_decode.npz")
     out = ragged_decode_attention(_dev(f["query"]), _dev(f["key"]), _dev(f["value"]), _idx(f["sequence_start"]),
                                   _idx(f["sequence_end"]), softmax_scale=float(f["softmax_scale"]), _flags=flags)
+    _check(out, f["expected"], 4)
+    f = load("ragged_decode_sinks.npz")
+    out = ragged_decode_attention(_dev(f["query"]), _dev(f["key"]), _dev(f["value"]), _idx(f["sequence_start"]),
+                                  _idx(f["sequence_end"]), _idx(f["softmax_aux"]), softmax_scale=float(f["softmax_scale"]),
+                                  sliding_window=(int(f["window_left"]), 0), _flags=flags)
     _check(out, f["expected"], 4)
