@@ -42,6 +42,39 @@ def test_struct_layout_matches_header_field_order():
     assert ctypes.sizeof(_native.RpaParams) % 8 == 0
 
 
+@pytest.mark.parametrize("name", ["RpaV3Params", "RpaPageAttnParams", "RpaRaggedDecodeParams"])
+def test_other_struct_layouts_match_header_field_order(name):
+    text = (ROOT / "include" / "rpa_mi355x.h").read_text()
+    body = text[text.index(f"typedef struct {name} {{"):text.index(f"}} {name};")]
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = re.findall(r"([a-z_]+)\s*;", body)
+    assert names == [f[0] for f in getattr(_native, name)._fields_]
+
+
+def test_ragged_decode_sink_arguments_are_checked_before_any_launch():
+    lib = _native.load()
+    p = _native.RpaRaggedDecodeParams()
+    p.batch, p.num_q_heads, p.num_kv_heads, p.head_dim, p.seq_len = 4, 8, 2, 128, 64
+    p.softmax_scale, p.window_left = 0.1, -1
+    plain = lib.rpa_ragged_decode_workspace_bytes(ctypes.byref(p))
+    p.num_sinks, p.aux_rows = 4, 1
+    with_sinks = lib.rpa_ragged_decode_workspace_bytes(ctypes.byref(p))
+    assert with_sinks >= plain + 4 * 8 * (128 + 2) * 4       # the sink keys' state per (sequence, query head)
+    buf = (ctypes.c_char * 64)()
+    addr = ctypes.addressof(buf)                              # never dereferenced: every call below fails first
+    for f in ("query", "key", "value", "sequence_start", "sequence_end", "out", "workspace"):
+        setattr(p, f, addr)
+    p.workspace_bytes = with_sinks
+    assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -1 and b"softmax_aux is null" in lib.rpa_last_error()
+    p.softmax_aux = addr
+    p.num_sinks = _native.RPA_MAX_SINK_KEYS + 1
+    assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -1 and b"num_sinks" in lib.rpa_last_error()
+    p.num_sinks, p.aux_rows = 4, 2                            # 4 query heads per kv head: 1 or 4 rows
+    assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -1 and b"aux_rows" in lib.rpa_last_error()
+    p.aux_rows, p.workspace_bytes = 4, plain
+    assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -3 and b"too small" in lib.rpa_last_error()
+
+
 def test_workspace_bytes_and_errors_without_gpu():
     lib = _native.load()
     p = _native.RpaParams()
