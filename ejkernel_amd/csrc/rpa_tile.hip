@@ -35,12 +35,16 @@ namespace rpa {
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
 constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
+constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
 constexpr int kDecodeShapedPadRows = 16; // token rows beyond one per sequence slot that still count as a decode batch
 
-// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints and 8 ints of scratch, then the data region
+// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 8 ints of scratch and the sequences with prefill
+// tiles in order of length (up to kSortMax ints), then the data region
 // shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
+__host__ __device__ constexpr int sort_entries(int max_num_seqs) { return max_num_seqs < kSortMax ? max_num_seqs : kSortMax; }
 __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
-  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 8) * sizeof(int) + 15) & ~static_cast<size_t>(15);
+  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 8 + sort_entries(max_num_seqs)) * sizeof(int) + 15) &
+         ~static_cast<size_t>(15);
 }
 
 // kWaveOnly: the prefill tiles are compiled out and sequences with many row tiles run as wave-level items too (right
@@ -63,6 +67,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   int* tile_start = item_start + (sched_n + 1);     // decode stream tiles
   int* wg_start = tile_start + (sched_n + 1);       // workgroup-level prefill tiles
   int* scratch = wg_start + (sched_n + 1);
+  int* wg_seq = scratch + 8;                        // sequence of the r-th entry of wg_start, when those are sorted
   char* lds_data = smem + sched_bytes(sched_n);
   char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
@@ -112,6 +117,60 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
     wg_start[nc] = total_wg;
   }
   __syncthreads();
+
+  // ---- prefill order.  Tiles are drawn from the queues in item order and a tile's cost grows with the number of
+  // keys it can see, so the longest sequences go first (as in longest-processing-time-first scheduling: the work left
+  // for the end is the short tiles).  wg_start is rebuilt over the sequences that have prefill tiles, by descending
+  // length; wg_seq names them.  The data region, not yet in use, holds the temporaries.
+  int n_sorted = 0;
+  if constexpr (!kWaveOnly) {
+    if (total_wg > 0 && shift == 0 && a.phase_mode == 4) {
+      int mine = 0;
+      for (int s = s_begin; s < s_end; ++s) {
+        int t, it, wg;
+        classify(seq_info<C::TT>(p, s, G), t, it, wg);
+        mine += wg > 0;
+      }
+      int n_pf;
+      int at = block_excl_scan(mine, scratch, n_pf);
+      n_pf = __builtin_amdgcn_readfirstlane(n_pf);
+      if (n_pf <= kSortMax) {
+        int* t_seq = reinterpret_cast<int*>(lds_data);
+        int* t_key = t_seq + kSortMax;
+        int* t_cnt = t_key + kSortMax;
+        int* o_cnt = t_cnt + kSortMax;
+        for (int s = s_begin; s < s_end; ++s) {
+          int t, it, wg;
+          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          classify(si, t, it, wg);
+          if (wg > 0) {
+            t_seq[at] = s;
+            t_key[at] = si.kv_len;
+            t_cnt[at] = wg;
+            ++at;
+          }
+        }
+        __syncthreads();
+        if (tid < n_pf) {
+          const int key = t_key[tid];
+          int r = 0;
+          for (int t = 0; t < n_pf; ++t) {
+            const int kt = t_key[t];
+            r += (kt > key || (kt == key && t < tid)) ? 1 : 0;
+          }
+          wg_seq[r] = t_seq[tid];
+          o_cnt[r] = t_cnt[tid];
+        }
+        __syncthreads();
+        int tot;
+        const int excl = block_excl_scan(tid < n_pf ? o_cnt[tid] : 0, scratch, tot);
+        if (tid < n_pf) wg_start[tid] = excl;
+        if (tid == 0) wg_start[n_pf] = tot;
+        n_sorted = n_pf;
+        __syncthreads();
+      }
+    }
+  }
 
   // ---- rows past the ragged batch are zero
   {
@@ -210,8 +269,19 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
             ++probe;
           }
           if (w < 0) break;
-          int s_base;
-          const int s = find(wg_start, 2, w, s_base);
+          int s_base, s;
+          if (n_sorted > 0) {
+            int lo = 0, hi = n_sorted;
+            while (hi - lo > 1) {
+              const int mid = (lo + hi) >> 1;
+              if (wg_start[mid] <= w) lo = mid; else hi = mid;
+            }
+            lo = __builtin_amdgcn_readfirstlane(lo);
+            s = __builtin_amdgcn_readfirstlane(wg_seq[lo]);
+            s_base = __builtin_amdgcn_readfirstlane(wg_start[lo]);
+          } else {
+            s = find(wg_start, 2, w, s_base);
+          }
           const SeqInfo si = seq_info<C::TT>(p, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
           const int local = w - s_base;
