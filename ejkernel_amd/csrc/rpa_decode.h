@@ -172,6 +172,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r] * post_scale;
     if (cap != 0.f) {
+      asm volatile("" : "+v"(sv[0][0]));  // keeps the soft cap inside this wave-uniform branch (it is not cheap)
 #pragma unroll
       for (int u = 0; u < NT; ++u)
 #pragma unroll

@@ -86,10 +86,17 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 
   // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
   const int w_row_lo = wg_row_lo + wave * C::WROWS;
-  bool row_valid[MRT];
   int pos_n[MRT];
-  size_t q_off[MRT];
-  int head[MRT];
+  // Row of the batch and head behind row tile m of this lane.  Needed before and after the key loop, and computed
+  // in both places rather than held in registers across it (an opaque zero keeps the compiler from doing so).
+  auto row_of = [&](int m, int opaque0, bool& valid, int& head, size_t& q_off) {
+    const int R = w_row_lo + 16 * m + i + opaque0;
+    valid = R < si.rows;
+    const int qi = valid ? R / G : 0;
+    head = j * G + (valid ? R - qi * G : 0);
+    q_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * hd;
+    return qi;
+  };
   int t_pos_lo[MRT], t_pos_hi[MRT];  // positions spanned by the valid rows of the row tile (wave-uniform)
   bool t_any[MRT];
   bf16x8_t qreg[MRT][C::NKS];
@@ -101,12 +108,11 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const float sf = fold_scale ? post_scale : 1.f, sf_log2e = sf * kLog2e;
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
-    const int R = w_row_lo + 16 * m + i;
-    row_valid[m] = R < si.rows;
-    const int qi = row_valid[m] ? R / G : 0;
-    head[m] = j * G + (row_valid[m] ? R - qi * G : 0);
-    pos_n[m] = row_valid[m] ? pos0 + qi : -1;
-    q_off[m] = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head[m]) * hd;
+    bool valid;
+    int head;
+    size_t q_off;
+    const int qi = row_of(m, 0, valid, head, q_off);
+    pos_n[m] = valid ? pos0 + qi : -1;
     const int tr_lo = w_row_lo + 16 * m, tr_hi = min(tr_lo + 16, si.rows);
     t_any[m] = tr_hi > tr_lo;
     t_pos_lo[m] = pos0 + tr_lo / G;
@@ -114,7 +120,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (row_valid[m] && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off[m] + 32 * ks + 8 * g);
+      if (valid && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e)
@@ -134,16 +140,30 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     nomask_hi[m] = min(t_pos_lo[m] - 31, range_hi - 32);
     nomask_lo[m] = max(W > 0 ? t_pos_hi[m] - W : -0x7fffffff, si.start - 1);
   }
+  // One interval test per row tile in the loop: no mask is needed iff clear_lo < a0 <= clear_hi.
+  int clear_lo[MRT], clear_hi[MRT];
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    clear_lo[m] = max(nomask_lo[m], act_lo[m]);
+    clear_hi[m] = min(nomask_hi[m], act_hi[m]);
+  }
   const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;  // < w_pos_lo when the wave has no rows
   const int w_pos_lo = pos0 + w_row_lo / G;
   const bool w_any = w_row_lo < si.rows;
+  // Halves that lie entirely in this wavefront's causal future or left of its window are skipped: a half is walked
+  // iff w_act_lo < a0 <= w_act_hi.
+  const int w_act_hi = w_any ? min(range_hi - 1, w_pos_hi) : -0x7fffffff;
+  const int w_act_lo = W > 0 ? w_pos_lo - W - 31 : -0x7fffffff;
 
   f32x4_t o_acc[MRT][C::NS][8];
   f32x4_t l_acc[MRT];
-  float m_run[MRT];
+  // Softmax reference point m per row, kept as the exp2 offset -m log2(e) (0 while the row has seen no key) and
+  // as the vote threshold for exp2 arguments: kLazy log2(e) once there is a reference point, -inf before.
+  float m_thr[MRT], m_neg[MRT];
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
-    m_run[m] = -INFINITY;
+    m_thr[m] = -INFINITY;
+    m_neg[m] = 0.f;
     l_acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sN = 0; sN < C::NS; ++sN)
@@ -280,7 +300,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       for (int h = 0; h < C::NH; ++h) {
         const int a0 = tile + 32 * h;  // first key of this half
         // halves that lie entirely in this wavefront's causal future or left of its window are skipped
-        const bool active = w_any && a0 < range_hi && a0 <= w_pos_hi && !(W > 0 && a0 + 31 <= w_pos_lo - W);
+        const bool active = a0 > w_act_lo && a0 <= w_act_hi;
         // V of one slice: with the transposing read, per column unit c the keys 4g..4g+3 of the two sub-tiles (one
         // A operand); otherwise eight 16-byte pieces (rows 4g..4g+3 of the two sub-tiles, piece i)
         u32x4_t vraw[8];
@@ -342,6 +362,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               for (int r = 0; r < 4; ++r) sv[u][r] *= post_scale;
           }
           if (cap != 0.f) {
+            asm volatile("" : "+v"(sv[0][0]));  // keeps the soft cap inside this wave-uniform branch (it is not cheap)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
@@ -349,7 +370,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                 sv[u][r] = soft_cap<kMimic>(sv[u][r], cap, inv_cap);
           }
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
-          const bool need_mask = a0 > nomask_hi[m] || a0 <= nomask_lo[m] || a0 > act_hi[m] || a0 <= act_lo[m];
+          const bool need_mask = a0 <= clear_lo[m] || a0 > clear_hi[m];
           if (need_mask) {
             int tok0 = a0 + 4 * g;
             asm volatile("" : "+v"(tok0));  // keeps the per-key compares inside this (rare) branch
@@ -362,32 +383,41 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                 sv[u][r] = keep ? sv[u][r] : -INFINITY;
               }
           }
-          float tmax = sf * fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
-                                  fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
-          // Lazy rescale: the reference point m_run (the same in the four lanes of a row) only moves when some
-          // logit exceeds it by more than kLazy; probabilities then stay below e^kLazy, far inside bf16 / fp32
-          // range.  The common case needs no cross-lane step at all: a wave-wide vote on the lane-local maxima.
-          float alpha = 1.f;
-          if (__builtin_expect(__any(tmax > m_run[m] + kLazy), 0)) {
+          // exp2 arguments against the current reference point: t = (logit - m) log2(e), with m = 0 while the row has
+          // seen no key.  They are arithmetic results, so their maximum needs no canonicalising self-maxima and
+          // compiles to three-operand maxima.
+          float t[2][4];
+#pragma unroll
+          for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) t[u][r] = fmaf(sv[u][r], sf_log2e, m_neg[m]);
+          float tmax = fmaxf(fmaxf(fmaxf(t[0][0], t[0][1]), fmaxf(t[0][2], t[0][3])),
+                             fmaxf(fmaxf(t[1][0], t[1][1]), fmaxf(t[1][2], t[1][3])));
+          // Lazy rescale: the reference point (the same in the four lanes of a row) only moves when some logit
+          // exceeds it by more than kLazy; probabilities then stay below e^kLazy, far inside bf16 / fp32 range.
+          // The common case needs no cross-lane step at all: a wave-wide vote on the lane-local maxima, and the t
+          // are the exp2 arguments as they stand.  When the point moves up by the row maximum, so do the t.
+          if (__builtin_expect(__any(tmax > m_thr[m]), 0)) {
             tmax = row_groups_max(tmax);
-            const bool bump = tmax > m_run[m] + kLazy;
-            const float m_new = bump ? tmax : m_run[m];
-            alpha = bump ? __builtin_amdgcn_exp2f((m_run[m] - m_new) * kLog2e) : 1.f;  // m_new is finite here
-            m_run[m] = m_new;
+            const bool bump = tmax > m_thr[m];  // then tmax is finite
+            const float shift = bump ? tmax : 0.f;
+            const float alpha = !bump ? 1.f : m_thr[m] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(-tmax);
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) t[u][r] -= shift;
+            m_neg[m] -= shift;
+            m_thr[m] = bump ? kLazy * kLog2e : m_thr[m];
             l_acc[m] *= alpha;
 #pragma unroll
             for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
               for (int c = 0; c < 8; ++c) o_acc[m][sN][c] *= alpha;
           }
-          const float m_use = m_run[m] == -INFINITY ? 0.f : m_run[m];
-          const float neg = -m_use * kLog2e;
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
-            float e0 = __builtin_amdgcn_exp2f(fmaf(sv[u][0], sf_log2e, neg));
-            float e1 = __builtin_amdgcn_exp2f(fmaf(sv[u][1], sf_log2e, neg));
-            float e2 = __builtin_amdgcn_exp2f(fmaf(sv[u][2], sf_log2e, neg));
-            float e3 = __builtin_amdgcn_exp2f(fmaf(sv[u][3], sf_log2e, neg));
+            const float e0 = __builtin_amdgcn_exp2f(t[u][0]), e1 = __builtin_amdgcn_exp2f(t[u][1]);
+            const float e2 = __builtin_amdgcn_exp2f(t[u][2]), e3 = __builtin_amdgcn_exp2f(t[u][3]);
             pw[m][2 * u] = pack_bf16x2(e0, e1);
             pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
           }
@@ -454,21 +484,28 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // ---- normalise (with optional sinks) and store
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
-    if (!row_valid[m]) continue;
+    bool valid;
+    int head;
+    size_t q_off;
+    int opaque0 = 0;
+    asm volatile("" : "+v"(opaque0));
+    row_of(m, opaque0, valid, head, q_off);
+    if (!valid) continue;
     const float l_run = l_acc[m][0];
+    const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
-      const float* __restrict__ sk = p.sinks + static_cast<size_t>(head[m]) * p.num_sinks;
+      const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
       float smax = -INFINITY;
       for (int k = 0; k < p.num_sinks; ++k) smax = fmaxf(smax, sk[k]);
-      const float mt = fmaxf(m_run[m], smax);
+      const float mt = fmaxf(m_row, smax);
       float ssum = 0.f;
       for (int k = 0; k < p.num_sinks; ++k) ssum += expf(sk[k] - mt);
-      num_scale = m_run[m] == -INFINITY ? 0.f : expf(m_run[m] - mt);
+      num_scale = m_row == -INFINITY ? 0.f : expf(m_row - mt);
       denom = num_scale * l_run + ssum;
     }
     const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
-    bf16_t* orow = out + q_off[m];
+    bf16_t* orow = out + q_off;
     if constexpr (C::TRV) {
       // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row
 #pragma unroll
