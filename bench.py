@@ -25,8 +25,8 @@ if ROOT not in sys.path:
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes (scaled by a plain 1 GiB device copy); a
 # workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_llama3_8b": (2185792 * 2.0 + 21519 * 1.0) * 1024,
-    "mixed_prefill_decode": (2162317 * 2.0 + 90297 * 1.0) * 1024,
+    "decode_llama3_8b": (2184714 * 2.0 + 18447 * 1.0) * 1024,
+    "mixed_prefill_decode": (2156653 * 2.0 + 90300 * 1.0) * 1024,
 }
 
 
@@ -42,6 +42,10 @@ def parse():
                          "page_attention = the decode workloads (decode_small, decode_llama3_8b) with separate K and V "
                          "caches of [blocks, kv heads, block, head_dim]; ragged_decode = ragged_decode_attention on the "
                          "same lengths with contiguous K and V of [batch, seq_len, kv heads, head_dim]")
+    ap.add_argument("--sinks", type=int, default=0,
+                    help="--op ragged_decode: attention sinks (softmax_aux of this many biases, shared by all heads)")
+    ap.add_argument("--window", type=int, default=0,
+                    help="--op ragged_decode: sliding_window=(WINDOW - 1, 0), i.e. the last WINDOW keys (0 = none)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the workload (debugging only)")
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -193,9 +197,18 @@ def page_attention_main(args):
     counts = algorithmic_counts(np.ones(S, np.int64), b.kv_lens, num_q_heads=m["num_q_heads"],
                                 num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=m.get("page_size", 16))
 
+    aux = torch.linspace(-1.0, 2.0, args.sinks, device=dev) if contiguous and args.sinks > 0 else None
+    window = (args.window - 1, 0) if contiguous and args.window > 0 else None
+    if contiguous and (aux is not None or window is not None):
+        # keys a sequence reads: its last WINDOW ones plus the sink range
+        seen = np.minimum(b.kv_lens, args.window) if window is not None else b.kv_lens
+        b.kv_lens = np.minimum(b.kv_lens, seen + args.sinks)
+        counts = algorithmic_counts(np.ones(S, np.int64), b.kv_lens, num_q_heads=m["num_q_heads"],
+                                    num_kv_heads=m["num_kv_heads"], head_dim=m["head_dim"], page_size=16)
+
     def step():
         if contiguous:
-            return ragged_decode_attention(*b.args(), softmax_scale=b.softmax_scale)
+            return ragged_decode_attention(*b.args(), aux, softmax_scale=b.softmax_scale, sliding_window=window)
         return page_attention(*b.args(), attn_scale=b.attn_scale)
 
     for _ in range(args.warmup):
@@ -219,7 +232,8 @@ def page_attention_main(args):
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": args.workload, "op": args.op, "description": WORKLOADS[args.workload], "scale": args.scale,
-                   "query_tokens": S, "num_seqs": S, "kv_tokens": int(b.kv_lens.sum())},
+                   "query_tokens": S, "num_seqs": S, "kv_tokens": int(b.kv_lens.sum()),
+                   **({"sinks": args.sinks, "window": args.window} if contiguous else {})},
         "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS,
                      "traffic": None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
                      "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
@@ -245,7 +259,8 @@ def page_attention_main(args):
             ids = torch.tensor(sorted(cand[:n]))
             a = [to_np(t[ids.to(dev)]) for t in b.args()]
             t0 = time.perf_counter()
-            ref = ragged_decode_strict(*a, softmax_scale=b.softmax_scale, block_size=int(m["seq_len"]))
+            ref = ragged_decode_strict(*a, softmax_scale=b.softmax_scale, block_size=int(m["seq_len"]),
+                                       sliding_window=window, softmax_aux=None if aux is None else to_np(aux))
             dt = time.perf_counter() - t0
             rows_idx, kv_tokens = ids, int(b.kv_lens[ids.numpy()].sum())
             what = ("NumPy restatement of the reference's XLA scan with one KV block per sequence (bf16 op by op)")
