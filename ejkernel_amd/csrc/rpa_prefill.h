@@ -13,8 +13,8 @@
 // operand read from LDS feeds MRT MFMAs, Q stays in registers, and each lane owns one row per row
 // tile, so the online softmax is lane-local as in the decode loop.  The row sums come from one
 // extra MFMA against a vector of ones (they add exactly the bf16 probabilities that enter P V).
-// Logits stay in fp32 here (the decode loop rounds them to bf16 as the reference does; on prefill
-// tiles that rounding only costs vector instructions: against the reference restatement the mean
+// Logits stay in fp32 here unless a soft cap follows (the decode loop rounds them to bf16 as the reference does; on
+// prefill tiles that rounding only costs vector instructions: against the reference restatement the mean
 // error moves from 4e-4 to 5.5e-4 of a 2e-3 budget).  The K operands of a half are requested one
 // half ahead and the barrier that publishes the next tile sits before the last P V of a tile, so
 // LDS latency and barrier skew hide behind matrix work.  Halves of a step that lie entirely in a
@@ -366,8 +366,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-                sv[u][r] = soft_cap<kMimic>(sv[u][r], cap, inv_cap);
+              for (int r = 0; r < 4; ++r)  // the cap's own bf16 roundings make it sensitive to its input: round that too
+                sv[u][r] = soft_cap<kMimic>(kMimic ? rbf(sv[u][r]) : sv[u][r], cap, inv_cap);
           }
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
           const bool need_mask = a0 <= clear_lo[m] || a0 > clear_hi[m];
