@@ -14,7 +14,7 @@ from ejkernel_amd import _native
 from ejkernel_amd.modules import PageAttentionConfig, page_attention
 from ejkernel_amd.workloads import make_page_attention_batch, page_attention_subset, page_attention_workload
 from oracle.page_attention_oracle import page_attention_exact, page_attention_strict
-from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, to_np
+from tests.helpers import F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, to_np
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -133,3 +133,22 @@ def test_full_size_workload(name, n_sample):
     sub = page_attention_subset(b, ids)
     ref = page_attention_strict(*np_args(sub), attn_scale=b.attn_scale)
     assert_bf16_parity(to_np(out[sub.meta["rows"].to(DEV)]), ref, len(ids), name)
+
+
+@pytest.mark.parametrize("seed", range(200, 216))
+def test_bf16_random_batches(seed):
+    """Seeded random shapes on both paths against the restatement of the reference program (explicit scale)."""
+    rng = np.random.default_rng(seed)
+    hq, hkv = [(8, 2), (4, 4), (16, 2), (32, 8), (8, 1), (40, 1), (12, 4)][rng.integers(7)]
+    D = int(rng.choice([64, 128, 256]))
+    bs = int(rng.choice([4, 8, 16, 32, 64]))
+    n = int(rng.integers(1, 12))
+    kv = [int(rng.integers(1, 500)) for _ in range(n)]       # context_len 0 is garbage in the reference: not drawn
+    mb = -(-max(kv) // bs) + int(rng.integers(0, 3))
+    b = make_page_attention_batch(kv, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, block_size=bs, max_blocks=mb,
+                                  seed=seed, device=DEV)
+    scale = float(rng.choice([D ** -0.5, 0.05, 0.2]))
+    ref = page_attention_strict(*np_args(b), attn_scale=scale)
+    for flags in (0, _native.RPA_FLAG_FORCE_GENERIC):
+        assert_bf16_parity_stepwise(run_hip(b, flags, attn_scale=scale), ref,
+                                    f"seed {seed}: {hq}/{hkv} D={D} block={bs} kv={kv} scale={scale:.3g} flags={flags}")

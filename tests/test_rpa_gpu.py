@@ -12,7 +12,8 @@ import torch
 from ejkernel_amd import _native
 from ejkernel_amd.modules import RaggedPageAttention, RaggedPageAttentionConfig, ragged_page_attention
 from ejkernel_amd.workloads import Batch, compact_for_host, make_batch, make_workload
-from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, run_exact, run_strict, to_np
+from tests.helpers import (F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, random_rpa_batch,
+                           run_exact, run_strict, to_np)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -244,44 +245,13 @@ def test_bf16_sinks(flags, shape):
     assert np.abs(base - out)[: b.total_valid_tokens].max() > 1e-3  # sinks change the result
 
 
-def _random_batch(seed):
-    """A seeded draw over the argument space: head counts, head_dim, page size, ragged lengths, window, cap."""
-    rng = np.random.default_rng(seed)
-    hq, hkv = [(8, 2), (4, 4), (16, 2), (32, 8), (8, 1), (12, 4)][rng.integers(6)]
-    D = int(rng.choice([64, 128, 256]))
-    page = int(rng.choice([4, 8, 16, 32, 64]))
-    n = int(rng.integers(1, 9))
-    kinds = rng.integers(0, 5, size=n)
-    q_lens, kv_lens = [], []
-    for k in kinds:
-        if k == 0:                       # absent query: the sequence contributes nothing
-            q, prior = 0, int(rng.integers(0, 40))
-        elif k == 1:                     # decode
-            q, prior = 1, int(rng.integers(0, 400))
-        elif k == 2:                     # a few rows
-            q, prior = int(rng.integers(2, 9)), int(rng.integers(0, 200))
-        elif k == 3:                     # prefill chunk with earlier context
-            q, prior = int(rng.integers(20, 150)), int(rng.integers(0, 300))
-        else:                            # prefill from scratch
-            q, prior = int(rng.integers(20, 150)), 0
-        q_lens.append(q)
-        kv_lens.append(q + prior)
-    pps = -(-max(max(kv_lens), 1) // page) + int(rng.integers(0, 3))
-    window = None if rng.random() < 0.5 else int(rng.integers(1, 200))
-    cap = None if rng.random() < 0.6 else float(rng.choice([5.0, 20.0, 50.0]))
-    extra = int(rng.integers(0, 4))
-    b = make_batch(q_lens, kv_lens, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, page_size=page, pages_per_seq=pps,
-                   seed=seed, device=DEV, sliding_window=window, logits_soft_cap=cap, max_num_seqs=n + extra)
-    return b, f"seed {seed}: {hq}/{hkv} D={D} page={page} q={q_lens} kv={kv_lens} W={window} cap={cap}"
-
-
 @pytest.mark.parametrize("seed", range(24))
 def test_bf16_random_batches(seed):
     """Seeded random shapes on the MFMA path and on the scalar path: the parity bound against the op-by-op restatement
     on every row where that is finite (rows it turns NaN -- its first-KV-block defect under a window -- are left to
     the second check), and a bound of 4e-2 / 2e-3 against the float64 evaluation on every row (bf16 logits alone put
     up to 2.5e-2 between the restatement and float64 here)."""
-    b, what = _random_batch(seed)
+    b, what = random_rpa_batch(seed, DEV)
     rows = b.total_valid_tokens
     strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
     finite = np.isfinite(strict).all(axis=(1, 2))
@@ -289,13 +259,7 @@ def test_bf16_random_batches(seed):
         out = to_np(run_hip(b, flags))
         assert np.isfinite(out[:rows]).all(), what
         if finite.any():
-            # the parity bound, widened to two bf16 steps of the value where that is larger: rows that see one or two
-            # keys return values of magnitude 2..8, whose step is 0.016..0.031, and the restatement's chain of bf16
-            # roundings puts it up to 1.5 steps from the float64 value there
-            d = np.abs(out[:rows][finite].astype(np.float64) - strict[finite])
-            ulp = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(strict[finite]), 1e-30))) - 7)
-            assert (d <= np.maximum(2e-2, 2 * ulp)).all() and d.mean() <= 2e-3, \
-                f"{what} flags={flags}: max-abs {d.max():.4g} mean-abs {d.mean():.4g}"
+            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}")
         mx, mean = err_stats(out, exact, rows)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
         assert not out[rows:].any()

@@ -14,7 +14,8 @@ from ejkernel_amd.modules import RaggedPageAttentionv3Config, ragged_page_attent
 from ejkernel_amd.workloads import compact_for_host, make_batch, make_workload, to_v3
 from oracle import rpa_oracle
 from oracle.rpa_v3_oracle import rpa_v3
-from tests.helpers import F32_MAX_ABS, assert_bf16_parity, err_stats, to_np
+from tests.helpers import (F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, random_rpa_batch,
+                           to_np)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -170,3 +171,18 @@ def test_full_size_workload(name, n_sample):
     assert torch.equal(rows_after[pg, pos % page, 1::2], v.values[:total])
     checksum_after = cache.view(torch.int16).sum(dtype=torch.int64).item()
     assert checksum_after != checksum_before
+
+
+@pytest.mark.parametrize("seed", range(100, 116))
+def test_bf16_random_batches(seed):
+    """Seeded random shapes (head_dim 128 and 256) on both paths: the cache bit for bit, the outputs within the parity
+    bound of the restatement (two bf16 steps of the value where that is larger)."""
+    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))
+    rows = b.total_valid_tokens
+    for flags in (0, _native.RPA_FLAG_FORCE_GENERIC):
+        v = to_v3(random_rpa_batch(seed, DEV, head_dims=(128, 256))[0], seed=seed)   # the call updates the cache in place
+        ref_out, ref_cache = oracle(v)
+        out, cache = run_hip(v, flags)
+        assert np.array_equal(to_np(cache), ref_cache), what
+        if rows:
+            assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
