@@ -123,8 +123,12 @@ def _sinks_per_q_head(softmax_aux: torch.Tensor, num_q_heads: int, num_kv_heads:
 
 
 def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tensor:
-    """Per-device workspace, grown on demand; its counters are cleared once per allocation."""
-    key = (device.index if device.index is not None else torch.cuda.current_device(), 0)
+    """Workspace of this (device, stream), grown on demand; its counters are cleared once per allocation.
+
+    Launches that share a workspace must not overlap in time, and launches on different streams may: every stream
+    gets its own.
+    """
+    key = (device.index if device.index is not None else torch.cuda.current_device(), int(stream_ptr))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)

@@ -338,6 +338,24 @@ def test_non_default_stream():
     assert torch.equal(out, base)
 
 
+def test_concurrent_streams_do_not_share_a_workspace():
+    """Two streams run split sequences (partial results and tickets in the workspace) at the same time; each stream has
+    a workspace of its own, so every result equals the one computed alone, bit for bit."""
+    batches = [make_workload("decode_long_context", device=DEV, scale=0.05), make_workload("mixed_prefill_decode", device=DEV, scale=0.1)]
+    alone = [run_hip(b) for b in batches]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    outs = [[], []]
+    for _ in range(8):
+        for k in range(2):
+            with torch.cuda.stream(streams[k]):
+                outs[k].append(ragged_page_attention(*batches[k].args(), **batches[k].kwargs()))
+    torch.cuda.synchronize()
+    for k in range(2):
+        for o in outs[k]:
+            assert torch.equal(o, alone[k])
+
+
 def test_launch_recorded_in_a_hip_graph_replays_correctly():
     """The launch only enqueues (no allocation, no synchronisation, tickets and queue counters left at zero), so it can
     be captured; every replay on new input values must equal the eager result bit for bit."""
