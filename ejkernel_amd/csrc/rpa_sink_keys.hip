@@ -14,6 +14,7 @@
 
 namespace rpa {
 
+constexpr int kSinkWgWaves = 4;                     // (sequence, head) pairs per workgroup, one per wavefront
 constexpr int kSinkGroups = 4;                      // keys in flight per wavefront: one per group of 16 lanes
 constexpr int kSinkLanes = kWave / kSinkGroups;     // lanes that share one key's dot product
 constexpr int kSinkMaxElemsPerLane = 512 / kSinkLanes;  // head_dim <= 512
@@ -22,8 +23,10 @@ constexpr int kSinkMaxElemsPerLane = 512 / kSinkLanes;  // head_dim <= 512
 // attention state (the K and V rows of different keys are independent loads, so four are in flight at a time);
 // the four states are merged at the end.
 template <typename T, bool kBf16Compute>
-__global__ __launch_bounds__(kWave) void sink_keys_kernel(RpaParams p, KvLayout kvl, SinkKeyArgs sk) {
-  const int s = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+__global__ __launch_bounds__(kSinkWgWaves * kWave) void sink_keys_kernel(RpaParams p, KvLayout kvl, SinkKeyArgs sk) {
+  // workgroups of several wavefronts: launching one workgroup per (sequence, head) costs more than the work itself
+  const int s = blockIdx.x, h = blockIdx.y * kSinkWgWaves + threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  if (h >= p.num_q_heads) return;
   const int grp = lane / kSinkLanes, l16 = lane % kSinkLanes;
   const int D = p.head_dim;
   const int G = p.num_q_heads / p.num_kv_heads;
@@ -122,7 +125,7 @@ __global__ __launch_bounds__(kWave) void sink_keys_kernel(RpaParams p, KvLayout 
 int launch_sink_keys(const RpaParams& p, const KvLayout& kv, const SinkKeyArgs& sk, hipStream_t stream) {
   if (p.head_dim > kSinkMaxElemsPerLane * kSinkLanes) return RPA_ERR_UNSUPPORTED;
   if (p.total_tokens == 0) return RPA_OK;
-  dim3 grid(p.total_tokens, p.num_q_heads), block(kWave);
+  dim3 grid(p.total_tokens, (p.num_q_heads + kSinkWgWaves - 1) / kSinkWgWaves), block(kSinkWgWaves * kWave);
   const size_t lds = 0;
   const bool bf16c = p.compute == RPA_COMPUTE_BF16;
   if (p.dtype == RPA_DTYPE_BF16) {
