@@ -18,6 +18,7 @@ RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
 RPA_FLAG_FP32_LOGITS = 2
+RPA_FLAG_PREFILL_TILES = 4
 
 EXPORTED_SYMBOLS = (
     "rpa_abi_version",

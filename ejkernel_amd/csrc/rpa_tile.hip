@@ -36,7 +36,7 @@ constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles tha
 constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
 constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
-constexpr int kDecodeShapedPadRows = 16; // token rows beyond one per sequence slot that still count as a decode batch
+constexpr int kWaveOnlyMaxRows = 20480;   // (token, query head) rows up to which a batch runs without prefill tiles
 
 // Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 8 ints of scratch and the sequences with prefill
 // tiles in order of length (up to kSortMax ints), then the data region
@@ -48,9 +48,9 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 }
 
 // kWaveOnly: the prefill tiles are compiled out and sequences with many row tiles run as wave-level items too (right
-// for every batch, slow for long prefill chunks).  That leaves the decode loop a register allocation of its own, about
-// 2 % faster on decode batches, which is why the host picks this instantiation for batches shaped like decode; it is
-// also the one that merges an attention state in a.pre into every row.
+// for every batch, slow for large prefill batches).  That leaves the decode loop a register allocation of its own, about
+// 2 % faster on decode batches, and spreads short prefill chunks over more wavefronts, which is why the host picks
+// this instantiation for small batches; it is also the one that merges an attention state in a.pre into every row.
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
   using C = Cfg<D, NT, kMimic>;
@@ -455,10 +455,14 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, con
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
-  // Decode-shaped batches -- one query token per sequence by construction, or a token buffer with no more rows than
-  // sequence slots plus the padding such buffers carry -- take the instantiation without prefill tiles.
-  const bool decode_shaped = p.query_start_loc == nullptr || p.total_tokens <= p.max_num_seqs + kDecodeShapedPadRows;
-  const bool wave_only = pre.ml != nullptr || (decode_shaped && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
+  // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
+  // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
+  // alone gets a register allocation without spills, and short prefill chunks spread over four times as many
+  // wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
+  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
+  const bool small_batch = p.query_start_loc == nullptr || ((p.flags & RPA_FLAG_PREFILL_TILES) == 0 &&
+                                                            rows <= env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows));
+  const bool wave_only = pre.ml != nullptr || (small_batch && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
   if (wave_only) {
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);

@@ -48,6 +48,9 @@ extern "C" {
 #define RPA_FLAG_FP32_LOGITS 2u   /* the arithmetic of ragged_page_attention_v3 (_kernel.py:228-262): q enters the   */
                                   /* contraction unscaled, logits stay fp32 and are scaled after it, probabilities  */
                                   /* are rounded to the cache dtype before P V                                      */
+#define RPA_FLAG_PREFILL_TILES 4u /* long chunks run as 128-row workgroup tiles whatever the size of the batch (by   */
+                                  /* default batches of up to 20480 (token, query head) rows run them as 16-row      */
+                                  /* wave-level items, which fills the device better when the tiles would be few)    */
 
 typedef struct RpaParams {
   /* ---- device buffers (argument names follow ragged_page_attention.py:540-547) ---- */

@@ -79,7 +79,7 @@ def _check(out, expected_bits, rows):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("flags", [0, 1], ids=["tiled", "generic"])
+@pytest.mark.parametrize("flags", [0, 4, 1], ids=["tiled", "tiles", "generic"])
 def test_device_kernels_against_the_frozen_outputs(flags):
     from ejkernel_amd.modules import (RaggedPageAttention, RaggedPageAttentionConfig, page_attention,
                                       ragged_decode_attention, ragged_page_attention_v3)
