@@ -205,12 +205,15 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
                           static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+      // Buffer addressing (scalar base in a resource descriptor, 32-bit per-lane offset): a wavefront is held for
+      // about 50 cycles per direct-to-LDS load it issues this way, against about 100 with 64-bit per-lane addresses.
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(sbase), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
       for (int n = 0; n < HB; ++n) {
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + pre_off[n]),
-                                         (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + v_src_off(n)),
-                                         (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + n * 1024), 16,
+                                                 pre_off[n], 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024),
+                                                 16, v_src_off(n), 0, 0, 0);
       }
       return;
     }
@@ -344,8 +347,16 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
                                                                     s_acc[m][u], 0, 0, 0);
         }
         load_v(0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 2 * C::NKS * MRT, 0);  // QK MFMAs
-        __builtin_amdgcn_sched_group_barrier(0x100, V_READS, 0);           // V of slice 0
+        {
+          // the V reads issue between the QK MFMAs, in the shadow of the matrix pipe, not after them
+          constexpr int N_MFMA = 2 * C::NKS * MRT, PER_READ = N_MFMA / V_READS;
+          static_assert(PER_READ >= 1 && PER_READ * V_READS == N_MFMA, "MFMAs per V read");
+#pragma unroll
+          for (int r = 0; r < V_READS; ++r) {
+            __builtin_amdgcn_sched_group_barrier(0x008, PER_READ, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          }
+        }
         __builtin_amdgcn_sched_barrier(0);
         // online softmax per row tile; this lane: row i of the tile, keys a0 + 16u + 4g + r
 #pragma unroll
