@@ -42,6 +42,8 @@ def parse():
                          "page_attention = the decode workloads (decode_small, decode_llama3_8b) with separate K and V "
                          "caches of [blocks, kv heads, block, head_dim]; ragged_decode = ragged_decode_attention on the "
                          "same lengths with contiguous K and V of [batch, seq_len, kv heads, head_dim]")
+    ap.add_argument("--cache-dtype", default="same", choices=["same", "fp8"],
+                    help="--op rpa_v3: dtype of the cache and of the new K/V rows; fp8 = float8_e4m3fn with bf16 queries")
     ap.add_argument("--sinks", type=int, default=0,
                     help="--op ragged_decode: attention sinks (softmax_aux of this many biases, shared by all heads)")
     ap.add_argument("--window", type=int, default=0,
@@ -138,13 +140,15 @@ def cpu_sample_and_parity_v3(batch, v3, out, want_baseline, want_parity, n_seqs,
 
     def run(ids):
         sub = compact_for_host(batch, sorted(ids))
-        sv = to_v3(sub)
+        fp8 = v3.kv_cache.dtype != v3.queries.dtype
+        sv = to_v3(sub, cache_dtype=v3.kv_cache.dtype if fp8 else None)
         rows_idx = sub.meta["rows"]
         sv.keys[: len(rows_idx)] = v3.keys[rows_idx.to(v3.keys.device)].cpu()
         sv.values[: len(rows_idx)] = v3.values[rows_idx.to(v3.keys.device)].cpu()
         a = [to_np(x) for x in sv.args()]
         t0 = time.perf_counter()
-        ref, _ = rpa_v3(*a, **sv.kwargs())
+        dt = dict(cache_dtype="float8_e4m3fn", query_dtype="bfloat16") if fp8 else {}
+        ref, _ = rpa_v3(*a, **sv.kwargs(), **dt)
         return sub, ref, time.perf_counter() - t0
 
     if n_seqs <= 0:
@@ -327,9 +331,13 @@ def main():
         from ejkernel_amd.modules import ragged_page_attention_v3
         from ejkernel_amd.workloads import to_v3
 
-        v3 = to_v3(batch, seed=1)
+        fp8 = args.cache_dtype == "fp8"
+        v3 = to_v3(batch, seed=1, cache_dtype=torch.float8_e4m3fn if fp8 else None)
+        if fp8:  # the algorithmic minimum reads every visible K/V row once, at one byte per element
+            counts["bytes"] -= counts["kv_bytes"] // 2
+            counts["kv_bytes"] //= 2
         # the new rows are read once and written once into the cache, on top of the attention traffic
-        row_bytes = 2 * m["num_kv_heads"] * m["head_dim"] * 2
+        row_bytes = 2 * m["num_kv_heads"] * m["head_dim"] * (1 if fp8 else 2)
         counts["bytes"] += 2 * counts["tokens"] * row_bytes
 
     def step():

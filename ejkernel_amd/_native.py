@@ -13,8 +13,8 @@ from pathlib import Path
 # RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
-RPA_ABI_VERSION = 4
-RPA_DTYPE_BF16, RPA_DTYPE_F32 = 0, 1
+RPA_ABI_VERSION = 5
+RPA_DTYPE_BF16, RPA_DTYPE_F32, RPA_DTYPE_FP8_E4M3 = 0, 1, 2
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
 RPA_FLAG_FP32_LOGITS = 2
@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "rpa_workspace_init",
     "rpa_fwd_launch",
     "rpa_v3_launch",
+    "rpa_v3_workspace_bytes",
     "rpa_page_attention_workspace_bytes",
     "rpa_page_attention_launch",
     "rpa_ragged_decode_workspace_bytes",
@@ -81,6 +82,8 @@ class RpaV3Params(ctypes.Structure):
         ("attn", RpaParams),
         ("new_keys", ctypes.c_void_p),
         ("new_values", ctypes.c_void_p),
+        ("cache_dtype", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 
@@ -176,6 +179,8 @@ def load() -> ctypes.CDLL:
     lib.rpa_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     lib.rpa_fwd_launch.restype = ctypes.c_int
     lib.rpa_fwd_launch.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
+    lib.rpa_v3_workspace_bytes.restype = ctypes.c_uint64
+    lib.rpa_v3_workspace_bytes.argtypes = [ctypes.POINTER(RpaV3Params)]
     lib.rpa_v3_launch.restype = ctypes.c_int
     lib.rpa_v3_launch.argtypes = [ctypes.POINTER(RpaV3Params), ctypes.c_void_p]
     lib.rpa_page_attention_workspace_bytes.restype = ctypes.c_uint64

@@ -282,6 +282,14 @@ static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStrea
 }
 }  // namespace rpa
 
+uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims) {
+  if (dims == nullptr) return 0;
+  const uint64_t base = rpa_workspace_bytes(&dims->attn);
+  if (base == 0 || dims->cache_dtype != RPA_DTYPE_FP8_E4M3) return base;
+  const uint64_t rows = static_cast<uint64_t>(dims->attn.total_tokens > 0 ? dims->attn.total_tokens : 0) * dims->attn.num_q_heads;
+  return ((base + 255) & ~255ull) + ((rows * 8 + 255) & ~255ull);
+}
+
 int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
   RpaV3Params v = *params;
@@ -290,11 +298,44 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (rc != RPA_OK) return rc;
   if (!v.new_keys || !v.new_values) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null new_keys / new_values");
   if (v.attn.num_sinks != 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "ragged_page_attention_v3 has no sinks");
-  rc = rpa::launch_kv_cache_update(v, static_cast<hipStream_t>(hip_stream));
+  const bool fp8 = v.cache_dtype == RPA_DTYPE_FP8_E4M3;
+  if (!fp8 && v.cache_dtype != v.attn.dtype)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_dtype=%d: the cache has the dtype of the queries (%d) or is RPA_DTYPE_FP8_E4M3",
+                     v.cache_dtype, v.attn.dtype);
+  hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  if (fp8) {
+    if (v.attn.dtype != RPA_DTYPE_BF16 || v.attn.compute != RPA_COMPUTE_BF16)
+      return rpa::fail(RPA_ERR_UNSUPPORTED, "an 8-bit cache takes bf16 queries and RPA_COMPUTE_BF16");
+    if (!rpa::tiled_supported(v.attn))
+      return rpa::fail(RPA_ERR_UNSUPPORTED,
+                       "an 8-bit cache runs on the MFMA kernel only (head_dim 64 / 128 / 256, page_size a power of two >= 4, "
+                       "no RPA_FLAG_FORCE_GENERIC)");
+    const uint64_t need = rpa_v3_workspace_bytes(&v);
+    if (v.attn.workspace == nullptr || v.attn.workspace_bytes < need)
+      return rpa::fail(RPA_ERR_WORKSPACE, "workspace of %llu bytes is too small, rpa_v3_workspace_bytes() asks for %llu",
+                       (unsigned long long)v.attn.workspace_bytes, (unsigned long long)need);
+  }
+  rc = rpa::launch_kv_cache_update(v, stream);
   if (rc == RPA_ERR_UNSUPPORTED)
     return rpa::fail(rc, "head_dim=%d rows are not a multiple of 16 bytes", v.attn.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "cache update launch failed: %s", hipGetErrorString(hipGetLastError()));
-  return rpa_fwd_launch(&v.attn, hip_stream);
+  if (!fp8) return rpa_fwd_launch(&v.attn, hip_stream);
+
+  const RpaParams& p = v.attn;
+  rpa::KvLayout kv;
+  kv.k_base = static_cast<const char*>(p.kv_pages);
+  kv.v_base = kv.k_base + p.head_dim;
+  kv.stride_b = 2u * p.num_kv_heads * p.head_dim;
+  kv.page_b = static_cast<uint64_t>(p.page_size) * kv.stride_b;
+  kv.head_b = 2u * p.head_dim;
+  kv.contiguous = 0;
+  const uint64_t base = (rpa_workspace_bytes(&p) + 255) & ~255ull;
+  float* stats = reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base);
+  RpaParams q = p;
+  q.workspace_bytes = base;
+  rc = rpa::launch_tiled_fp8(q, kv, stats, stream);
+  if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
+  return RPA_OK;
 }
 
 }  // extern "C"

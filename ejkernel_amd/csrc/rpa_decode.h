@@ -1,6 +1,8 @@
 // Wave-level attention loop: one wavefront streams a key range of one (sequence, kv head) for up to 16 rows.
 #pragma once
 
+#include <type_traits>
+
 #include "rpa_tile_common.h"
 
 namespace rpa {
@@ -15,10 +17,41 @@ struct Cfg {
   static constexpr int LDS_PER_WAVE = TT * ROWB;
 };
 
+// Cache element types (kKv): 0 = the query dtype (bf16), 1 = 8-bit float, OCP e4m3 (finite, no infinities).
+// Eight e4m3 elements in two dwords -> the same eight values as bf16 in four dwords (exact).
+__device__ __forceinline__ u32x4_t fp8x8_to_bf16x8(u32x2_t w) {
+  u32x4_t o;
+#pragma unroll
+  for (int d = 0; d < 2; ++d) {
+    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w[d]), false);  // bytes 0, 1
+    const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w[d]), true);   // bytes 2, 3
+    o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(lo[1]), __float_as_uint(lo[0]), 0x07060302u);
+    o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(hi[1]), __float_as_uint(hi[0]), 0x07060302u);
+  }
+  return o;
+}
+// Bytes 2 half, 2 half + 1 of a dword as floats (the half must fold to a constant: the instruction encodes it).
+__device__ __forceinline__ auto fp8_pair(uint32_t w, int half) {
+  const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
+  const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
+  return half ? hi : lo;
+}
+// Two floats rounded to e4m3 (nearest even; the callers keep them inside +-448) and back.
+__device__ __forceinline__ void round_fp8x2(float& a, float& b) {
+  const int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+  const auto f = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+  a = f[0];
+  b = f[1];
+}
+
 // Everything one wavefront needs for one work item.  kWaveOnly: the state in TileArgs::pre, if any, is merged into
 // every row (only in the kernel instantiation without prefill tiles, so that the common one keeps its register
 // allocation).
-template <int D, int NT, bool kMimic, bool kWaveOnly = false>
+// kPass: 0 = attention with the online softmax.  An 8-bit cache takes the reference's rounding of the *normalised*
+// probabilities to the cache dtype (ragged_page_attention_v3, _kernel.py:279), which needs the row maximum and sum
+// before the first P V product, so it runs as two launches: 1 = row statistics only (maximum and sum of exp over
+// the visible keys, written to TileArgs::stats), 2 = P = round(exp(s - m) / l) with m, l from there, O = P V.
+template <int D, int NT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
                                              int j, int rt, int range_lo, int range_hi, const Part& part) {
   using C = Cfg<D, NT, kMimic>;
@@ -27,7 +60,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const int i = lane & 15, g = lane >> 4;
   const int G = p.num_q_heads / p.num_kv_heads;
   const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
-  const bf16_t* __restrict__ kv = static_cast<const bf16_t*>(p.kv_pages);
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
   const int W = p.sliding_window;
 
@@ -58,8 +90,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
-                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
+        float q0 = q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale);
+        float q1 = q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale);
+        if (kKv == 1 && p.q_scale > 0.f) {
+          // q / q_scale in the query dtype, clipped to the cache dtype's range and cast to it (_kernel.py:249-254)
+          q0 = fminf(fmaxf(rbf(q0), -448.f), 448.f);
+          q1 = fminf(fmaxf(rbf(q1), -448.f), 448.f);
+          round_fp8x2(q0, q1);
+        }
+        sc[e] = pack_bf16x2(q0, q1);
       }
       qreg[ks] = __builtin_bit_cast(bf16x8_t, sc);
     }
@@ -72,6 +111,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
+  float m_fix = 0.f, inv_l = 0.f;  // kPass == 2: the row's maximum and 1 / sum from the statistics launch
+  if constexpr (kPass == 2) {
+    const size_t idx = static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head;
+    const float ms = a.stats[2 * idx], ls = a.stats[2 * idx + 1];
+    m_fix = ms == -INFINITY ? 0.f : ms;
+    inv_l = ls > 0.f ? 1.f / ls : 0.f;
+    m_run = 0.f;  // every part carries the same reference point: parts merge by plain addition
+    l_run = 0.f;
+  }
 
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
   // Same row through the constant address space: reads with a wave-uniform index become scalar loads, which
@@ -81,8 +129,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const float cap = p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
 
-  u32x4_t kreg[C::NSLOT][C::NS];
-  u32x4_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
+  using raw_t = typename std::conditional<kKv == 1, u32x2_t, u32x4_t>::type;  // one lane's piece: eight elements
+  constexpr uint32_t PIECE_B = kKv == 1 ? 8u : 16u, SLICE_B = 16u * PIECE_B;
+  raw_t kreg[C::NSLOT][C::NS];
+  raw_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
 
   // Fetch K and V of the TT tokens starting at `tile`: lane (i, g) takes tokens 16u + 4g + r (u < NT, r < 4),
   // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.
@@ -98,8 +148,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const uint64_t page_b = a.kv.page_b;
   const uint32_t head_off = static_cast<uint32_t>(j) * a.kv.head_b;
   const int piece = i & (hd / 8 - 1);  // i itself from head_dim 128 up
-  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + static_cast<uint32_t>(16 * piece);
-  auto issue_loads = [&](int tile, u32x4_t (&kr)[C::NSLOT][C::NS], u32x4_t (&vr)[C::NSLOT][C::NS]) {
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + PIECE_B * static_cast<uint32_t>(piece);
+  auto issue_loads = [&](int tile, raw_t (&kr)[C::NSLOT][C::NS], raw_t (&vr)[C::NSLOT][C::NS]) {
     if (a.uniform_page && tile + C::TT <= range_hi) {
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
@@ -114,8 +164,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const char* row_v = row + v_delta;
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN) {
-            kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + (lane_off + 256u * sN));
-            vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row_v + (lane_off + 256u * sN));
+            kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + (lane_off + SLICE_B * sN));
+            if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row_v + (lane_off + SLICE_B * sN));
           }
         }
       }
@@ -128,28 +178,32 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       int page = a.kv.contiguous ? s : bt[t4c >> a.page_shift];
       page = min(max(page, 0), p.num_pages - 1);
       const char* base = kvb + static_cast<uint64_t>(page) * page_b +
-                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + 16 * piece);
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + PIECE_B * piece);
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
-          kr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + 256 * sN);
-          vr[4 * u + r][sN] = *reinterpret_cast<const u32x4_t*>(row + v_delta + 256 * sN);
+          kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + SLICE_B * sN);
+          if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + v_delta + SLICE_B * sN);
         }
       }
     }
   };
 
-  auto body = [&](int tile, u32x4_t (&vcur)[C::NSLOT][C::NS], u32x4_t (&vnext)[C::NSLOT][C::NS]) {
+  auto body = [&](int tile, raw_t (&vcur)[C::NSLOT][C::NS], raw_t (&vnext)[C::NSLOT][C::NS]) {
     // 1. K rows to the wave-private LDS tile: row = token within the tile, 16-byte piece i (+16 per slice)
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
-        for (int sN = 0; sN < C::NS; ++sN)
-          *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kreg[4 * u + r][sN];
+        for (int sN = 0; sN < C::NS; ++sN) {
+          u32x4_t kw;
+          if constexpr (kKv == 1) kw = fp8x8_to_bf16x8(kreg[4 * u + r][sN]);
+          else kw = kreg[4 * u + r][sN];
+          *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kw;
+        }
     // 2. next tile's K and V are requested now, a full iteration before they are needed
     if (tile + C::TT < range_hi) issue_loads(tile + C::TT, kreg, vnext);
     // 3. S^T = K Q^T: lane (token i of sub-tile u, group g) reads piece 4 ks + g of its row
@@ -189,6 +243,20 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           sv[u][r] = keep ? sv[u][r] : -INFINITY;
         }
     }
+    uint32_t pw[2 * NT];
+    if constexpr (kPass == 2) {
+      // normalised probabilities, rounded to the cache dtype
+#pragma unroll
+      for (int u = 0; u < NT; ++u) {
+        float pv[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) pv[r] = __builtin_amdgcn_exp2f((sv[u][r] - m_fix) * kLog2e) * inv_l;
+        round_fp8x2(pv[0], pv[1]);
+        round_fp8x2(pv[2], pv[3]);
+        pw[2 * u] = (__float_as_uint(pv[0]) >> 16) | (__float_as_uint(pv[1]) & 0xffff0000u);
+        pw[2 * u + 1] = (__float_as_uint(pv[2]) >> 16) | (__float_as_uint(pv[3]) & 0xffff0000u);
+      }
+    } else {
     float tmax = -INFINITY;
 #pragma unroll
     for (int u = 0; u < NT; ++u)
@@ -199,7 +267,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     const float m_use = m_new == -INFINITY ? 0.f : m_new;
     const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
     float psum = 0.f;
-    uint32_t pw[2 * NT];
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       float pv[4];
@@ -208,7 +275,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         float d = sv[u][r] - m_use;
         if (kMimic) d = rbf(d);
         float e = __builtin_amdgcn_exp2f(d * kLog2e);
-        e = rbf(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
+        if (kPass == 0) e = rbf(e);  // probabilities enter P V as bf16, and the row sum adds the same rounded values
         pv[r] = e;
         psum += e;
       }
@@ -217,12 +284,14 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     }
     l_run = l_run * alpha + psum;
     m_run = m_new;
-    if (__any(alpha != 1.f)) {
+    if (kPass == 0 && __any(alpha != 1.f)) {
 #pragma unroll
       for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
         for (int c = 0; c < 8; ++c) o_acc[sN][c] *= alpha;
     }
+    }
+    if constexpr (kPass == 1) return;  // statistics only: no P V
     // 5. O^T += V^T P^T.  MFMA number c of slice sN yields d = 128 sN + 8 (row of the MFMA) + c; its A operand is
     //    column c of every fetched 8-wide piece, gathered from the token rows by byte permutes.
 #pragma unroll
@@ -232,8 +301,16 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
         uint32_t aw[2 * NT];
 #pragma unroll
-        for (int h = 0; h < 2 * NT; ++h)
-          aw[h] = __builtin_amdgcn_perm(vcur[2 * h + 1][sN][c >> 1], vcur[2 * h][sN][c >> 1], sel);
+        for (int h = 0; h < 2 * NT; ++h) {
+          if constexpr (kKv == 1) {
+            // elements c of the two tokens' pieces: byte c of each piece, widened (bf16 = upper half of the float)
+            const auto f1 = fp8_pair(vcur[2 * h + 1][sN][c >> 2], (c >> 1) & 1);
+            const auto f0 = fp8_pair(vcur[2 * h][sN][c >> 2], (c >> 1) & 1);
+            aw[h] = __builtin_amdgcn_perm(__float_as_uint(f1[c & 1]), __float_as_uint(f0[c & 1]), 0x07060302u);
+          } else {
+            aw[h] = __builtin_amdgcn_perm(vcur[2 * h + 1][sN][c >> 1], vcur[2 * h][sN][c >> 1], sel);
+          }
+        }
         if constexpr (NT == 2) {
           const u32x4_t av = {aw[0], aw[1], aw[2], aw[3]};
           const u32x4_t pvv = {pw[0], pw[1], pw[2], pw[3]};
@@ -258,7 +335,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   }
 
   // ---- row sum across the four lane groups
-  l_run = row_groups_sum(l_run);
+  if constexpr (kPass != 2) l_run = row_groups_sum(l_run);
 
   if (part.partial) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
@@ -268,6 +345,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     const size_t slot = static_cast<size_t>(part.slot);
     if (row_valid) {
       uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
+      if constexpr (kPass != 1)
 #pragma unroll
       for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -324,6 +402,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const size_t sl = part_slot(min(k0 + c, part.last_w), part.stream_a, part.sh);
           mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
+          if constexpr (kPass != 1)
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -340,6 +419,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const float lk = __uint_as_float(static_cast<uint32_t>(mlv[c] >> 32));
           const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
           L += w * lk;
+          if constexpr (kPass != 1)
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -359,7 +439,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 
   // ---- normalise (with optional sinks) and store
   if (!row_valid) return;
-  if (kWaveOnly && a.pre.ml != nullptr) {
+  if constexpr (kPass == 1) {
+    if (g == 0) {
+      float* st = a.stats + 2 * (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head);
+      st[0] = m_run;
+      st[1] = l_run;
+    }
+    return;
+  }
+  if (kWaveOnly && kPass == 0 && a.pre.ml != nullptr) {
     // keys an earlier kernel accumulated for this (token, head): one more part
     const size_t idx = static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head;
     const float ms = a.pre.ml[2 * idx], ls = a.pre.ml[2 * idx + 1];
@@ -395,7 +483,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     num_scale = m_run == -INFINITY ? 0.f : expf(m_run - mt);
     denom = num_scale * l_run + ssum;
   }
-  const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
+  const float inv = kPass == 2 ? out_scale(p) : num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
   bf16_t* orow = out + q_row_off;
 #pragma unroll
   for (int sN = 0; sN < C::NS; ++sN)

@@ -51,7 +51,7 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 // for every batch, slow for large prefill batches).  That leaves the decode loop a register allocation of its own, about
 // 2 % faster on decode batches, and spreads short prefill chunks over more wavefronts, which is why the host picks
 // this instantiation for small batches; it is also the one that merges an attention state in a.pre into every row.
-template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false>
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -329,7 +329,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         const int range_lo = max(p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0, si.start) & ~(C::TT - 1);
         Part part;
         part.partial = false;
-        process_item<D, NT, kMimic, kWaveOnly>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+        process_item<D, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
       }
 
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
@@ -368,7 +368,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           part.last_w = sh.owner(part.stream_a + per_head - 1);
           part.partial = part.first_w != part.last_w;
           part.slot = part_slot(worker, part.stream_a, sh);
-          process_item<D, NT, kMimic, kWaveOnly>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+          process_item<D, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
           x += t1 - t0;
         }
       }
@@ -414,7 +414,7 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
 }
 
-template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false>
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<D, NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -425,16 +425,16 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
   if (allowed[dev].load(std::memory_order_acquire) < lds) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
       return RPA_ERR_LAUNCH;
     allowed[dev].store(lds, std::memory_order_release);
   }
-  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly>), dim3(grid), dim3(kWgThreads), lds, stream, a);
+  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass>), dim3(grid), dim3(kWgThreads), lds, stream, a);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
-int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
+static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre, float* stats) {
   WorkspaceLayout wl;
   tiled_workspace_layout(p, &wl);
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
@@ -442,6 +442,7 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, con
   a.p = p;
   a.kv = kv;
   a.pre = pre;
+  a.stats = stats;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
   a.page_shift = __builtin_ctz(p.page_size);
@@ -454,6 +455,17 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, con
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
+  if (stats != nullptr) {
+    // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities; both launches run
+    // every sequence through the wave-level loop.  A wavefront has half the bytes in flight that it has with a
+    // 16-bit cache, so both workgroups of a compute unit stream (0.70 ms against 0.84 ms on 256 x 512..8192 keys).
+    a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 2));
+    int rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
+                               : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
+    if (rc != RPA_OK) return rc;
+    return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
+                             : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
+  }
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
   // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
   // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
@@ -471,6 +483,13 @@ int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, con
   if (p.head_dim <= 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);
+}
+
+int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
+  return launch_tiled_impl(p, kv, stream, pre, nullptr);
+}
+int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, float* stats, hipStream_t stream) {
+  return launch_tiled_impl(p, kv, stream, PreState(), stats);
 }
 
 }  // namespace rpa

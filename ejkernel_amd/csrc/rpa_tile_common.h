@@ -31,6 +31,7 @@ struct TileArgs {
   uint32_t* counters; // split tickets [max_num_seqs * num_kv_heads], then the queue counters; zero between launches
   float* partial_o;   // [2 * wavefronts of the grid][16][D]
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
+  float* stats;       // row maximum and row sum per (token, query head) of a two-launch call (null otherwise)
   PreState pre;       // state accumulated by an earlier kernel, merged by the wave-level loop (null: none)
 };
 

@@ -77,8 +77,16 @@ def _static_validate(q, k, v, kv_cache, kv_lens, block_tables, query_start_loc, 
         raise ValueError(f"head_dim={d} must be a multiple of 128 here (a padded cache row is not supported)")
     if hx2_per_pack * pack != 2 * hkv:
         raise ValueError("a cache with padded combined heads is not supported")
-    if not (q.dtype == k.dtype == v.dtype == kv_cache.dtype) or q.dtype not in (torch.bfloat16, torch.float32):
-        raise ValueError("queries, keys, values and kv_cache must share one dtype (bfloat16 or float32)")
+    if not (k.dtype == v.dtype == kv_cache.dtype):
+        raise ValueError("keys, values and kv_cache must share one dtype")  # merge_kv asserts it, the update needs it
+    fp8 = kv_cache.dtype == torch.float8_e4m3fn
+    if fp8:
+        if q.dtype != torch.bfloat16:
+            raise ValueError("a float8_e4m3fn cache takes bfloat16 queries")
+    elif q.dtype != kv_cache.dtype or q.dtype not in (torch.bfloat16, torch.float32):
+        raise ValueError("queries, keys, values and kv_cache must share one dtype (bfloat16 or float32), or the cache "
+                         "(with keys and values) is float8_e4m3fn and the queries bfloat16; other 8-bit types are not "
+                         "built")
 
 
 def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, *, softmax_scale,
@@ -141,10 +149,12 @@ def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_
     p.v_scale = 0.0 if v_scale is None else float(v_scale)
     v3.new_keys = keys.data_ptr()
     v3.new_values = values.data_ptr()
+    v3.cache_dtype = _native.RPA_DTYPE_FP8_E4M3 if kv_cache.dtype == torch.float8_e4m3fn else p.dtype
+    v3.reserved = 0
 
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream
-        nbytes = int(lib.rpa_workspace_bytes(ctypes.byref(p)))
+        nbytes = int(lib.rpa_v3_workspace_bytes(ctypes.byref(v3)))
         ws = _workspace(dev, nbytes, stream_ptr)
         p.workspace = ws.data_ptr()
         p.workspace_bytes = ws.numel()

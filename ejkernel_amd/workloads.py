@@ -76,24 +76,27 @@ class V3Batch:
                     logits_soft_cap=self.base.logits_soft_cap)
 
 
-def to_v3(batch: Batch, seed: int = 0) -> V3Batch:
+def to_v3(batch: Batch, seed: int = 0, cache_dtype: torch.dtype | None = None) -> V3Batch:
     """New K/V rows for every query token; the cache shares ``batch.kv_pages``' memory, viewed in five dimensions.
 
     The positions the new tokens will occupy hold random data beforehand, so a missed write shows in the output.
+    With ``cache_dtype`` (an 8-bit float type) the cache is a copy of ``batch.kv_pages`` cast to it, and so are the new rows.
     """
     dev = batch.queries.device
     dtype = batch.queries.dtype
     t_alloc, _, head_dim = batch.queries.shape
     num_pages, page_size, hx2, _ = batch.kv_pages.shape
-    pack = 32 // torch.finfo(dtype).bits
+    cdt = cache_dtype or dtype
+    pack = 32 // torch.finfo(cdt).bits
     gen = torch.Generator(device=dev)
     gen.manual_seed(int(seed) + 7919)
-    keys = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype)
-    values = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype)
+    keys = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype).to(cdt)
+    values = _randn_chunked((t_alloc, hx2 // 2, head_dim), gen, dev, dtype).to(cdt)
     S = int(batch.num_seqs.reshape(-1)[0])
+    pages = batch.kv_pages if cdt == dtype else batch.kv_pages.to(cdt)
     return V3Batch(
         queries=batch.queries, keys=keys, values=values,
-        kv_cache=batch.kv_pages.view(num_pages, page_size, hx2 // pack, pack, head_dim),
+        kv_cache=pages.view(num_pages, page_size, hx2 // pack, pack, head_dim),
         kv_lens=batch.context_lens, block_tables=batch.block_tables.reshape(-1).contiguous(),
         query_start_loc=batch.query_start_loc,
         distribution=torch.tensor([0, 0, S], dtype=torch.int32, device=dev), base=batch)

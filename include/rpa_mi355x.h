@@ -25,11 +25,12 @@
 extern "C" {
 #endif
 
-#define RPA_ABI_VERSION 4
+#define RPA_ABI_VERSION 5
 
 /* element type of queries / kv_pages / out */
 #define RPA_DTYPE_BF16 0
 #define RPA_DTYPE_F32 1
+#define RPA_DTYPE_FP8_E4M3 2 /* OCP e4m3 (finite, no infinities; jnp.float8_e4m3fn): cache of rpa_v3_launch only */
 
 /* arithmetic mode */
 #define RPA_COMPUTE_BF16 0 /* bf16 MFMA contractions, fp32 online softmax, reference rounding points */
@@ -115,6 +116,13 @@ typedef struct RpaV3Params {
                           /* tokens); num_seqs = &distribution[2]; RPA_FLAG_FP32_LOGITS is implied                 */
   const void* new_keys;   /* [total_tokens, num_kv_heads, head_dim], dtype of the cache                            */
   const void* new_values; /* [total_tokens, num_kv_heads, head_dim]                                                */
+  int32_t cache_dtype;    /* dtype of the cache and of the new rows: attn.dtype, or RPA_DTYPE_FP8_E4M3 with bf16    */
+                          /* queries.  An 8-bit cache follows the program's casts (_kernel.py:249-254, :279): with  */
+                          /* q_scale, q / q_scale is rounded to the query dtype, clipped to +-448 and cast to e4m3; */
+                          /* the normalised probabilities are cast to e4m3 before P V.  It runs as two passes over  */
+                          /* the keys (row maximum and sum, then the attention) on the MFMA kernel only, and needs  */
+                          /* rpa_v3_workspace_bytes() of workspace.                                                 */
+  int32_t reserved;       /* 0 */
 } RpaV3Params;
 
 /* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */
@@ -126,6 +134,10 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
 
 /* Enqueues the forward pass on `hip_stream` (a hipStream_t; NULL = default stream). */
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
+
+/* Bytes of workspace rpa_v3_launch needs (rpa_workspace_bytes() of `attn`, plus the row statistics of an 8-bit
+ * cache). */
+uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims);
 
 /* Enqueues the cache update (token t of sequence s goes to position kv_len - q_len + (t - q_start) of s) and then
  * the forward pass, both on `hip_stream`.  Sequences whose block tables share a page that one of them writes see

@@ -68,12 +68,30 @@ def bf16_from_bits(b):
     return (b.astype(np.uint32) << np.uint32(16)).view(np.float32)
 
 
+def fp8_e4m3fn_round(a):
+    """float32 values rounded to the nearest ``float8_e4m3fn`` (ties to even), as float32.
+
+    OCP e4m3: 4 exponent bits (bias 7), 3 mantissa bits, no infinities; normal numbers from 2**-6 to 448,
+    subnormal multiples of 2**-9 below.  A value that rounds past 448 becomes NaN (what the cast does; the
+    callers here clip first).
+    """
+    x = np.asarray(a, dtype=np.float32)
+    _, e = np.frexp(x)  # |x| = m 2**e with m in [0.5, 1): the binade's exponent is e - 1
+    quantum = np.ldexp(np.float32(1.0), np.maximum(e - 1, -6) - 3).astype(np.float32)
+    with np.errstate(invalid="ignore"):
+        y = (np.rint(x / quantum) * quantum).astype(np.float32)
+    y = np.where(np.abs(y) > np.float32(448.0), np.float32(np.nan), y)
+    return np.where(np.isfinite(x), y, np.float32(np.nan)).astype(np.float32)
+
+
 def _rounder(dtype):
     name = np.dtype(dtype).name if not isinstance(dtype, str) else dtype
     if name in ("bfloat16", "bf16"):
         return bf16_round
     if name in ("float32", "f32"):
         return lambda a: np.asarray(a, dtype=np.float32)
+    if name in ("float8_e4m3fn", "fp8_e4m3"):
+        return fp8_e4m3fn_round
     raise ValueError(f"unsupported dtype {dtype!r}")
 
 

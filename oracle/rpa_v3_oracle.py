@@ -28,7 +28,12 @@ Two functions:
     contributes ``exp(S + mask_value - max) == 0`` exactly in float32), usable at
     benchmark sizes.
 
-Arrays are float32 holding values representable in ``cache_dtype``.
+Arrays are float32 holding values representable in their dtype: ``cache_dtype`` for the cache and
+the new keys / values ("bfloat16", "float32" or "float8_e4m3fn"), ``query_dtype`` for the queries
+(the cache dtype unless given; "bfloat16" with an 8-bit cache).  The output takes the query dtype
+(``:190``), ``Q / q_scale`` is computed in it, clipped to the cache dtype's finite range and cast
+to the cache dtype (``:249-254``), and the normalised probabilities are cast to the cache dtype
+(``:279``).
 
 Not restated: what XLA does when a block table repeats a page id among the entries the
 scatter writes (``.at[indices].set`` with duplicate indices has no defined winner) and
@@ -56,7 +61,7 @@ DEFAULT_MASK_VALUE = np.float32(-0.7 * float(np.finfo(np.float32).max))  # _kern
 
 def packing(cache_dtype):
     """32 // bit width (_kernel.py:38-39)."""
-    return 2 if cache_dtype == "bfloat16" else 1
+    return {"bfloat16": 2, "float8_e4m3fn": 4}.get(cache_dtype, 1)
 
 
 def merge_kv(k, v, cache_dtype="bfloat16"):
@@ -76,6 +81,11 @@ def _unpack(flat, num_kv_heads, dalign):
     tcap = flat.shape[0]
     kv = flat.reshape(tcap, -1, dalign)[:, : 2 * num_kv_heads, :].reshape(tcap, num_kv_heads, 2 * dalign)
     return kv[:, :, :dalign], kv[:, :, dalign:]
+
+
+def _clip_to(x, cache_dtype):
+    """jnp.clip(x, finfo.min, finfo.max) of the cache dtype (_kernel.py:251-253): only an 8-bit range cuts anything."""
+    return np.clip(x, np.float32(-448.0), np.float32(448.0)) if cache_dtype == "float8_e4m3fn" else x
 
 
 def _softmax_f32(s):
@@ -100,9 +110,10 @@ def _prep(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_lo
 
 def rpa_v3_literal(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, *,
                    softmax_scale=1.0, sliding_window=None, logits_soft_cap=None, q_scale=None, k_scale=None,
-                   v_scale=None, cache_dtype="bfloat16"):
+                   v_scale=None, cache_dtype="bfloat16", query_dtype=None):
     """Step-by-step restatement (_kernel.py:163-318); returns (out [T, Hq, D], updated cache)."""
     R = _rounder(cache_dtype)
+    Rq = _rounder(query_dtype or cache_dtype)
     queries, keys, values, cache, kv_lens, bt, qsl, num_seqs = _prep(
         queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution)
     T, Hq, D = queries.shape
@@ -137,7 +148,7 @@ def rpa_v3_literal(queries, keys, values, kv_cache, kv_lens, block_tables, query
         iq = q_start + positions
         Q = np.where((iq < T)[:, None, None], queries[np.clip(iq, 0, T - 1)], 0.0).astype(np.float32)
         if q_scale is not None:
-            Q = R(Q / np.float32(q_scale))  # divided in the query dtype, clipped (no-op for floats), cast to K's dtype
+            Q = R(_clip_to(Rq(Q / np.float32(q_scale)), cache_dtype))  # divided in the query dtype, clipped, cast to K's dtype
         S = np.einsum("qhd,khd->hqk", Q, K, dtype=np.float32) * np.float32(softmax_scale)
         if k_scale is not None:
             S = S * np.float32(k_scale)
@@ -155,23 +166,24 @@ def rpa_v3_literal(queries, keys, values, kv_cache, kv_lens, block_tables, query
         if v_scale is not None:
             O = O * np.float32(v_scale)
         O = O * (positions < q_len).astype(np.float32)[:, None, None]
-        blk = R(O[:B])
+        blk = Rq(O[:B])
         if q_start + B <= T:
             out[q_start:q_start + B] = blk
         else:  # scatter-add of the rows that fit (_kernel.py:273-289); the rows it adds to are still zero or are rewritten
             n = T - q_start
-            out[q_start:] = R(out[q_start:] + blk[:n])
+            out[q_start:] = Rq(out[q_start:] + blk[:n])
     return out, cache
 
 
 def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, *,
            softmax_scale=1.0, sliding_window=None, logits_soft_cap=None, q_scale=None, k_scale=None, v_scale=None,
-           cache_dtype="bfloat16", seqs=None):
+           cache_dtype="bfloat16", query_dtype=None, seqs=None):
     """Same results as ``rpa_v3_literal`` from the visible keys only; returns (out, updated cache).
 
     ``seqs`` restricts the attention (not the cache update) to some sequences; the other rows stay zero.
     """
     R = _rounder(cache_dtype)
+    Rq = _rounder(query_dtype or cache_dtype)
     queries, keys, values, cache, kv_lens, bt, qsl, num_seqs = _prep(
         queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution)
     T, Hq, D = queries.shape
@@ -202,7 +214,7 @@ def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_l
         V = rows[:, 1:2 * Hkv:2, :D]
         Q = queries[q_start:q_start + q_len]
         if q_scale is not None:
-            Q = R(Q / np.float32(q_scale))
+            Q = R(_clip_to(Rq(Q / np.float32(q_scale)), cache_dtype))
         Qg = Q.reshape(q_len, Hkv, hrep, D)
         S = np.einsum("qjgd,kjd->jgqk", Qg, K, dtype=np.float32, optimize=True) * np.float32(softmax_scale)
         if k_scale is not None:
@@ -221,5 +233,5 @@ def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_l
         O = np.einsum("jgqk,kjd->qjgd", Pm, V, dtype=np.float32, optimize=True).reshape(q_len, Hq, D)
         if v_scale is not None:
             O = O * np.float32(v_scale)
-        out[q_start:q_start + q_len] = R(O)
+        out[q_start:q_start + q_len] = Rq(O)
     return out, cache

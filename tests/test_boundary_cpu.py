@@ -75,6 +75,37 @@ def test_ragged_decode_sink_arguments_are_checked_before_any_launch():
     assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -3 and b"too small" in lib.rpa_last_error()
 
 
+def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
+    lib = _native.load()
+    v = _native.RpaV3Params()
+    p = v.attn
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = 16, 8, 2, 128
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = 16, 64, 4, 16
+    p.softmax_scale = 0.1
+    p.dtype, p.compute = _native.RPA_DTYPE_BF16, _native.RPA_COMPUTE_BF16
+    v.cache_dtype = _native.RPA_DTYPE_BF16
+    plain = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    assert plain == lib.rpa_workspace_bytes(ctypes.byref(p)) > 0
+    v.cache_dtype = _native.RPA_DTYPE_FP8_E4M3
+    with_stats = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    assert with_stats >= plain + 16 * 8 * 2 * 4              # row maximum and sum per (token, query head)
+    buf = (ctypes.c_char * 64)()
+    addr = ctypes.addressof(buf)                              # never dereferenced: every call below fails first
+    for f in ("queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs", "out", "workspace"):
+        setattr(p, f, addr)
+    v.new_keys = v.new_values = addr
+    p.workspace_bytes = plain
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -3 and b"rpa_v3_workspace_bytes" in lib.rpa_last_error()
+    p.workspace_bytes = with_stats
+    p.flags = _native.RPA_FLAG_FORCE_GENERIC
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -2 and b"MFMA kernel only" in lib.rpa_last_error()
+    p.flags = 0
+    p.dtype, p.compute = _native.RPA_DTYPE_F32, _native.RPA_COMPUTE_F32
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -2 and b"bf16 queries" in lib.rpa_last_error()
+    v.cache_dtype = _native.RPA_DTYPE_BF16                    # a float32 call with a bf16 cache: neither rule holds
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_dtype" in lib.rpa_last_error()
+
+
 def test_workspace_bytes_and_errors_without_gpu():
     lib = _native.load()
     p = _native.RpaParams()

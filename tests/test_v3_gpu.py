@@ -189,3 +189,104 @@ def test_bf16_random_batches(seed):
         assert np.array_equal(to_np(cache), ref_cache), what
         if rows:
             assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
+
+
+# ---------------------------------------------------------------- 8-bit cache (float8_e4m3fn, bf16 queries)
+# The device follows the program's casts (Q / q_scale clipped and cast to the cache dtype, normalised probabilities
+# cast to the cache dtype), so against the restatement the only differences left are float32 evaluation order and
+# the exponential: with 4-bit significands on both sides of P V the sums are exact, and a difference shows only
+# where a probability sits on a rounding boundary.  The bound stays the bf16 one.
+
+F8 = torch.float8_e4m3fn
+
+
+def small_e4m3(q_lens, kv_lens, **kw):
+    args = dict(num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=16, seed=3, device=DEV)
+    args.update(kw)
+    return to_v3(make_batch(q_lens, kv_lens, **args), seed=args["seed"], cache_dtype=F8)
+
+
+def oracle_e4m3(v, **kw):
+    k = dict(v.kwargs())
+    k.update(kw)
+    return rpa_v3(*[to_np(a) for a in v.args()], cache_dtype="float8_e4m3fn", query_dtype="bfloat16", **k)
+
+
+E4M3_CASES = dict(CASES)
+E4M3_CASES["long_decode"] = ([1, 1, 1, 1], [4000, 2500, 4096, 777], dict(pages_per_seq=256))
+
+
+@pytest.mark.parametrize("scales", [{}, dict(q_scale=0.05, k_scale=0.5, v_scale=2.0)], ids=["plain", "scales"])
+@pytest.mark.parametrize("case", list(E4M3_CASES))
+def test_e4m3_cache_parity_and_cache_update(case, scales):
+    q_lens, kv_lens, kw = E4M3_CASES[case]
+    v = small_e4m3(q_lens, kv_lens, **kw)
+    assert v.kv_cache.dtype == F8 and v.keys.dtype == F8 and v.kv_cache.shape[3] == 4
+    ref_out, ref_cache = oracle_e4m3(v, **scales)
+    out, cache = run_hip(v, **scales)
+    assert out.dtype == torch.bfloat16
+    assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
+    rows = int(sum(q_lens))
+    got, ref = to_np(out), ref_out
+    if scales:
+        got, ref = got / 2.0, ref / 2.0          # v_scale doubles the outputs
+    assert_bf16_parity(got, ref, rows, case)
+    assert not out[rows:].any()
+
+
+def test_e4m3_probabilities_below_half_the_smallest_subnormal_vanish():
+    # q = 0 over 1024 keys: p = 2**-10 rounds to zero in e4m3, the row is zero; over 64 keys p = 2**-6 survives and
+    # the row is the mean of V.  An implementation that rounds exp(s - max) instead of the normalised value fails this.
+    for n, zero in ((64, False), (1024, True)):
+        v = small_e4m3([1], [n], pages_per_seq=64)
+        v.queries.zero_()
+        ref_out, _ = oracle_e4m3(v)
+        out, _ = run_hip(v)
+        assert np.array_equal(to_np(out)[:1], ref_out[:1])
+        assert bool(out[:1].any()) != zero
+
+
+def test_e4m3_rejections():
+    v = small_e4m3([2, 1], [20, 30])
+    with pytest.raises(RuntimeError, match="MFMA kernel only"):
+        ragged_page_attention_v3(*v.args(), _flags=_native.RPA_FLAG_FORCE_GENERIC, **v.kwargs())
+    a = list(v.args())
+    with pytest.raises(ValueError, match="share one dtype"):
+        ragged_page_attention_v3(a[0], a[1].to(torch.bfloat16), *a[2:])
+    with pytest.raises(ValueError, match="bfloat16 queries"):
+        ragged_page_attention_v3(a[0].float(), *a[1:])
+    e5 = [a[0]] + [t.to(torch.float32).to(torch.float8_e5m2) for t in a[1:4]] + a[4:]
+    with pytest.raises(ValueError, match="not built"):
+        ragged_page_attention_v3(*e5)
+
+
+@pytest.mark.parametrize("seed", range(200, 212))
+def test_e4m3_random_batches(seed):
+    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))
+    if b.meta["num_kv_heads"] % 2:
+        pytest.skip("an odd number of kv heads pads the packed cache: rejected")
+    rows = b.total_valid_tokens
+    v = to_v3(b, seed=seed, cache_dtype=F8)
+    ref_out, ref_cache = oracle_e4m3(v)
+    out, cache = run_hip(v)
+    assert np.array_equal(to_np(cache), ref_cache), what
+    if rows:
+        assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], what)
+
+
+def test_e4m3_full_size_decode_sample():
+    b = make_workload("decode_llama3_8b", device=DEV)
+    v = to_v3(b, seed=5, cache_dtype=F8)
+    rng = np.random.default_rng(1)
+    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:10])
+    sub = compact_for_host(b, ids)
+    rows_idx = sub.meta["rows"]
+    sub_v = to_v3(sub, seed=0, cache_dtype=F8)
+    sub_v.keys[: len(rows_idx)] = v.keys[rows_idx.to(DEV)].cpu()
+    sub_v.values[: len(rows_idx)] = v.values[rows_idx.to(DEV)].cpu()
+    ref_out, _ = oracle_e4m3(sub_v)
+    out, cache = run_hip(v)
+    out2, _ = run_hip(v)                          # the second call rewrites the same rows: same result, bit for bit
+    assert torch.equal(out, out2)
+    assert_bf16_parity(to_np(out[rows_idx.to(DEV)]), ref_out, sub.total_valid_tokens, "decode_llama3_8b e4m3")
+    assert torch.isfinite(out.float()).all() and not out[b.total_valid_tokens:].any()

@@ -123,3 +123,87 @@ def test_scales_fold_as_the_reference_composes_them():
     c, _ = rpa_v3(*args, softmax_scale=0.1, v_scale=2.0)
     assert np.array_equal(a, base) and np.array_equal(b, base)
     np.testing.assert_allclose(c, 2 * base, rtol=2 ** -7)
+
+
+# ---------------------------------------------------------------- 8-bit cache (float8_e4m3fn)
+
+def test_e4m3_rounding_agrees_with_the_cast_of_torch():
+    # the restatement's rounding to float8_e4m3fn against an independent implementation of the same cast
+    import torch
+
+    rng = np.random.default_rng(0)
+    x = np.concatenate([rng.standard_normal(50000).astype(np.float32) * s for s in (1e-3, 1e-2, 0.1, 1, 10, 100)]
+                       + [np.array([0, 448, -448, 2.0**-9, 2.0**-10, 3 * 2.0**-10, 2.0**-6, 1.5 * 2.0**-10, 0.0625 * 17 / 16,
+                                    0.0625 * 19 / 16], np.float32)])
+    x = np.clip(x, -448, 448)
+    ours = rpa_oracle.fp8_e4m3fn_round(x)
+    theirs = torch.from_numpy(x).to(torch.float8_e4m3fn).to(torch.float32).numpy()
+    assert np.array_equal(ours, theirs)
+    # ties go to the even mantissa; half of the smallest subnormal goes to zero
+    assert rpa_oracle.fp8_e4m3fn_round(np.float32(2.0**-10)) == 0.0
+    assert rpa_oracle.fp8_e4m3fn_round(np.float32(0.0625 * 17 / 16)) == np.float32(0.0625)      # 1.0001|1 -> 1.000
+    assert rpa_oracle.fp8_e4m3fn_round(np.float32(0.0625 * 19 / 16)) == np.float32(0.0625 * 1.25)  # 1.001|1 -> 1.010
+
+
+def make_e4m3(rng, q_lens, kv_lens, **kw):
+    q, k, v, cache, lens, bt, qsl, dist = make(rng, q_lens, kv_lens, dtype="float32", **kw)
+    f8 = rpa_oracle.fp8_e4m3fn_round
+    P, page, hx2, _, D = cache.shape
+    return bf(q), f8(k), f8(v), f8(cache).reshape(P, page, hx2 // 4, 4, D), lens, bt, qsl, dist
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_e4m3_efficient_restatement_agrees_with_the_literal_one(seed):
+    rng = np.random.default_rng(100 + seed)
+    S = int(rng.integers(1, 4))
+    kv_lens = [int(rng.integers(1, 14)) for _ in range(S)]
+    q_lens = [int(rng.integers(0, min(k, 5) + 1)) for k in kv_lens]
+    args = make_e4m3(rng, q_lens, kv_lens, page=4)
+    kw = dict(softmax_scale=0.09, cache_dtype="float8_e4m3fn", query_dtype="bfloat16")
+    if seed % 2:
+        kw.update(q_scale=0.03, k_scale=0.5, v_scale=2.0, sliding_window=6)
+    a, ca = rpa_v3_literal(*args, **kw)
+    b, cb = rpa_v3(*args, **kw)
+    assert np.array_equal(ca, cb)
+    np.testing.assert_allclose(a, b, atol=1e-6, rtol=0)
+
+
+def test_e4m3_probabilities_are_rounded_after_normalisation():
+    # q = 0: every visible key gets p = 1 / n.  n = 64: 2**-6 is representable, the output is the mean of V (exact in
+    # float32: sums of multiples of 2**-15).  n = 1024: 2**-10 is half of the smallest subnormal and rounds to zero,
+    # so the row is zero -- the cast of the *normalised* probabilities (_kernel.py:279) decides, not exp(s - max) = 1.
+    rng = np.random.default_rng(7)
+    for n, zero in ((64, False), (1024, True)):
+        q, k, v, cache, lens, bt, qsl, dist = make_e4m3(rng, [1], [n], page=4, Hq=2, Hkv=2)
+        q[:] = 0
+        out, cache_after = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, softmax_scale=1.0, cache_dtype="float8_e4m3fn",
+                                  query_dtype="bfloat16")
+        if zero:
+            assert not out.any()
+            continue
+        P, page, _, _, D = cache_after.shape
+        rows = cache_after.reshape(P, page, -1, D)
+        pps = bt.size // lens.shape[0]
+        vis = np.stack([rows[bt[pos // page], pos % page] for pos in range(n)])  # [n, 2 Hkv, D] of sequence 0
+        for h in range(2):
+            np.testing.assert_array_equal(out[0, h], bf(vis[:, 2 * h + 1].astype(np.float64).mean(axis=0)))
+
+
+def test_e4m3_query_is_clipped_and_cast_when_q_scale_is_given():
+    # Closed form.  One query element is 100, q_scale 0.01: Q / q_scale = 10000 is clipped to 448 (_kernel.py:251-253).
+    # Two keys, +1 and -1 in that element, zero elsewhere: the logits differ by 2 * 448 * softmax_scale * q_scale = ln 3,
+    # so p = (0.75, 0.25), both on the e4m3 grid, and the output is 0.75 v1 + 0.25 v2.  Without the clip the
+    # difference would be 24.5 and the output v1.
+    rng = np.random.default_rng(9)
+    q, k, v, cache, lens, bt, qsl, dist = make_e4m3(rng, [2], [2], page=4, Hq=2, Hkv=2)
+    q[:] = 0
+    q[1, :, 0] = 100.0   # the second token sees both keys (the first one only key 0)
+    k[:] = 0
+    k[0, :, 0] = 1.0
+    k[1, :, 0] = -1.0
+    scale = float(np.log(3.0) / (2 * 448 * 0.01))
+    out, _ = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, softmax_scale=scale, q_scale=0.01,
+                    cache_dtype="float8_e4m3fn", query_dtype="bfloat16")
+    for h in range(2):
+        np.testing.assert_array_equal(out[1, h], bf(0.75 * v[0, h] + 0.25 * v[1, h]))
+        np.testing.assert_array_equal(out[0, h], bf(v[0, h]))
