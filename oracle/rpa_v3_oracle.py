@@ -46,8 +46,13 @@ imported here (no jax).  Pins (``tests/test_v3_oracle_pins.py``): ``rpa_v3`` aga
 ``rpa_v3_literal`` on random tiny batches; the cache update against a closed form
 (every new row lands at its page and slot, nothing else changes); the attention
 against the float64 dense oracle of the v2 operation on the updated cache; ``q = 0``
-closed form.  **Parity unpinned:** the summation order of XLA's float32 matmul /
-softmax reductions (below 1e-5 relative).
+closed form.  For an 8-bit cache: the e4m3 rounding against the cast of torch on 3e5
+values including ties and subnormals; closed forms for the cast of the normalised
+probabilities (p = 2**-6 survives, p = 2**-10 becomes zero) and for the clip of
+``Q / q_scale`` to +-448; ``rpa_v3`` against ``rpa_v3_literal``.  **Parity unpinned:** the
+summation order of XLA's float32 matmul / softmax reductions (below 1e-5 relative), and
+with an 8-bit cache which side of a rounding boundary a probability falls on when that
+order moves it across.
 """
 
 from __future__ import annotations

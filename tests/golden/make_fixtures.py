@@ -68,6 +68,26 @@ def main():
                         block_tables=bt, query_start_loc=qsl, distribution=dist, softmax_scale=np.float32(D ** -0.5),
                         expected=rpa_oracle.bf16_bits(out), expected_cache=rpa_oracle.bf16_bits(new))
 
+    # the same operation with a float8_e4m3fn cache (values stored as float16, which holds every e4m3 value exactly)
+    rng = np.random.default_rng(13)
+    f8 = rpa_oracle.fp8_e4m3fn_round
+    q_lens, kv_lens, Hq, Hkv, D, page, pps = [3, 1, 24], [40, 64, 24], 4, 2, 128, 16, 4
+    S, P, T = 3, 3 * 4 + 1, 28 + 4
+    q = bf(rng.standard_normal((T, Hq, D)))
+    k, v = (f8(rng.standard_normal((T, Hkv, D))) for _ in range(2))
+    cache = f8(rng.standard_normal((P, page, 2 * Hkv // 4, 4, D)))
+    bt = rng.permutation(P)[: S * pps].astype(np.int32)
+    qsl = np.concatenate([[0], np.cumsum(q_lens)]).astype(np.int32)
+    lens = np.asarray(kv_lens, np.int32)
+    dist = np.array([0, 0, S], np.int32)
+    kw = dict(softmax_scale=D ** -0.5, q_scale=0.05, k_scale=0.5, v_scale=2.0)
+    out, new = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, cache_dtype="float8_e4m3fn", query_dtype="bfloat16", **kw)
+    assert all(np.array_equal(a.astype(np.float16).astype(np.float32), a) for a in (k, v, cache, new))
+    np.savez_compressed(os.path.join(HERE, "rpa_v3_e4m3.npz"), queries=rpa_oracle.bf16_bits(q), keys=k.astype(np.float16),
+                        values=v.astype(np.float16), kv_cache=cache.astype(np.float16), kv_lens=lens, block_tables=bt,
+                        query_start_loc=qsl, distribution=dist, expected=rpa_oracle.bf16_bits(out),
+                        expected_cache=new.astype(np.float16), **{n: np.float32(x) for n, x in kw.items()})
+
     rng = np.random.default_rng(4)
     ctx = np.array([1, 17, 100, 64], np.int32)
     nb, bs, mb = 4 * 7, 16, 7

@@ -43,6 +43,12 @@ def test_other_oracles_reproduce_their_fixtures():
     out, new = rpa_v3(*[bf16_from_bits(f[k]) for k in ("queries", "keys", "values", "kv_cache")], f["kv_lens"],
                       f["block_tables"], f["query_start_loc"], f["distribution"], softmax_scale=float(f["softmax_scale"]))
     assert np.array_equal(bf16_bits(out), f["expected"]) and np.array_equal(bf16_bits(new), f["expected_cache"])
+    f = load("rpa_v3_e4m3.npz")
+    scales = {n: float(f[n]) for n in ("softmax_scale", "q_scale", "k_scale", "v_scale")}
+    out, new = rpa_v3(bf16_from_bits(f["queries"]), *[f[k].astype(np.float32) for k in ("keys", "values", "kv_cache")],
+                      f["kv_lens"], f["block_tables"], f["query_start_loc"], f["distribution"],
+                      cache_dtype="float8_e4m3fn", query_dtype="bfloat16", **scales)
+    assert np.array_equal(bf16_bits(out), f["expected"]) and np.array_equal(new, f["expected_cache"].astype(np.float32))
     f = load("page_attention.npz")
     out = page_attention_strict(*[bf16_from_bits(f[k]) for k in ("query", "key_cache", "value_cache")],
                                 f["context_lens"], f["block_tables"], attn_scale=float(f["attn_scale"]))
@@ -72,9 +78,9 @@ def _idx(a):
     return torch.from_numpy(np.ascontiguousarray(a)).to("cuda:0")
 
 
-def _check(out, expected_bits, rows):
+def _check(out, expected_bits, rows, scale=1.0):
     got = out.float().cpu().numpy()[:rows]
-    d = np.abs(got - bf16_from_bits(expected_bits)[:rows])
+    d = np.abs(got - bf16_from_bits(expected_bits)[:rows]) / scale   # scale: what v_scale multiplied the outputs by
     assert d.max() <= 2e-2 and d.mean() <= 2e-3, (d.max(), d.mean())
 
 
@@ -99,6 +105,17 @@ def test_device_kernels_against_the_frozen_outputs(flags):
                                           _idx(f["distribution"]), softmax_scale=float(f["softmax_scale"]), _flags=flags)
     _check(out, f["expected"], int(f["query_start_loc"][-1]))
     assert np.array_equal(bf16_bits(cache.float().cpu().numpy()), f["expected_cache"])
+    if flags != 1:  # an 8-bit cache runs on the MFMA kernel only
+        f = load("rpa_v3_e4m3.npz")
+        import torch
+
+        f8 = lambda a: torch.from_numpy(a.astype(np.float32)).to(torch.float8_e4m3fn).to("cuda:0")  # noqa: E731
+        scales = {n: float(f[n]) for n in ("softmax_scale", "q_scale", "k_scale", "v_scale")}
+        out, cache = ragged_page_attention_v3(_dev(f["queries"]), f8(f["keys"]), f8(f["values"]), f8(f["kv_cache"]),
+                                              _idx(f["kv_lens"]), _idx(f["block_tables"]), _idx(f["query_start_loc"]),
+                                              _idx(f["distribution"]), _flags=flags, **scales)
+        _check(out, f["expected"], int(f["query_start_loc"][-1]), scale=2.0)
+        assert np.array_equal(cache.float().cpu().numpy(), f["expected_cache"].astype(np.float32))
     f = load("page_attention.npz")
     out = page_attention(_dev(f["query"]), _dev(f["key_cache"]), _dev(f["value_cache"]), _idx(f["context_lens"]),
                          _idx(f["block_tables"]), attn_scale=float(f["attn_scale"]), _flags=flags)
