@@ -14,6 +14,13 @@ head_dim that is a multiple of 128 and an even combined-head count, byte for byt
 shapes (padded head_dim, a padded odd head count) are rejected here.
 
 ``distribution[-1]`` is the number of sequences (``_kernel.py:195``).
+
+Cache dtypes: the dtype of the queries (bfloat16 or float32), or ``torch.float8_e4m3fn`` with
+bfloat16 queries (keys and values then come in float8_e4m3fn too, as the reference's
+``merge_kv`` demands; packing 4).  With an 8-bit cache the program's casts apply:
+``Q / q_scale`` is clipped to the e4m3 range and cast to e4m3 when ``q_scale`` is given
+(``_kernel.py:249-254``), and the normalised probabilities are cast to e4m3 (``:279``), so
+probabilities below 2**-10 count as zero.
 """
 
 from __future__ import annotations
