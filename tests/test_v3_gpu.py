@@ -290,3 +290,33 @@ def test_e4m3_full_size_decode_sample():
     assert torch.equal(out, out2)
     assert_bf16_parity(to_np(out[rows_idx.to(DEV)]), ref_out, sub.total_valid_tokens, "decode_llama3_8b e4m3")
     assert torch.isfinite(out.float()).all() and not out[b.total_valid_tokens:].any()
+
+
+def test_e4m3_call_recorded_in_a_hip_graph_replays_correctly():
+    """Cache update and both attention passes only enqueue kernels, so the call can be captured; every replay on new
+    queries and new rows must equal the eager result bit for bit."""
+    v = small_e4m3([9, 1, 0, 17, 2, 4], [40, 250, 8, 17, 133, 256], max_num_seqs=8)
+    kw = dict(v.kwargs(), q_scale=0.05, v_scale=2.0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            ragged_page_attention_v3(*v.args(), **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, _ = ragged_page_attention_v3(*v.args(), **kw)
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for rep in range(3):
+        v.queries.copy_(torch.randn(v.queries.shape, generator=gen, device=DEV).to(v.queries.dtype))
+        v.keys.copy_(torch.randn(v.keys.shape, generator=gen, device=DEV).to(F8))
+        v.values.copy_(torch.randn(v.values.shape, generator=gen, device=DEV).to(F8))
+        want, _ = ragged_page_attention_v3(*v.args(), **kw)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), rep
+    ref_out, ref_cache = oracle_e4m3(v, q_scale=0.05, v_scale=2.0)   # the cache already holds the last new rows
+    assert np.array_equal(to_np(v.kv_cache), ref_cache)
+    assert_bf16_parity(to_np(out_g) / 2.0, ref_out / 2.0, 33, "graph replay")
