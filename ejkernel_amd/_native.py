@@ -14,7 +14,7 @@ from pathlib import Path
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
 RPA_ABI_VERSION = 5
-RPA_DTYPE_BF16, RPA_DTYPE_F32, RPA_DTYPE_FP8_E4M3 = 0, 1, 2
+RPA_DTYPE_BF16, RPA_DTYPE_F32, RPA_DTYPE_FP8_E4M3, RPA_DTYPE_FP8_E5M2 = 0, 1, 2, 3
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
 RPA_FLAG_FP32_LOGITS = 2

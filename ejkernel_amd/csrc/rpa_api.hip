@@ -285,7 +285,7 @@ static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStrea
 uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims) {
   if (dims == nullptr) return 0;
   const uint64_t base = rpa_workspace_bytes(&dims->attn);
-  if (base == 0 || dims->cache_dtype != RPA_DTYPE_FP8_E4M3) return base;
+  if (base == 0 || (dims->cache_dtype != RPA_DTYPE_FP8_E4M3 && dims->cache_dtype != RPA_DTYPE_FP8_E5M2)) return base;
   const uint64_t rows = static_cast<uint64_t>(dims->attn.total_tokens > 0 ? dims->attn.total_tokens : 0) * dims->attn.num_q_heads;
   return ((base + 255) & ~255ull) + ((rows * 8 + 255) & ~255ull);
 }
@@ -298,9 +298,9 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (rc != RPA_OK) return rc;
   if (!v.new_keys || !v.new_values) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null new_keys / new_values");
   if (v.attn.num_sinks != 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "ragged_page_attention_v3 has no sinks");
-  const bool fp8 = v.cache_dtype == RPA_DTYPE_FP8_E4M3;
+  const bool fp8 = v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2;
   if (!fp8 && v.cache_dtype != v.attn.dtype)
-    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_dtype=%d: the cache has the dtype of the queries (%d) or is RPA_DTYPE_FP8_E4M3",
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_dtype=%d: the cache has the dtype of the queries (%d) or is RPA_DTYPE_FP8_E4M3 / RPA_DTYPE_FP8_E5M2",
                      v.cache_dtype, v.attn.dtype);
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   if (fp8) {
@@ -333,7 +333,7 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   float* stats = reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base);
   RpaParams q = p;
   q.workspace_bytes = base;
-  rc = rpa::launch_tiled_fp8(q, kv, stats, stream);
+  rc = rpa::launch_tiled_fp8(q, kv, v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 2 : 1, stats, stream);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
   return RPA_OK;
 }

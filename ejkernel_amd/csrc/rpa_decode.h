@@ -17,32 +17,55 @@ struct Cfg {
   static constexpr int LDS_PER_WAVE = TT * ROWB;
 };
 
-// Cache element types (kKv): 0 = the query dtype (bf16), 1 = 8-bit float, OCP e4m3 (finite, no infinities).
-// Eight e4m3 elements in two dwords -> the same eight values as bf16 in four dwords (exact).
+// Cache element types (kKv): 0 = the query dtype (bf16); 8-bit floats of the OCP formats: 1 = e4m3 (finite, no
+// infinities, largest value 448), 2 = e5m2 (largest finite value 57344).
+template <int kKv>
+__device__ __forceinline__ auto fp8_pair_lo(uint32_t w) {
+  if constexpr (kKv == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(static_cast<int>(w), false);
+  else return __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
+}
+template <int kKv>
+__device__ __forceinline__ auto fp8_pair_hi(uint32_t w) {
+  if constexpr (kKv == 2) return __builtin_amdgcn_cvt_pk_f32_bf8(static_cast<int>(w), true);
+  else return __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
+}
+// Bytes 2 half, 2 half + 1 of a dword as floats (the half must fold to a constant: the instruction encodes it).
+template <int kKv>
+__device__ __forceinline__ auto fp8_pair(uint32_t w, int half) {
+  const auto lo = fp8_pair_lo<kKv>(w);
+  const auto hi = fp8_pair_hi<kKv>(w);
+  return half ? hi : lo;
+}
+// Eight 8-bit elements in two dwords -> the same eight values as bf16 in four dwords (exact).
+template <int kKv>
 __device__ __forceinline__ u32x4_t fp8x8_to_bf16x8(u32x2_t w) {
   u32x4_t o;
 #pragma unroll
   for (int d = 0; d < 2; ++d) {
-    const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w[d]), false);  // bytes 0, 1
-    const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w[d]), true);   // bytes 2, 3
+    const auto lo = fp8_pair_lo<kKv>(w[d]);  // bytes 0, 1
+    const auto hi = fp8_pair_hi<kKv>(w[d]);  // bytes 2, 3
     o[2 * d] = __builtin_amdgcn_perm(__float_as_uint(lo[1]), __float_as_uint(lo[0]), 0x07060302u);
     o[2 * d + 1] = __builtin_amdgcn_perm(__float_as_uint(hi[1]), __float_as_uint(hi[0]), 0x07060302u);
   }
   return o;
 }
-// Bytes 2 half, 2 half + 1 of a dword as floats (the half must fold to a constant: the instruction encodes it).
-__device__ __forceinline__ auto fp8_pair(uint32_t w, int half) {
-  const auto lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), false);
-  const auto hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(w), true);
-  return half ? hi : lo;
-}
-// Two floats rounded to e4m3 (nearest even; the callers keep them inside +-448) and back.
+// Two floats rounded to the 8-bit type (nearest even; the callers keep them inside its finite range) and back.
+template <int kKv>
 __device__ __forceinline__ void round_fp8x2(float& a, float& b) {
-  const int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
-  const auto f = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
-  a = f[0];
-  b = f[1];
+  if constexpr (kKv == 2) {
+    const int w = __builtin_amdgcn_cvt_pk_bf8_f32(a, b, 0, false);
+    const auto f = __builtin_amdgcn_cvt_pk_f32_bf8(w, false);
+    a = f[0];
+    b = f[1];
+  } else {
+    const int w = __builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false);
+    const auto f = __builtin_amdgcn_cvt_pk_f32_fp8(w, false);
+    a = f[0];
+    b = f[1];
+  }
 }
+template <int kKv>
+constexpr float fp8_max() { return kKv == 2 ? 57344.f : 448.f; }
 
 // Everything one wavefront needs for one work item.  kWaveOnly: the state in TileArgs::pre, if any, is merged into
 // every row (only in the kernel instantiation without prefill tiles, so that the common one keeps its register
@@ -92,11 +115,13 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       for (int e = 0; e < 4; ++e) {
         float q0 = q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale);
         float q1 = q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale);
-        if (kKv == 1 && p.q_scale > 0.f) {
-          // q / q_scale in the query dtype, clipped to the cache dtype's range and cast to it (_kernel.py:249-254)
-          q0 = fminf(fmaxf(rbf(q0), -448.f), 448.f);
-          q1 = fminf(fmaxf(rbf(q1), -448.f), 448.f);
-          round_fp8x2(q0, q1);
+        if constexpr (kKv != 0) {
+          if (p.q_scale > 0.f) {
+            // q / q_scale in the query dtype, clipped to the cache dtype's range and cast to it (_kernel.py:249-254)
+            q0 = fminf(fmaxf(rbf(q0), -fp8_max<kKv>()), fp8_max<kKv>());
+            q1 = fminf(fmaxf(rbf(q1), -fp8_max<kKv>()), fp8_max<kKv>());
+            round_fp8x2<kKv>(q0, q1);
+          }
         }
         sc[e] = pack_bf16x2(q0, q1);
       }
@@ -129,8 +154,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const float cap = p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
 
-  using raw_t = typename std::conditional<kKv == 1, u32x2_t, u32x4_t>::type;  // one lane's piece: eight elements
-  constexpr uint32_t PIECE_B = kKv == 1 ? 8u : 16u, SLICE_B = 16u * PIECE_B;
+  using raw_t = typename std::conditional<kKv != 0, u32x2_t, u32x4_t>::type;  // one lane's piece: eight elements
+  constexpr uint32_t PIECE_B = kKv != 0 ? 8u : 16u, SLICE_B = 16u * PIECE_B;
   raw_t kreg[C::NSLOT][C::NS];
   raw_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
 
@@ -200,7 +225,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
           u32x4_t kw;
-          if constexpr (kKv == 1) kw = fp8x8_to_bf16x8(kreg[4 * u + r][sN]);
+          if constexpr (kKv != 0) kw = fp8x8_to_bf16x8<kKv>(kreg[4 * u + r][sN]);
           else kw = kreg[4 * u + r][sN];
           *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kw;
         }
@@ -251,8 +276,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         float pv[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) pv[r] = __builtin_amdgcn_exp2f((sv[u][r] - m_fix) * kLog2e) * inv_l;
-        round_fp8x2(pv[0], pv[1]);
-        round_fp8x2(pv[2], pv[3]);
+        round_fp8x2<kKv>(pv[0], pv[1]);
+        round_fp8x2<kKv>(pv[2], pv[3]);
         pw[2 * u] = (__float_as_uint(pv[0]) >> 16) | (__float_as_uint(pv[1]) & 0xffff0000u);
         pw[2 * u + 1] = (__float_as_uint(pv[2]) >> 16) | (__float_as_uint(pv[3]) & 0xffff0000u);
       }
@@ -302,10 +327,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         uint32_t aw[2 * NT];
 #pragma unroll
         for (int h = 0; h < 2 * NT; ++h) {
-          if constexpr (kKv == 1) {
+          if constexpr (kKv != 0) {
             // elements c of the two tokens' pieces: byte c of each piece, widened (bf16 = upper half of the float)
-            const auto f1 = fp8_pair(vcur[2 * h + 1][sN][c >> 2], (c >> 1) & 1);
-            const auto f0 = fp8_pair(vcur[2 * h][sN][c >> 2], (c >> 1) & 1);
+            const auto f1 = fp8_pair<kKv>(vcur[2 * h + 1][sN][c >> 2], (c >> 1) & 1);
+            const auto f0 = fp8_pair<kKv>(vcur[2 * h][sN][c >> 2], (c >> 1) & 1);
             aw[h] = __builtin_amdgcn_perm(__float_as_uint(f1[c & 1]), __float_as_uint(f0[c & 1]), 0x07060302u);
           } else {
             aw[h] = __builtin_amdgcn_perm(vcur[2 * h + 1][sN][c >> 1], vcur[2 * h][sN][c >> 1], sel);

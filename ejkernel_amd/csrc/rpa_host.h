@@ -81,9 +81,9 @@ struct WorkspaceLayout {
 bool tiled_supported(const RpaParams& p);
 void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl);
 int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre = PreState());
-// The same for an 8-bit (e4m3) cache described by `kv`: two launches, row statistics into `stats`
-// [total_tokens, num_q_heads, 2] and then the attention (RPA_FLAG_FP32_LOGITS arithmetic, no sinks).
-int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, float* stats, hipStream_t stream);
+// The same for an 8-bit cache described by `kv` (kv_elem 1 = e4m3, 2 = e5m2): two launches, row statistics into
+// `stats` [total_tokens, num_q_heads, 2] and then the attention (RPA_FLAG_FP32_LOGITS arithmetic, no sinks).
+int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, hipStream_t stream);
 
 // Compute units of the current device (cached per device).
 int device_cu_count();

@@ -36,7 +36,7 @@ __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const
 int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream) {
   const RpaParams& p = v.attn;
   if (p.total_tokens == 0) return RPA_OK;
-  const int row_bytes = p.head_dim * (v.cache_dtype == RPA_DTYPE_FP8_E4M3 ? 1 : v.cache_dtype == RPA_DTYPE_BF16 ? 2 : 4);
+  const int row_bytes = p.head_dim * (v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 1 : v.cache_dtype == RPA_DTYPE_BF16 ? 2 : 4);
   if (row_bytes % 16 != 0) return RPA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_cache_update_kernel, dim3(p.total_tokens), dim3(256), 0, stream, p,
                      static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes);

@@ -434,7 +434,8 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
-static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre, float* stats) {
+static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre, float* stats,
+                             int kv_elem = 0) {
   WorkspaceLayout wl;
   tiled_workspace_layout(p, &wl);
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
@@ -460,8 +461,16 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // every sequence through the wave-level loop.  A wavefront has half the bytes in flight that it has with a
     // 16-bit cache, so both workgroups of a compute unit stream (0.70 ms against 0.84 ms on 256 x 512..8192 keys).
     a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 2));
-    int rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
-                               : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
+    int rc;
+    if (kv_elem == 2) {
+      rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)
+                             : launch_cfg<256, 1, 1, false, true, 2, 1>(a, grid, stream);
+      if (rc != RPA_OK) return rc;
+      return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 2>(a, grid, stream)
+                               : launch_cfg<256, 1, 1, false, true, 2, 2>(a, grid, stream);
+    }
+    rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
+                           : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
     if (rc != RPA_OK) return rc;
     return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
                              : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
@@ -488,8 +497,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
 int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
   return launch_tiled_impl(p, kv, stream, pre, nullptr);
 }
-int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, float* stats, hipStream_t stream) {
-  return launch_tiled_impl(p, kv, stream, PreState(), stats);
+int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, hipStream_t stream) {
+  return launch_tiled_impl(p, kv, stream, PreState(), stats, kv_elem);
 }
 
 }  // namespace rpa

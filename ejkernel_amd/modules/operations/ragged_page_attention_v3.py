@@ -15,12 +15,12 @@ shapes (padded head_dim, a padded odd head count) are rejected here.
 
 ``distribution[-1]`` is the number of sequences (``_kernel.py:195``).
 
-Cache dtypes: the dtype of the queries (bfloat16 or float32), or ``torch.float8_e4m3fn`` with
-bfloat16 queries (keys and values then come in float8_e4m3fn too, as the reference's
-``merge_kv`` demands; packing 4).  With an 8-bit cache the program's casts apply:
-``Q / q_scale`` is clipped to the e4m3 range and cast to e4m3 when ``q_scale`` is given
-(``_kernel.py:249-254``), and the normalised probabilities are cast to e4m3 (``:279``), so
-probabilities below 2**-10 count as zero.
+Cache dtypes: the dtype of the queries (bfloat16 or float32), or ``torch.float8_e4m3fn`` /
+``torch.float8_e5m2`` with bfloat16 queries (keys and values then come in the same 8-bit
+type, as the reference's ``merge_kv`` demands; packing 4).  With an 8-bit cache the program's
+casts apply: ``Q / q_scale`` is clipped to the type's finite range and cast to it when
+``q_scale`` is given (``_kernel.py:249-254``), and the normalised probabilities are cast to it
+(``:279``), so in e4m3 probabilities below 2**-10 count as zero (2**-17 in e5m2).
 """
 
 from __future__ import annotations
@@ -35,6 +35,9 @@ from .configs import _PLATFORMS, RaggedPageAttentionv3Config
 from .ragged_page_attention import _workspace
 
 __all__ = ["RaggedPageAttentionv3", "ragged_page_attention_v3"]
+
+# 8-bit cache dtypes (the OCP formats; the fnuz variants are other encodings and are not accepted)
+_FP8 = {torch.float8_e4m3fn: _native.RPA_DTYPE_FP8_E4M3, torch.float8_e5m2: _native.RPA_DTYPE_FP8_E5M2}
 
 
 def _packing(dtype: torch.dtype) -> int:
@@ -86,14 +89,13 @@ def _static_validate(q, k, v, kv_cache, kv_lens, block_tables, query_start_loc, 
         raise ValueError("a cache with padded combined heads is not supported")
     if not (k.dtype == v.dtype == kv_cache.dtype):
         raise ValueError("keys, values and kv_cache must share one dtype")  # merge_kv asserts it, the update needs it
-    fp8 = kv_cache.dtype == torch.float8_e4m3fn
-    if fp8:
+    if kv_cache.dtype in _FP8:
         if q.dtype != torch.bfloat16:
-            raise ValueError("a float8_e4m3fn cache takes bfloat16 queries")
+            raise ValueError("an 8-bit cache takes bfloat16 queries")
     elif q.dtype != kv_cache.dtype or q.dtype not in (torch.bfloat16, torch.float32):
         raise ValueError("queries, keys, values and kv_cache must share one dtype (bfloat16 or float32), or the cache "
-                         "(with keys and values) is float8_e4m3fn and the queries bfloat16; other 8-bit types are not "
-                         "built")
+                         "(with keys and values) is float8_e4m3fn or float8_e5m2 and the queries bfloat16; other "
+                         "cache types are not built")
 
 
 def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, *, softmax_scale,
@@ -156,7 +158,7 @@ def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_
     p.v_scale = 0.0 if v_scale is None else float(v_scale)
     v3.new_keys = keys.data_ptr()
     v3.new_values = values.data_ptr()
-    v3.cache_dtype = _native.RPA_DTYPE_FP8_E4M3 if kv_cache.dtype == torch.float8_e4m3fn else p.dtype
+    v3.cache_dtype = _FP8.get(kv_cache.dtype, p.dtype)
     v3.reserved = 0
 
     with torch.cuda.device(dev):

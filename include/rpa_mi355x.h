@@ -31,6 +31,7 @@ extern "C" {
 #define RPA_DTYPE_BF16 0
 #define RPA_DTYPE_F32 1
 #define RPA_DTYPE_FP8_E4M3 2 /* OCP e4m3 (finite, no infinities; jnp.float8_e4m3fn): cache of rpa_v3_launch only */
+#define RPA_DTYPE_FP8_E5M2 3 /* OCP e5m2 (jnp.float8_e5m2): cache of rpa_v3_launch only */
 
 /* arithmetic mode */
 #define RPA_COMPUTE_BF16 0 /* bf16 MFMA contractions, fp32 online softmax, reference rounding points */
@@ -116,10 +117,11 @@ typedef struct RpaV3Params {
                           /* tokens); num_seqs = &distribution[2]; RPA_FLAG_FP32_LOGITS is implied                 */
   const void* new_keys;   /* [total_tokens, num_kv_heads, head_dim], dtype of the cache                            */
   const void* new_values; /* [total_tokens, num_kv_heads, head_dim]                                                */
-  int32_t cache_dtype;    /* dtype of the cache and of the new rows: attn.dtype, or RPA_DTYPE_FP8_E4M3 with bf16    */
-                          /* queries.  An 8-bit cache follows the program's casts (_kernel.py:249-254, :279): with  */
-                          /* q_scale, q / q_scale is rounded to the query dtype, clipped to +-448 and cast to e4m3; */
-                          /* the normalised probabilities are cast to e4m3 before P V.  It runs as two passes over  */
+  int32_t cache_dtype;    /* dtype of the cache and of the new rows: attn.dtype, or RPA_DTYPE_FP8_E4M3 / _E5M2 with */
+                          /* bf16 queries.  An 8-bit cache follows the program's casts (_kernel.py:249-254, :279):  */
+                          /* with q_scale, q / q_scale is rounded to the query dtype, clipped to the 8-bit type's   */
+                          /* finite range (+-448 / +-57344) and cast to it; the normalised probabilities are cast   */
+                          /* to it before P V.  It runs as two passes over                                          */
                           /* the keys (row maximum and sum, then the attention) on the MFMA kernel only, and needs  */
                           /* rpa_v3_workspace_bytes() of workspace.                                                 */
   int32_t reserved;       /* 0 */

@@ -84,6 +84,18 @@ def fp8_e4m3fn_round(a):
     return np.where(np.isfinite(x), y, np.float32(np.nan)).astype(np.float32)
 
 
+def fp8_e5m2_round(a):
+    """The same for ``float8_e5m2``: 5 exponent bits (bias 15), 2 mantissa bits, normal numbers from 2**-14 to
+    57344, subnormal multiples of 2**-16, infinities (a value that rounds past 57344 becomes infinite)."""
+    x = np.asarray(a, dtype=np.float32)
+    _, e = np.frexp(x)
+    quantum = np.ldexp(np.float32(1.0), np.maximum(e - 1, -14) - 2).astype(np.float32)
+    with np.errstate(invalid="ignore", over="ignore"):
+        y = (np.rint(x / quantum) * quantum).astype(np.float32)
+    y = np.where(np.abs(y) > np.float32(57344.0), np.copysign(np.float32(np.inf), x), y)
+    return np.where(np.isnan(x), np.float32(np.nan), y).astype(np.float32)
+
+
 def _rounder(dtype):
     name = np.dtype(dtype).name if not isinstance(dtype, str) else dtype
     if name in ("bfloat16", "bf16"):
@@ -92,6 +104,8 @@ def _rounder(dtype):
         return lambda a: np.asarray(a, dtype=np.float32)
     if name in ("float8_e4m3fn", "fp8_e4m3"):
         return fp8_e4m3fn_round
+    if name in ("float8_e5m2", "fp8_e5m2"):
+        return fp8_e5m2_round
     raise ValueError(f"unsupported dtype {dtype!r}")
 
 

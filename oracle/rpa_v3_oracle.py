@@ -29,7 +29,7 @@ Two functions:
     benchmark sizes.
 
 Arrays are float32 holding values representable in their dtype: ``cache_dtype`` for the cache and
-the new keys / values ("bfloat16", "float32" or "float8_e4m3fn"), ``query_dtype`` for the queries
+the new keys / values ("bfloat16", "float32", "float8_e4m3fn" or "float8_e5m2"), ``query_dtype`` for the queries
 (the cache dtype unless given; "bfloat16" with an 8-bit cache).  The output takes the query dtype
 (``:190``), ``Q / q_scale`` is computed in it, clipped to the cache dtype's finite range and cast
 to the cache dtype (``:249-254``), and the normalised probabilities are cast to the cache dtype
@@ -66,7 +66,7 @@ DEFAULT_MASK_VALUE = np.float32(-0.7 * float(np.finfo(np.float32).max))  # _kern
 
 def packing(cache_dtype):
     """32 // bit width (_kernel.py:38-39)."""
-    return {"bfloat16": 2, "float8_e4m3fn": 4}.get(cache_dtype, 1)
+    return {"bfloat16": 2, "float8_e4m3fn": 4, "float8_e5m2": 4}.get(cache_dtype, 1)
 
 
 def merge_kv(k, v, cache_dtype="bfloat16"):
@@ -90,7 +90,8 @@ def _unpack(flat, num_kv_heads, dalign):
 
 def _clip_to(x, cache_dtype):
     """jnp.clip(x, finfo.min, finfo.max) of the cache dtype (_kernel.py:251-253): only an 8-bit range cuts anything."""
-    return np.clip(x, np.float32(-448.0), np.float32(448.0)) if cache_dtype == "float8_e4m3fn" else x
+    top = {"float8_e4m3fn": 448.0, "float8_e5m2": 57344.0}.get(cache_dtype)
+    return x if top is None else np.clip(x, np.float32(-top), np.float32(top))
 
 
 def _softmax_f32(s):

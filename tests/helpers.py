@@ -13,7 +13,7 @@ F32_MAX_ABS = 1e-5    # tolerance of the fp32 path against the float64 evaluatio
 
 def to_np(t: torch.Tensor) -> np.ndarray:
     t = t.detach().cpu()
-    if t.dtype in (torch.bfloat16, torch.float8_e4m3fn):
+    if t.dtype in (torch.bfloat16, torch.float8_e4m3fn, torch.float8_e5m2):
         return t.to(torch.float32).numpy()
     return t.numpy()
 

@@ -198,30 +198,33 @@ def test_bf16_random_batches(seed):
 # where a probability sits on a rounding boundary.  The bound stays the bf16 one.
 
 F8 = torch.float8_e4m3fn
+F8_NAME = {torch.float8_e4m3fn: "float8_e4m3fn", torch.float8_e5m2: "float8_e5m2"}
+BOTH_F8 = [pytest.param(torch.float8_e4m3fn, id="e4m3"), pytest.param(torch.float8_e5m2, id="e5m2")]
 
 
-def small_e4m3(q_lens, kv_lens, **kw):
+def small_e4m3(q_lens, kv_lens, f8=F8, **kw):
     args = dict(num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=16, seed=3, device=DEV)
     args.update(kw)
-    return to_v3(make_batch(q_lens, kv_lens, **args), seed=args["seed"], cache_dtype=F8)
+    return to_v3(make_batch(q_lens, kv_lens, **args), seed=args["seed"], cache_dtype=f8)
 
 
 def oracle_e4m3(v, **kw):
     k = dict(v.kwargs())
     k.update(kw)
-    return rpa_v3(*[to_np(a) for a in v.args()], cache_dtype="float8_e4m3fn", query_dtype="bfloat16", **k)
+    return rpa_v3(*[to_np(a) for a in v.args()], cache_dtype=F8_NAME[v.kv_cache.dtype], query_dtype="bfloat16", **k)
 
 
 E4M3_CASES = dict(CASES)
 E4M3_CASES["long_decode"] = ([1, 1, 1, 1], [4000, 2500, 4096, 777], dict(pages_per_seq=256))
 
 
+@pytest.mark.parametrize("f8", BOTH_F8)
 @pytest.mark.parametrize("scales", [{}, dict(q_scale=0.05, k_scale=0.5, v_scale=2.0)], ids=["plain", "scales"])
 @pytest.mark.parametrize("case", list(E4M3_CASES))
-def test_e4m3_cache_parity_and_cache_update(case, scales):
+def test_e4m3_cache_parity_and_cache_update(case, scales, f8):
     q_lens, kv_lens, kw = E4M3_CASES[case]
-    v = small_e4m3(q_lens, kv_lens, **kw)
-    assert v.kv_cache.dtype == F8 and v.keys.dtype == F8 and v.kv_cache.shape[3] == 4
+    v = small_e4m3(q_lens, kv_lens, f8=f8, **kw)
+    assert v.kv_cache.dtype == f8 and v.keys.dtype == f8 and v.kv_cache.shape[3] == 4
     ref_out, ref_cache = oracle_e4m3(v, **scales)
     out, cache = run_hip(v, **scales)
     assert out.dtype == torch.bfloat16
@@ -238,7 +241,7 @@ def test_e4m3_probabilities_below_half_the_smallest_subnormal_vanish():
     # q = 0 over 1024 keys: p = 2**-10 rounds to zero in e4m3, the row is zero; over 64 keys p = 2**-6 survives and
     # the row is the mean of V.  An implementation that rounds exp(s - max) instead of the normalised value fails this.
     for n, zero in ((64, False), (1024, True)):
-        v = small_e4m3([1], [n], pages_per_seq=64)
+        v = small_e4m3([1], [n], pages_per_seq=64)           # e5m2 keeps 2**-10: covered by the parity cases
         v.queries.zero_()
         ref_out, _ = oracle_e4m3(v)
         out, _ = run_hip(v)
@@ -255,9 +258,9 @@ def test_e4m3_rejections():
         ragged_page_attention_v3(a[0], a[1].to(torch.bfloat16), *a[2:])
     with pytest.raises(ValueError, match="bfloat16 queries"):
         ragged_page_attention_v3(a[0].float(), *a[1:])
-    e5 = [a[0]] + [t.to(torch.float32).to(torch.float8_e5m2) for t in a[1:4]] + a[4:]
+    fnuz = [a[0]] + [t.to(torch.float32).to(torch.float8_e4m3fnuz) for t in a[1:4]] + a[4:]
     with pytest.raises(ValueError, match="not built"):
-        ragged_page_attention_v3(*e5)
+        ragged_page_attention_v3(*fnuz)
 
 
 @pytest.mark.parametrize("seed", range(200, 212))
@@ -266,7 +269,7 @@ def test_e4m3_random_batches(seed):
     if b.meta["num_kv_heads"] % 2:
         pytest.skip("an odd number of kv heads pads the packed cache: rejected")
     rows = b.total_valid_tokens
-    v = to_v3(b, seed=seed, cache_dtype=F8)
+    v = to_v3(b, seed=seed, cache_dtype=F8 if seed % 2 == 0 else torch.float8_e5m2)
     ref_out, ref_cache = oracle_e4m3(v)
     out, cache = run_hip(v)
     assert np.array_equal(to_np(cache), ref_cache), what

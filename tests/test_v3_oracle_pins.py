@@ -145,6 +145,36 @@ def test_e4m3_rounding_agrees_with_the_cast_of_torch():
     assert rpa_oracle.fp8_e4m3fn_round(np.float32(0.0625 * 19 / 16)) == np.float32(0.0625 * 1.25)  # 1.001|1 -> 1.010
 
 
+def test_e5m2_rounding_agrees_with_the_cast_of_torch():
+    import torch
+
+    rng = np.random.default_rng(1)
+    x = np.concatenate([rng.standard_normal(50000).astype(np.float32) * s for s in (1e-5, 1e-3, 0.1, 1, 100, 30000)]
+                       + [np.array([0, 57344, -57344, 2.0**-16, 2.0**-17, 3 * 2.0**-17, 2.0**-14, 61439, 61440, 1e6, 1.125, 1.375],
+                                   np.float32)])
+    ours = rpa_oracle.fp8_e5m2_round(x)
+    theirs = torch.from_numpy(x).to(torch.float8_e5m2).to(torch.float32).numpy()
+    assert np.array_equal(ours, theirs)
+    assert rpa_oracle.fp8_e5m2_round(np.float32(1.125)) == 1.0 and rpa_oracle.fp8_e5m2_round(np.float32(1.375)) == 1.5
+    assert np.isinf(rpa_oracle.fp8_e5m2_round(np.float32(61440.0))) and rpa_oracle.fp8_e5m2_round(np.float32(61439.0)) == 57344.0
+
+
+def test_e5m2_probabilities_are_rounded_after_normalisation():
+    # as for e4m3, with this type's grid: p = 1/3 becomes 0.3125 (1.01b x 2**-2), so q = 0 over three keys returns
+    # 0.3125 (v1 + v2 + v3), not their mean
+    rng = np.random.default_rng(8)
+    q, k, v, cache, lens, bt, qsl, dist = make(rng, [1], [3], dtype="float32", page=4, Hq=2, Hkv=2)
+    f8 = rpa_oracle.fp8_e5m2_round
+    P, page, hx2, _, D = cache.shape
+    q, k, v, cache = bf(q) * 0, f8(k), f8(v), f8(cache).reshape(P, page, hx2 // 4, 4, D)
+    out, after = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, softmax_scale=1.0, cache_dtype="float8_e5m2",
+                        query_dtype="bfloat16")
+    rows = after.reshape(P, page, -1, D)
+    vis = np.stack([rows[bt[pos // page], pos % page] for pos in range(3)])
+    for h in range(2):
+        np.testing.assert_array_equal(out[0, h], bf(np.float32(0.3125) * vis[:, 2 * h + 1].sum(axis=0, dtype=np.float32)))
+
+
 def make_e4m3(rng, q_lens, kv_lens, **kw):
     q, k, v, cache, lens, bt, qsl, dist = make(rng, q_lens, kv_lens, dtype="float32", **kw)
     f8 = rpa_oracle.fp8_e4m3fn_round
