@@ -277,21 +277,23 @@ def test_e4m3_random_batches(seed):
         assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], what)
 
 
-def test_e4m3_full_size_decode_sample():
-    b = make_workload("decode_llama3_8b", device=DEV)
-    v = to_v3(b, seed=5, cache_dtype=F8)
+@pytest.mark.parametrize("name,n_sample,f8", [("decode_llama3_8b", 10, torch.float8_e4m3fn),
+                                              ("mixed_prefill_decode", 12, torch.float8_e5m2)])
+def test_8bit_cache_full_size_sample(name, n_sample, f8):
+    b = make_workload(name, device=DEV)
+    v = to_v3(b, seed=5, cache_dtype=f8)
     rng = np.random.default_rng(1)
-    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:10])
+    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:n_sample])
     sub = compact_for_host(b, ids)
     rows_idx = sub.meta["rows"]
-    sub_v = to_v3(sub, seed=0, cache_dtype=F8)
+    sub_v = to_v3(sub, seed=0, cache_dtype=f8)
     sub_v.keys[: len(rows_idx)] = v.keys[rows_idx.to(DEV)].cpu()
     sub_v.values[: len(rows_idx)] = v.values[rows_idx.to(DEV)].cpu()
     ref_out, _ = oracle_e4m3(sub_v)
     out, cache = run_hip(v)
     out2, _ = run_hip(v)                          # the second call rewrites the same rows: same result, bit for bit
     assert torch.equal(out, out2)
-    assert_bf16_parity(to_np(out[rows_idx.to(DEV)]), ref_out, sub.total_valid_tokens, "decode_llama3_8b e4m3")
+    assert_bf16_parity(to_np(out[rows_idx.to(DEV)]), ref_out, sub.total_valid_tokens, f"{name} {f8}")
     assert torch.isfinite(out.float()).all() and not out[b.total_valid_tokens:].any()
 
 
