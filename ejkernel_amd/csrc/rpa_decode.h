@@ -394,12 +394,97 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     ticket = __shfl(ticket, 0, kWave);
     if (ticket != static_cast<uint32_t>(part.last_w - part.first_w)) return;
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    float M = -INFINITY, L = 0.f;
+    if constexpr (kWaveOnly) {
+      // A decode row tile has few rows (one per query head of the group), and a (sequence, kv head) of a small batch is
+      // cut into many parts -- 128 for one sequence on 1024 wavefronts -- which this wavefront would read one after
+      // the other at one memory latency each.  The lanes of the rows that do not exist take parts instead: with R
+      // rows padded to rp = 2^k, lane row i reads row i % rp of part k0 + i / rp, 16 / rp parts at a time (times the
+      // chunk), and the lanes of one row add up their sums at the end.
+      const int R = row_hi - row_lo;
+      const int rp = R <= 1 ? 1 : R <= 2 ? 2 : R <= 4 ? 4 : R <= 8 ? 8 : 16;
+      const int pp = 16 / rp;
+      const int rrow = i & (rp - 1), sub = i / rp;
+      const bool rv = rrow < R;
+      constexpr int kChunk = C::NS == 1 ? 2 : 1;
+      const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + rrow;
+      if (rv)
+        for (int k0 = part.first_w; k0 <= part.last_w; k0 += 4 * pp) {
+          uint64_t v[4];
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int k = min(k0 + c * pp + sub, part.last_w);
+            v[c] = __hip_atomic_load(ml + static_cast<size_t>(part_slot(k, part.stream_a, part.sh)) * 16, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int c = 0; c < 4; ++c) M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v[c])));
+        }
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1)
+        if (d >= rp) M = fmaxf(M, __shfl_xor(M, d, kWave));
+      const float M_use = M == -INFINITY ? 0.f : M;
+#pragma unroll
+      for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+        for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      if (rv) {
+        for (int k0 = part.first_w; k0 <= part.last_w; k0 += kChunk * pp) {
+          uint64_t mlv[kChunk];
+          uint64_t ov[kChunk][C::NS][4][4];
+#pragma unroll
+          for (int c = 0; c < kChunk; ++c) {
+            const size_t sl = part_slot(min(k0 + c * pp + sub, part.last_w), part.stream_a, part.sh);
+            mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + rrow) * D);
+            if constexpr (kPass != 1)
+#pragma unroll
+            for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                  ov[c][sN][r][e] = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
+                                                      __HIP_MEMORY_SCOPE_AGENT);
+          }
+#pragma unroll
+          for (int c = 0; c < kChunk; ++c) {
+            if (k0 + c * pp + sub > part.last_w) continue;  // past the last part: the load repeated it, it is not added again
+            const float mk = __uint_as_float(static_cast<uint32_t>(mlv[c]));
+            const float lk = __uint_as_float(static_cast<uint32_t>(mlv[c] >> 32));
+            const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
+            L += w * lk;
+            if constexpr (kPass != 1)
+#pragma unroll
+            for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+              for (int r = 0; r < 4; ++r)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                  o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e]));
+                  o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e] >> 32));
+                }
+          }
+        }
+      }
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1)
+        if (d >= rp) {
+          L += __shfl_xor(L, d, kWave);
+          if constexpr (kPass != 1)
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int c = 0; c < 8; ++c)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) o_acc[sN][c][r] += __shfl_xor(o_acc[sN][c][r], d, kWave);
+        }
+    } else {
     // The parts are read kMergeChunk at a time (more would take registers from the prefill tile, which shares this
     // kernel): all loads of a chunk are issued before the first is used, so the
     // merge costs one memory latency per chunk instead of two per part.
     constexpr int kMergeChunk = C::NS == 1 ? 2 : 1;
     const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + i;
-    float M = -INFINITY;
     if (row_valid)
       for (int k0 = part.first_w; k0 <= part.last_w; k0 += 2 * kMergeChunk) {
         uint64_t v[2 * kMergeChunk];
@@ -413,7 +498,6 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         for (int c = 0; c < 2 * kMergeChunk; ++c) M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v[c])));
       }
     const float M_use = M == -INFINITY ? 0.f : M;
-    float L = 0.f;
 #pragma unroll
     for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -456,6 +540,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
               }
         }
       }
+    }
     }
     m_run = M;
     l_run = L;

@@ -33,6 +33,7 @@
 namespace rpa {
 
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
+constexpr int kMaxMinShareTiles = 16;  // ... and the most the length of the (sequence, kv head)s raises that to
 constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
 constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
@@ -340,7 +341,13 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           // instead, kMinShareTiles tiles each: a (sequence, kv head) cut into many one-tile parts would spend its
           // time in the merge, which reads the parts one after the other.
           const int q = total_tiles / n_workers, half = n_workers / 2;
-          const int min_share = a.min_share_tiles;
+          // With T tiles per (sequence, kv head) cut into P parts a wavefront streams T / P tiles and the merge reads P
+          // parts, a few at a time: the sum is smallest near P = 3 sqrt(T), i.e. sqrt(T) / 3 tiles per part.
+          int min_share = a.min_share_tiles;
+          if constexpr (kWaveOnly) {
+            const float avg = static_cast<float>(total_tiles) / static_cast<float>(max(1, nseq * p.num_kv_heads));
+            min_share = max(min_share, min(kMaxMinShareTiles, static_cast<int>(__builtin_sqrtf(avg) * (1.f / 3.f))));
+          }
           if (q >= min_share) {
             const int rem = total_tiles - q * n_workers;
             int first_tiles = half * q + min(half, rem);
