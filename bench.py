@@ -25,8 +25,8 @@ if ROOT not in sys.path:
 # HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes (scaled by a plain 1 GiB device copy); a
 # workload without a counter run reports null.
 MEASURED_TRAFFIC_BYTES = {
-    "decode_llama3_8b": (2184731 * 2.0 + 18447 * 1.0) * 1024,
-    "mixed_prefill_decode": (2149118 * 2.0 + 85692 * 1.0) * 1024,
+    "decode_llama3_8b": (2184963 * 2.0 + 18447 * 1.0) * 1024,
+    "mixed_prefill_decode": (2148880 * 2.0 + 85691 * 1.0) * 1024,
 }
 
 
