@@ -126,14 +126,15 @@ def test_bf16_gqa_ratios(flags, hq, hkv):
     assert_bf16_parity(to_np(run_hip(b, flags)), run_strict(b), b.total_valid_tokens, f"gqa {hq}/{hkv}")
 
 
+@pytest.mark.parametrize("D", [128, 256, 64])
 @pytest.mark.parametrize("hq,hkv,q_len", [(2, 2, 1), (8, 4, 1), (8, 2, 1), (16, 2, 1), (16, 2, 2), (12, 4, 1), (8, 2, 3)])
-def test_bf16_few_long_sequences_split_into_many_parts(hq, hkv, q_len):
+def test_bf16_few_long_sequences_split_into_many_parts(hq, hkv, q_len, D):
     """One or two long sequences on the whole grid: every (sequence, kv head) is cut into dozens of parts, which the
     last wavefront to arrive merges several at a time on the lanes of the rows a decode tile does not have (1, 2, 4,
     8 or 16 rows per tile here, 3 and 6 padded to 4 and 8).  Parity, and the same bits on every call."""
-    b = small([q_len, q_len], [8192, 5000], num_q_heads=hq, num_kv_heads=hkv, pages_per_seq=512)
+    b = small([q_len, q_len], [8192, 5000], num_q_heads=hq, num_kv_heads=hkv, pages_per_seq=512, head_dim=D)
     out = run_hip(b)
-    assert_bf16_parity(to_np(out), run_strict(b), b.total_valid_tokens, f"{hq}/{hkv} q_len {q_len}")
+    assert_bf16_parity(to_np(out), run_strict(b), b.total_valid_tokens, f"{hq}/{hkv} q_len {q_len} D {D}")
     for _ in range(3):
         assert torch.equal(run_hip(b), out)
     assert_bf16_parity(to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES)), run_strict(b), b.total_valid_tokens, "tiles")
