@@ -324,6 +324,8 @@ WORKLOADS = {
     # the two halves of mixed_prefill_decode on their own (same lengths), to price each against its own roofline
     "mixed_prefill_only": "the 16 prefill chunks of mixed_prefill_decode: 512 tokens each, prior 0..4096",
     "mixed_decode_only": "the 240 decode sequences of mixed_prefill_decode: 1 token each, kv 256..8192",
+    # long prompts: every prefill tile walks thousands of keys (the per-tile costs of the 512-token chunks vanish)
+    "prefill_long": "2 prompts x 8192 tokens from scratch, 32q/8kv heads, D=128, page 32",
 }
 
 
@@ -369,6 +371,10 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         pps = pages(max(n(8192), n(4096) + chunk), 32)
         return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
                           pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=only or name)
+    if name == "prefill_long":
+        L = n(8192)
+        return make_batch(np.full(2, L), np.full(2, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
+                          pages_per_seq=pages(L, 32), seed=seed, device=device, dtype=dtype, name=name)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)
