@@ -183,10 +183,15 @@ def rpa_v3_literal(queries, keys, values, kv_cache, kv_lens, block_tables, query
 
 def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, *,
            softmax_scale=1.0, sliding_window=None, logits_soft_cap=None, q_scale=None, k_scale=None, v_scale=None,
-           cache_dtype="bfloat16", query_dtype=None, seqs=None):
+           cache_dtype="bfloat16", query_dtype=None, seqs=None, slack=None):
     """Same results as ``rpa_v3_literal`` from the visible keys only; returns (out, updated cache).
 
     ``seqs`` restricts the attention (not the cache update) to some sequences; the other rows stay zero.
+    ``slack`` (a float array [T, Hq], filled in place) receives, per output row, how far an evaluation of the same
+    program with another float32 exponential or summation order may land from this one because of the cast of the
+    probabilities to an 8-bit cache type: the sum, over the probabilities that lie within 1e-5 (relative) of a
+    rounding boundary of that type, of the rounding step there times the largest |V| of that key.  It is zero for
+    almost every row; a checker adds it to its bound.
     """
     R = _rounder(cache_dtype)
     Rq = _rounder(query_dtype or cache_dtype)
@@ -235,9 +240,15 @@ def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_l
         if logits_soft_cap is not None:
             S = np.float32(logits_soft_cap) * np.tanh(S / np.float32(logits_soft_cap))
         S = np.where(bad[None, None], S + DEFAULT_MASK_VALUE, S).astype(np.float32)
-        Pm = R(_softmax_f32(S))
+        P32 = _softmax_f32(S)
+        Pm = R(P32)
         O = np.einsum("jgqk,kjd->qjgd", Pm, V, dtype=np.float32, optimize=True).reshape(q_len, Hq, D)
         if v_scale is not None:
             O = O * np.float32(v_scale)
         out[q_start:q_start + q_len] = Rq(O)
+        if slack is not None:
+            jump = np.abs(R(P32 * np.float32(1 + 1e-5)) - R(P32 * np.float32(1 - 1e-5)))    # [Hkv, hrep, q, k]
+            vmax = np.abs(V.astype(np.float32)).max(axis=2)                                 # [k, Hkv]
+            row = np.einsum("jgqk,kj->qjg", jump, vmax).reshape(q_len, Hq)
+            slack[q_start:q_start + q_len] = row * np.float32(1.0 if v_scale is None else v_scale)
     return out, cache

@@ -65,16 +65,24 @@ def assert_bf16_parity(out, ref, rows, what=""):
     return mx, mean
 
 
-def assert_bf16_parity_stepwise(out, ref, what=""):
+def assert_bf16_parity_stepwise(out, ref, what="", exact=None):
     """The parity bound, widened to two bf16 steps of the value where that is larger: rows that see one or two keys
     return values of magnitude 2..8, whose step is 0.016..0.031, and the reference's chain of bf16 roundings puts its
-    restatement up to 1.5 steps from the float64 value there."""
+    restatement up to 1.5 steps from the float64 value there.  With `exact` (the float64 evaluation) an element may
+    pass that bound only where the restatement is the outlier: the device value must then lie within one bf16 step of
+    the float64 value and nearer to it than the restatement does (rows of a few keys on the prefill tiles, whose
+    fp32 logits land on the bf16 value next to the float64 one while the restatement sits three steps away)."""
     ref = np.asarray(ref, np.float64)
-    d = np.abs(np.asarray(out, np.float64) - ref)
+    out64 = np.asarray(out, np.float64)
+    d = np.abs(out64 - ref)
     step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 7)
     assert np.isfinite(np.asarray(out)).all(), f"{what}: non-finite output"
-    assert (d <= np.maximum(BF16_MAX_ABS, 2 * step)).all() and d.mean() <= BF16_MEAN_ABS, \
-        f"{what}: max-abs {d.max():.4g} mean-abs {d.mean():.4g}"
+    over = d > np.maximum(BF16_MAX_ABS, 2 * step)
+    if exact is not None and over.any():
+        ex = np.asarray(exact, np.float64)
+        near = (np.abs(out64 - ex) <= step) & (np.abs(out64 - ex) < np.abs(ref - ex))
+        over &= ~near
+    assert not over.any() and d.mean() <= BF16_MEAN_ABS, f"{what}: max-abs {d.max():.4g} mean-abs {d.mean():.4g}"
 
 
 def random_rpa_batch(seed, device, head_dims=(64, 128, 256)):
@@ -100,6 +108,8 @@ def random_rpa_batch(seed, device, head_dims=(64, 128, 256)):
         q_lens.append(q)
         kv_lens.append(q + prior)
     pps = -(-max(max(kv_lens), 1) // page) + int(rng.integers(0, 3))
+    if pps >= 64:  # the reference's block-table windows of 64 entries clamp at the end of a row that is not a multiple
+        pps = -(-pps // 64) * 64  # of 64 long and then read the wrong pages: the restatement reproduces that, avoid it
     window = None if rng.random() < 0.5 else int(rng.integers(1, 200))
     cap = None if rng.random() < 0.6 else float(rng.choice([5.0, 20.0, 50.0]))
     extra = int(rng.integers(0, 4))

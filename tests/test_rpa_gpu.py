@@ -261,12 +261,14 @@ def test_bf16_sinks(flags, shape):
     assert np.abs(base - out)[: b.total_valid_tokens].max() > 1e-3  # sinks change the result
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", list(range(24)) + list(range(1000, 1120)))
 def test_bf16_random_batches(seed):
     """Seeded random shapes on the MFMA path and on the scalar path: the parity bound against the op-by-op restatement
     on every row where that is finite (rows it turns NaN -- its first-KV-block defect under a window -- are left to
     the second check), and a bound of 4e-2 / 2e-3 against the float64 evaluation on every row (bf16 logits alone put
-    up to 2.5e-2 between the restatement and float64 here)."""
+    up to 2.5e-2 between the restatement and float64 here).  An element further from the restatement than the bound
+    is accepted only where the device value is the one next to the float64 value (seeds 1039 and 1118 hold one such
+    element each on the prefill tiles: restatement 0.018-0.021 from float64, device 0.003-0.005)."""
     b, what = random_rpa_batch(seed, DEV)
     rows = b.total_valid_tokens
     strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
@@ -275,7 +277,7 @@ def test_bf16_random_batches(seed):
         out = to_np(run_hip(b, flags))
         assert np.isfinite(out[:rows]).all(), what
         if finite.any():
-            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}")
+            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}", exact=exact[finite])
         mx, mean = err_stats(out, exact, rows)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
         assert not out[rows:].any()

@@ -176,7 +176,7 @@ def test_full_size_workload(name, n_sample):
     assert checksum_after != checksum_before
 
 
-@pytest.mark.parametrize("seed", range(100, 116))
+@pytest.mark.parametrize("seed", range(100, 164))
 def test_bf16_random_batches(seed):
     """Seeded random shapes (head_dim 128 and 256) on both paths: the cache bit for bit, the outputs within the parity
     bound of the restatement (two bf16 steps of the value where that is larger)."""
@@ -263,18 +263,31 @@ def test_e4m3_rejections():
         ragged_page_attention_v3(*fnuz)
 
 
-@pytest.mark.parametrize("seed", range(200, 212))
+@pytest.mark.parametrize("seed", list(range(200, 240)) + [1123, 1341])
 def test_e4m3_random_batches(seed):
+    """Seeded random shapes with an 8-bit cache (e4m3 on even seeds, e5m2 on odd ones): the cache bit for bit, the
+    outputs within the parity bound.  A probability that sits on a rounding boundary of the 8-bit type may round the
+    other way on the device (another exponential, a reciprocal instead of a division), which moves the row by one 8-bit
+    step of that probability times the value row: the restatement reports that allowance per row (zero nearly
+    everywhere) and it is added to the bound.  Seeds 1123 and 1341 hold such a row (0.027 and 0.19 from the
+    restatement in one (token, head) row each, every other row bit for bit)."""
     b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))
     if b.meta["num_kv_heads"] % 2:
         pytest.skip("an odd number of kv heads pads the packed cache: rejected")
     rows = b.total_valid_tokens
     v = to_v3(b, seed=seed, cache_dtype=F8 if seed % 2 == 0 else torch.float8_e5m2)
-    ref_out, ref_cache = oracle_e4m3(v)
+    slack = np.zeros((v.queries.shape[0], v.queries.shape[1]), np.float32)
+    ref_out, ref_cache = oracle_e4m3(v, slack=slack)
     out, cache = run_hip(v)
     assert np.array_equal(to_np(cache), ref_cache), what
     if rows:
-        assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], what)
+        got, ref = to_np(out)[:rows].astype(np.float64), np.asarray(ref_out[:rows], np.float64)
+        d = np.abs(got - ref)
+        step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 7)
+        bound = np.maximum(2e-2, 2 * step) + 1.01 * slack[:rows, :, None] + step * (slack[:rows, :, None] > 0)
+        assert np.isfinite(got).all() and (d <= bound).all(), f"{what}: max-abs {d.max():.4g}, over the bound {(d > bound).sum()}"
+        assert d[slack[:rows] == 0].mean() <= 2e-3 if (slack[:rows] == 0).any() else True
+        assert (slack[:rows] > 0).mean() <= 0.05, f"{what}: {(slack[:rows] > 0).mean():.3f} of the rows carry an allowance"
 
 
 @pytest.mark.parametrize("name,n_sample,f8", [("decode_llama3_8b", 10, torch.float8_e4m3fn),
