@@ -237,3 +237,31 @@ def test_e4m3_query_is_clipped_and_cast_when_q_scale_is_given():
     for h in range(2):
         np.testing.assert_array_equal(out[1, h], bf(0.75 * v[0, h] + 0.25 * v[1, h]))
         np.testing.assert_array_equal(out[0, h], bf(v[0, h]))
+
+
+def test_slack_reports_probabilities_on_a_rounding_boundary_only():
+    # Two keys whose logits differ by ln(0.40625 / 0.59375): p = (0.40625, 0.59375).  In e5m2 the first is the
+    # midpoint of 0.375 and 0.4375 (step 0.0625), the second lies 0.03 from the nearest midpoint (0.5625): the row's
+    # allowance is 0.0625 * max|v1|.  The first token sees one key (p = 1, exact): no allowance.
+    rng = np.random.default_rng(10)
+    q, k, v, cache, lens, bt, qsl, dist = make_e4m3(rng, [2], [2], page=4, Hq=2, Hkv=2)
+    R = rpa_oracle._rounder("float8_e5m2")
+    k, v, cache = R(k), R(v), R(cache)
+    q[:] = 0
+    q[1, :, 0] = 1.0
+    k[:] = 0
+    k[0, :, 0] = 1.0
+    scale = float(np.log(0.40625 / 0.59375))
+    slack = np.full((2, 2), np.nan, np.float32)
+    out, _ = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, softmax_scale=scale, cache_dtype="float8_e5m2",
+                    query_dtype="bfloat16", slack=slack)
+    for h in range(2):
+        assert slack[0, h] == 0
+        assert slack[1, h] == np.float32(0.0625) * np.abs(v[0, h]).max()
+        p0 = 0.375 if np.array_equal(out[1, h], bf(0.375 * v[0, h] + 0.625 * v[1, h])) else 0.4375
+        np.testing.assert_array_equal(out[1, h], bf(np.float32(p0) * v[0, h] + np.float32(0.625) * v[1, h]))
+    # away from every boundary the allowance is zero: p = (0.75, 0.25)
+    slack[:] = np.nan
+    rpa_v3(q, k, v, cache, lens, bt, qsl, dist, softmax_scale=float(np.log(3.0)), cache_dtype="float8_e5m2",
+           query_dtype="bfloat16", slack=slack)
+    assert not slack.any()
