@@ -315,6 +315,15 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
       return rpa::fail(RPA_ERR_WORKSPACE, "workspace of %llu bytes is too small, rpa_v3_workspace_bytes() asks for %llu",
                        (unsigned long long)v.attn.workspace_bytes, (unsigned long long)need);
   }
+  // Everything that can fail is checked before the cache is touched: a rejected call leaves the cache as it was.
+  if (!fp8 && rpa::tiled_supported(v.attn)) {
+    const uint64_t need = rpa_workspace_bytes(&v.attn);
+    if (v.attn.workspace == nullptr || v.attn.workspace_bytes < need)
+      return rpa::fail(RPA_ERR_WORKSPACE, "workspace of %llu bytes is too small, rpa_v3_workspace_bytes() asks for %llu",
+                       (unsigned long long)v.attn.workspace_bytes, (unsigned long long)need);
+  }
+  if (v.attn.head_dim > 512 || (static_cast<uint64_t>(v.attn.head_dim) * (fp8 ? 1 : v.attn.dtype == RPA_DTYPE_BF16 ? 2 : 4)) % 16 != 0)
+    return rpa::fail(RPA_ERR_UNSUPPORTED, "head_dim=%d: rows must be a multiple of 16 bytes and head_dim at most 512", v.attn.head_dim);
   rc = rpa::launch_kv_cache_update(v, stream);
   if (rc == RPA_ERR_UNSUPPORTED)
     return rpa::fail(rc, "head_dim=%d rows are not a multiple of 16 bytes", v.attn.head_dim);

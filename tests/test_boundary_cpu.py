@@ -104,6 +104,13 @@ def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
     assert lib.rpa_v3_launch(ctypes.byref(v), None) == -2 and b"bf16 queries" in lib.rpa_last_error()
     v.cache_dtype = _native.RPA_DTYPE_BF16                    # a float32 call with a bf16 cache: neither rule holds
     assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_dtype" in lib.rpa_last_error()
+    # what the attention step would reject is rejected before the cache update runs: a failed call leaves the cache alone
+    p.dtype, p.compute = _native.RPA_DTYPE_BF16, _native.RPA_COMPUTE_BF16
+    p.workspace_bytes = plain - 1
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -3 and b"too small" in lib.rpa_last_error()
+    p.workspace_bytes = plain
+    p.head_dim = 520                                          # beyond the scalar kernel
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -2 and b"at most 512" in lib.rpa_last_error()
 
 
 def test_workspace_bytes_and_errors_without_gpu():
