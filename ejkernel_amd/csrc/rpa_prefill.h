@@ -28,7 +28,9 @@ namespace rpa {
 
 template <int D, int MRT>
 struct PCfg {
-  static constexpr int NS = D / 128;                 // 128-wide slices of head_dim
+  static constexpr int SW = D < 128 ? D : 128;       // width of a slice of head_dim
+  static constexpr int NS = D / SW;                  // slices
+  static constexpr int CB = SW / 16;                 // MFMA column blocks (16 output elements) per slice
   static constexpr int NKS = D / 32;                 // k-steps of the QK^T contraction
 #ifndef RPA_PF_NH
 #define RPA_PF_NH 2
@@ -36,7 +38,7 @@ struct PCfg {
 #ifndef RPA_PF_NSTG
 #define RPA_PF_NSTG 2
 #endif
-  static constexpr int NH = D == 128 ? RPA_PF_NH : 1;  // 32-token halves per step
+  static constexpr int NH = D <= 128 ? RPA_PF_NH : 1;  // 32-token halves per step
   static constexpr int TK = 32 * NH;                 // tokens per step
   static constexpr int ROWB = D * 2;                 // LDS bytes per row
   static constexpr int WROWS = 16 * MRT;             // rows per wavefront
@@ -51,7 +53,12 @@ struct PCfg {
   // V^T operands come from the transposing LDS read (V tile stored by column units) or, where the tile is LDS-bound
   // (16 rows per wavefront at head_dim 256), from 16-byte reads of a row-major tile plus byte permutes: the
   // transposing read moves 8 bytes per lane and takes more LDS time for the same operands.
-  static constexpr bool TRV = D == 128;
+  static constexpr bool TRV = D <= 128;
+  // K rows sit unpadded in LDS with their 16-byte pieces XOR-swizzled by a function of the row number, chosen so
+  // that the 16 rows read by one quarter of a wave-wide operand read cover all 64 banks: with 256-byte rows (and
+  // longer ones) the row number itself; with 128-byte rows two rows share a bank line, and the row pair number is
+  // what has to differ.  The function only depends on the row modulo 16, so sub-tiles are compile-time offsets.
+  static __device__ __forceinline__ int swz(int row) { return D == 64 ? (row >> 1) & 7 : row & 15; }
 };
 
 constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point by this much before O is rescaled
@@ -72,8 +79,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const float cap = p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
   const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
-  // head_dim 64 runs on the 128-wide instantiation: q is padded with zeros and the upper half of every K / V row in
-  // LDS repeats the lower half (K: multiplied by zero; V: output elements that are not stored).
+  // (A head_dim below the instantiation's runs too: q is padded with zeros and the upper part of every K / V row in
+  // LDS repeats the lower part -- K: multiplied by zero; V: output elements that are not stored.)
   const int hd = p.head_dim;
   const uint32_t pmask = static_cast<uint32_t>(hd / 8 - 1);  // 16-byte pieces of a row that exist in memory
 
@@ -155,7 +162,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const int w_act_hi = w_any ? min(range_hi - 1, w_pos_hi) : -0x7fffffff;
   const int w_act_lo = W > 0 ? w_pos_lo - W - 31 : -0x7fffffff;
 
-  f32x4_t o_acc[MRT][C::NS][8];
+  f32x4_t o_acc[MRT][C::NS][C::CB];
   f32x4_t l_acc[MRT];
   // Softmax reference point m per row, kept as the exp2 offset -m log2(e) (0 while the row has seen no key) and
   // as the vote threshold for exp2 arguments: kLazy log2(e) once there is a reference point, -inf before.
@@ -168,12 +175,13 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-      for (int c = 0; c < 8; ++c) o_acc[m][sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      for (int c = 0; c < C::CB; ++c) o_acc[m][sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 
   // ---- cooperative fetch.  One wave-wide direct-to-LDS load moves a block of RB rows: the LDS side is 1 KiB in
   // lane order, so lane l fills piece slot l % PR of row l / PR and fetches the piece that the swizzle assigns
-  // to that slot.  Block-table entries are scalar loads (the rows of a block always share a page).
+  // to that slot.  Block-table entries are scalar loads (the rows of a block share a page, except with pages
+  // shorter than a block).
   const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * hd) * 2u;
   const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
@@ -190,7 +198,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
   for (int n = 0; n < HB; ++n) {
     const int t_local = GROUP * wave + C::RB * n + l_row;
-    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
   }
   const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + hd * 2;  // V block 0; block n adds RB rows
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
@@ -221,16 +229,31 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int n = 0; n < HB; ++n) {
       const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
+      if (C::RB > 4 && p.page_size < C::RB) {
+        // pages shorter than a block (pages of 4 tokens under 128-byte rows): every lane looks its own row's page up
+        const int t_local = GROUP * wave + C::RB * n + l_row;
+        auto row_base = [&](int tok) {
+          const int pg = min(max(p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + (tok >> a.page_shift)], 0), p.num_pages - 1);
+          return kvb + static_cast<uint64_t>(pg) * page_b + static_cast<uint64_t>(tok & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+        };
+        __builtin_amdgcn_global_load_lds(
+            reinterpret_cast<const u32x4_t*>(row_base(min(t_c + l_row, t_last)) + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask)),
+            (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
+        const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(row_base(min(t_c + v_row, t_last)) + v_piece + hd * 2),
+                                         (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+        continue;
+      }
       const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
                           static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
       const int tok = min(t_c + l_row, t_last);
       const int t_local = GROUP * wave + C::RB * n + l_row;
-      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
+      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
       __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
                                        (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
       const int v_tok = min(t_c + v_row, t_last);
-      const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ (t_local & 15)) & pmask);
+      const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
       __builtin_amdgcn_global_load_lds(
           reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + hd * 2),
           (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
@@ -257,7 +280,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // a later sub-tile or half is a compile-time constant on top of them (the swizzle only uses row & 15).
   int k_off[C::NKS];
 #pragma unroll
-  for (int ks = 0; ks < C::NKS; ++ks) k_off[ks] = i * C::ROWB + 16 * ((4 * ks + g) ^ i);
+  for (int ks = 0; ks < C::NKS; ++ks) k_off[ks] = i * C::ROWB + 16 * ((4 * ks + g) ^ C::swz(i));
   // V^T operands come from the transposing 64-bit LDS read: in each group of 16 lanes, lanes 4e..4e+3 point at
   // 16 consecutive elements of row e (8 bytes per lane) and lane x receives element x of rows 0..3.  Rows are the
   // four keys 4g..4g+3 of a 16-key sub-tile, the elements one 32-byte column unit; everything else about the
@@ -282,7 +305,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     // so their LDS latency (and the barrier that publishes the next tile) hides behind matrix work.  At head_dim
     // 256 only the first sub-tile's operands are held that long, for lack of registers; the second sub-tile's are
     // requested when the half starts and land while the first sub-tile's MFMAs run.
-    constexpr int KAHEAD = D == 128 ? 2 : 1;
+    constexpr int KAHEAD = D <= 128 ? 2 : 1;
     u32x4_t kop[2][C::NKS];
     auto load_k_sub = [&](const char* kt_n, int h_n, int u) {
 #pragma unroll
@@ -310,11 +333,11 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         auto load_v = [&](int sN) {
           if constexpr (C::TRV) {
 #pragma unroll
-            for (int c = 0; c < 8; ++c)
+            for (int c = 0; c < C::CB; ++c)
 #pragma unroll
               for (int u = 0; u < 2; ++u) {
                 const s16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
-                    vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + 8 * sN) * (C::RB * 32)));
+                    vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + C::CB * sN) * (C::RB * 32)));
                 const u32x2_t t2 = __builtin_bit_cast(u32x2_t, t);
                 vraw[c][2 * u] = t2[0];
                 vraw[c][2 * u + 1] = t2[1];
@@ -325,7 +348,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               vraw[e] = *reinterpret_cast<const u32x4_t*>(vt + (32 * h + 16 * (e >> 2)) * C::ROWB + v_off[sN][e & 3]);
           }
         };
-        constexpr int V_READS = C::TRV ? 16 : 8;
+        constexpr int V_READS = C::TRV ? 2 * C::CB : 8;
         u32x4_t pw[MRT];
         if (active) {
         // S^T = K Q^T for the two 16-key sub-tiles, then the V operands of the first slice are requested: they
@@ -423,7 +446,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
             for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int c = 0; c < 8; ++c) o_acc[m][sN][c] *= alpha;
+              for (int c = 0; c < C::CB; ++c) o_acc[m][sN][c] *= alpha;
           }
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
@@ -461,7 +484,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           for (int sN = 0; sN < C::NS; ++sN) {
             if (sN > 0) load_v(sN);
 #pragma unroll
-            for (int c = 0; c < 8; ++c) {
+            for (int c = 0; c < C::CB; ++c) {
               u32x4_t av;
               if constexpr (C::TRV) {
                 av = vraw[c];
@@ -522,7 +545,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-        for (int c = 0; c < 8; ++c) {
+        for (int c = 0; c < C::CB; ++c) {
           u32x2_t w;
           w[0] = pack_bf16x2(o_acc[m][sN][c][0] * inv, o_acc[m][sN][c][1] * inv);
           w[1] = pack_bf16x2(o_acc[m][sN][c][2] * inv, o_acc[m][sN][c][3] * inv);

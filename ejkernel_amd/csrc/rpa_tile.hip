@@ -54,7 +54,8 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 // this instantiation for small batches; it is also the one that merges an attention state in a.pre into every row.
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
-  using C = Cfg<D, NT, kMimic>;
+  constexpr int DD = D < 128 ? 128 : D;  // head_dim 64: the wave-level loop works 128 wide, prefill tiles 64 wide
+  using C = Cfg<DD, NT, kMimic>;
   using PC = PCfg<D, MRT>;
   extern __shared__ __align__(16) char smem[];
   const RpaParams& p = a.p;
@@ -330,7 +331,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         const int range_lo = max(p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0, si.start) & ~(C::TT - 1);
         Part part;
         part.partial = false;
-        process_item<D, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+        process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
       }
 
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           part.last_w = sh.owner(part.stream_a + per_head - 1);
           part.partial = part.first_w != part.last_w;
           part.slot = part_slot(worker, part.stream_a, sh);
-          process_item<D, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
           x += t1 - t0;
         }
       }
@@ -401,7 +402,7 @@ static int tiled_grid() {
 bool tiled_supported(const RpaParams& p) {
   if (p.flags & RPA_FLAG_FORCE_GENERIC) return false;
   if (p.dtype != RPA_DTYPE_BF16 || p.compute != RPA_COMPUTE_BF16) return false;
-  if (p.head_dim != 64 && p.head_dim != 128 && p.head_dim != 256) return false;  // 64 runs on the 128-wide kernel
+  if (p.head_dim != 64 && p.head_dim != 128 && p.head_dim != 256) return false;
   if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
   if (p.max_num_seqs > (kTiledMaxSeqs << kTiledMaxSchedShift)) return false;
   if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kQueueCounterIndex * 4ull) return false;
@@ -423,7 +424,7 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
 
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
-  using C = Cfg<D, NT, kMimic>;
+  using C = Cfg<(D < 128 ? 128 : D), NT, kMimic>;
   using PC = PCfg<D, MRT>;
   const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE, static_cast<size_t>(PC::LDS));
   const size_t lds = sched_bytes((a.p.max_num_seqs + (1 << a.sched_shift) - 1) >> a.sched_shift) + data;
@@ -496,6 +497,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);
     return mimic ? launch_cfg<256, 1, 1, true, true>(a, grid, stream) : launch_cfg<256, 1, 1, false, true>(a, grid, stream);
   }
+  if (p.head_dim == 64)
+    return mimic ? launch_cfg<64, 2, 4, true>(a, grid, stream) : launch_cfg<64, 2, 4, false>(a, grid, stream);
   if (p.head_dim <= 128)
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);

@@ -167,6 +167,31 @@ def test_bf16_prefill_tiles_over_many_key_tiles(flags, hq, hkv, D, window):
     assert_bf16_parity(out, run_strict(b), b.total_valid_tokens, f"prefill tiles {hq}/{hkv} D={D} W={window}")
 
 
+@pytest.mark.parametrize("page", [4, 8, 16, 64])
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (16, 2), (6, 2)])
+@pytest.mark.parametrize("window,sinks", [(None, False), (48, True)])
+def test_bf16_head_dim_64_prefill_tiles(page, hq, hkv, window, sinks):
+    """head_dim 64 has prefill tiles of its own: 256 rows per workgroup, 128-byte K/V rows (two rows per LDS bank
+    line, eight rows per fetch block -- more than a page of four tokens holds).  Chunks of one partial tile, of two
+    and of five tiles, with and without earlier context, a window and sinks (the attention shape of gpt-oss)."""
+    pps = -(-576 // page)
+    pps = pps if pps < 64 else -(-pps // 64) * 64   # the reference's block-table windows clamp in rows of other lengths
+    b = small([300, 1, 70, 130, 3], [300, 300, 100, 517, 90], num_q_heads=hq, num_kv_heads=hkv, head_dim=64,
+              page_size=page, pages_per_seq=pps, sliding_window=window)
+    aux = None
+    if sinks:
+        aux = torch.from_numpy(np.random.default_rng(4).standard_normal((hq, 1)).astype(np.float32)).to(torch.bfloat16)
+    out = to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES, softmax_aux=None if aux is None else aux.to(DEV)))
+    aux_np = None if aux is None else aux.float().numpy()
+    rows, what = b.total_valid_tokens, f"D=64 tiles page {page} {hq}/{hkv} W={window} sinks={sinks}"
+    strict, exact = run_strict(b, softmax_aux=aux_np)[:rows], run_exact(b, softmax_aux=aux_np)[:rows]
+    finite = np.isfinite(strict).all(axis=(1, 2))  # short pages: the restatement's first KV block under a window is NaN
+    assert finite.mean() > 0.5
+    assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], what, exact=exact[finite])
+    mx, mean = err_stats(out, exact, rows)
+    assert mx <= 4e-2 and mean <= 2e-3, f"{what}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
+
+
 @pytest.mark.parametrize("hq,hkv,D", [(8, 2, 128), (16, 2, 256), (8, 2, 64)])
 @pytest.mark.parametrize("window", [None, 48])
 def test_bf16_long_chunks_in_a_decode_shaped_batch(hq, hkv, D, window):
