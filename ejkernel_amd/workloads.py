@@ -326,6 +326,8 @@ WORKLOADS = {
     "mixed_decode_only": "the 240 decode sequences of mixed_prefill_decode: 1 token each, kv 256..8192",
     # long prompts: every prefill tile walks thousands of keys (the per-tile costs of the 512-token chunks vanish)
     "prefill_long": "2 prompts x 8192 tokens from scratch, 32q/8kv heads, D=128, page 32",
+    # head_dim 64 with many query heads per kv head (the attention shape of gpt-oss), chunked prefill
+    "prefill_head_dim_64": "32 chunks x 512 tokens after 2048, 64q/8kv heads, D=64, page 32",
 }
 
 
@@ -375,6 +377,11 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         L = n(8192)
         return make_batch(np.full(2, L), np.full(2, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
                           pages_per_seq=pages(L, 32), seed=seed, device=device, dtype=dtype, name=name)
+    if name == "prefill_head_dim_64":
+        S, chunk, prior = n(32), n(512), n(2048)
+        return make_batch(np.full(S, chunk), np.full(S, prior + chunk), num_q_heads=64, num_kv_heads=8, head_dim=64,
+                          page_size=32, pages_per_seq=pages(prior + chunk, 32), seed=seed, device=device, dtype=dtype,
+                          name=name)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)
