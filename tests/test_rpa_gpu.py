@@ -192,6 +192,19 @@ def test_bf16_head_dim_64_prefill_tiles(page, hq, hkv, window, sinks):
     assert mx <= 4e-2 and mean <= 2e-3, f"{what}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
 
 
+@pytest.mark.parametrize("D", [64, 128, 256])
+@pytest.mark.parametrize("window,cap", [(None, None), (48, 20.0)])
+def test_bf16_fp32_logit_arithmetic_on_prefill_tiles(D, window, cap):
+    """RPA_FLAG_FP32_LOGITS (the arithmetic of ragged_page_attention_v3: the query enters unscaled, the fp32 logits
+    take the scale) on the prefill tiles of every head_dim, against the float64 evaluation: what is left is the bf16
+    rounding of the probabilities and of the output."""
+    b = small([300, 1, 70, 130, 3], [300, 300, 100, 517, 90], num_q_heads=8, num_kv_heads=2, head_dim=D,
+              page_size=16, pages_per_seq=36, sliding_window=window, logits_soft_cap=cap)
+    out = to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_FP32_LOGITS))
+    mx, mean = err_stats(out, run_exact(b), b.total_valid_tokens)
+    assert np.isfinite(out).all() and mx <= 2e-2 and mean <= 1e-3, f"D={D} W={window} cap={cap}: max-abs {mx:.4g} mean-abs {mean:.4g}"
+
+
 @pytest.mark.parametrize("hq,hkv,D", [(8, 2, 128), (16, 2, 256), (8, 2, 64)])
 @pytest.mark.parametrize("window", [None, 48])
 def test_bf16_long_chunks_in_a_decode_shaped_batch(hq, hkv, D, window):
