@@ -13,7 +13,7 @@ from pathlib import Path
 # RPA_LIBRARY points at another build of the same library (e.g. one compiled with different tile constants).
 LIB_PATH = Path(os.environ.get("RPA_LIBRARY") or Path(__file__).resolve().parent / "lib" / "librpa_mi355x.so")
 
-RPA_ABI_VERSION = 5
+RPA_ABI_VERSION = 6
 RPA_DTYPE_BF16, RPA_DTYPE_F32, RPA_DTYPE_FP8_E4M3, RPA_DTYPE_FP8_E5M2 = 0, 1, 2, 3
 RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
@@ -83,7 +83,7 @@ class RpaV3Params(ctypes.Structure):
         ("new_keys", ctypes.c_void_p),
         ("new_values", ctypes.c_void_p),
         ("cache_dtype", ctypes.c_int32),
-        ("reserved", ctypes.c_int32),
+        ("cache_head_dim", ctypes.c_int32),
     ]
 
 

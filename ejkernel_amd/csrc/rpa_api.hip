@@ -303,6 +303,11 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
     return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_dtype=%d: the cache has the dtype of the queries (%d) or is RPA_DTYPE_FP8_E4M3 / RPA_DTYPE_FP8_E5M2",
                      v.cache_dtype, v.attn.dtype);
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+  const uint32_t esize = fp8 ? 1u : v.attn.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
+  const int chd = v.cache_head_dim > 0 ? v.cache_head_dim : v.attn.head_dim;  // elements per cache row
+  if (chd < v.attn.head_dim || (static_cast<uint64_t>(chd) * esize) % 16 != 0)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_head_dim=%d: rows hold head_dim=%d elements at least and are a multiple of 16 bytes",
+                     v.cache_head_dim, v.attn.head_dim);
   if (fp8) {
     if (v.attn.dtype != RPA_DTYPE_BF16 || v.attn.compute != RPA_COMPUTE_BF16)
       return rpa::fail(RPA_ERR_UNSUPPORTED, "an 8-bit cache takes bf16 queries and RPA_COMPUTE_BF16");
@@ -328,16 +333,19 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (rc == RPA_ERR_UNSUPPORTED)
     return rpa::fail(rc, "head_dim=%d rows are not a multiple of 16 bytes", v.attn.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "cache update launch failed: %s", hipGetErrorString(hipGetLastError()));
-  if (!fp8) return rpa_fwd_launch(&v.attn, hip_stream);
+  if (!fp8 && chd == v.attn.head_dim) return rpa_fwd_launch(&v.attn, hip_stream);
 
+  // 8-bit elements or padded rows: the cache is addressed through its own strides (K row of head j at combined
+  // head 2j, its V row at 2j + 1, chd elements each)
   const RpaParams& p = v.attn;
   rpa::KvLayout kv;
   kv.k_base = static_cast<const char*>(p.kv_pages);
-  kv.v_base = kv.k_base + p.head_dim;
-  kv.stride_b = 2u * p.num_kv_heads * p.head_dim;
+  kv.v_base = kv.k_base + static_cast<size_t>(chd) * esize;
+  kv.stride_b = 2u * p.num_kv_heads * chd * esize;
   kv.page_b = static_cast<uint64_t>(p.page_size) * kv.stride_b;
-  kv.head_b = 2u * p.head_dim;
+  kv.head_b = 2u * chd * esize;
   kv.contiguous = 0;
+  if (!fp8) return rpa::dispatch(p, kv, rpa::tiled_supported(p), stream);
   const uint64_t base = (rpa_workspace_bytes(&p) + 255) & ~255ull;
   float* stats = reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base);
   RpaParams q = p;

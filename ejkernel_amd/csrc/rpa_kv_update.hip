@@ -1,4 +1,4 @@
-// Cache update of ragged_page_attention_v3: token t of sequence s (t in [q_start, q_start + q_len)) is the key /
+// Cache update of ragged_page_attention_v3 (rows of the cache may be longer than head_dim: the padding stays as it is): token t of sequence s (t in [q_start, q_start + q_len)) is the key /
 // value at position kv_len - q_len + (t - q_start) of that sequence, and its rows go to
 // cache[block_tables[s, pos / page], pos % page, 2j | 2j + 1, :] for every kv head j
 // (ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:44-57 merge_kv, :207-218 update).
@@ -10,7 +10,7 @@
 namespace rpa {
 
 __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const char* __restrict__ new_k,
-                                                              const char* __restrict__ new_v, int row_bytes) {
+                                                              const char* __restrict__ new_v, int row_bytes, int dst_row_bytes) {
   const int t = blockIdx.x;
   int nseq = p.num_seqs[0];
   nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
@@ -23,23 +23,25 @@ __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const
   int page = p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + pos / p.page_size];
   page = page < 0 ? 0 : (page >= p.num_pages ? p.num_pages - 1 : page);
   const size_t tok = static_cast<size_t>(page) * p.page_size + pos % p.page_size;
-  char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * 2 * p.num_kv_heads * row_bytes;
+  char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * 2 * p.num_kv_heads * dst_row_bytes;
   const size_t src_off = static_cast<size_t>(t) * p.num_kv_heads * row_bytes;
   const int pieces_per_row = row_bytes / 16, n = 2 * p.num_kv_heads * pieces_per_row;
   for (int k = threadIdx.x; k < n; k += blockDim.x) {
     const int row = k / pieces_per_row, piece = k - row * pieces_per_row;  // row = combined head 2j (K) or 2j + 1 (V)
     const char* src = ((row & 1) ? new_v : new_k) + src_off + static_cast<size_t>(row >> 1) * row_bytes + 16 * piece;
-    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(row) * row_bytes + 16 * piece) = *reinterpret_cast<const uint4*>(src);
+    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(row) * dst_row_bytes + 16 * piece) = *reinterpret_cast<const uint4*>(src);
   }
 }
 
 int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream) {
   const RpaParams& p = v.attn;
   if (p.total_tokens == 0) return RPA_OK;
-  const int row_bytes = p.head_dim * (v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 1 : v.cache_dtype == RPA_DTYPE_BF16 ? 2 : 4);
-  if (row_bytes % 16 != 0) return RPA_ERR_UNSUPPORTED;
+  const int esize = v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 1 : v.cache_dtype == RPA_DTYPE_BF16 ? 2 : 4;
+  const int row_bytes = p.head_dim * esize;
+  const int dst_row_bytes = (v.cache_head_dim > 0 ? v.cache_head_dim : p.head_dim) * esize;
+  if (row_bytes % 16 != 0 || dst_row_bytes % 16 != 0 || dst_row_bytes < row_bytes) return RPA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_cache_update_kernel, dim3(p.total_tokens), dim3(256), 0, stream, p,
-                     static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes);
+                     static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes, dst_row_bytes);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 

@@ -491,7 +491,12 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
   const bool small_batch = p.query_start_loc == nullptr || ((p.flags & RPA_FLAG_PREFILL_TILES) == 0 &&
                                                             rows <= env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows));
-  const bool wave_only = pre.ml != nullptr || (small_batch && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
+  // Prefill tiles address the cache as [page][slot][2 * kv heads][head_dim]; any other layout (two caches, one
+  // contiguous cache per sequence, rows padded beyond head_dim) runs through the wave-level loop alone.
+  const KvLayout canon = interleaved_layout(p);
+  const bool canonical = kv.k_base == canon.k_base && kv.v_base == canon.v_base && kv.stride_b == canon.stride_b &&
+                         kv.head_b == canon.head_b && kv.page_b == canon.page_b && kv.contiguous == 0;
+  const bool wave_only = pre.ml != nullptr || !canonical || (small_batch && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
   if (wave_only) {
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);

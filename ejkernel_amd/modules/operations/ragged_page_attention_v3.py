@@ -10,8 +10,10 @@ The cache is updated in place and returned (the reference donates it,
 ``_kernel.py:124``).  Its five-dimensional layout
 ``[num_pages, page_size, 2 * num_kv_heads / packing, packing, head_dim_padded]`` is, for a
 head_dim that is a multiple of 128 and an even combined-head count, byte for byte the
-``[num_pages, page_size, 2 * num_kv_heads, head_dim]`` layout of the v2 operation; other
-shapes (padded head_dim, a padded odd head count) are rejected here.
+``[num_pages, page_size, 2 * num_kv_heads, head_dim]`` layout of the v2 operation.  A head_dim
+that is no multiple of 128 has its rows padded to one (``merge_kv``, ``_kernel.py:44-57``): the
+kernels then walk the cache with the row pitch of the padded rows and neither read nor write
+the padding.  A padded combined-head count is rejected here.
 
 ``distribution[-1]`` is the number of sequences (``_kernel.py:195``).
 
@@ -83,8 +85,6 @@ def _static_validate(q, k, v, kv_cache, kv_lens, block_tables, query_start_loc, 
     if logits_soft_cap is not None and logits_soft_cap == 0.0:
         raise ValueError("soft_cap != 0")
     # limits of this implementation
-    if dalign != d:
-        raise ValueError(f"head_dim={d} must be a multiple of 128 here (a padded cache row is not supported)")
     if hx2_per_pack * pack != 2 * hkv:
         raise ValueError("a cache with padded combined heads is not supported")
     if not (k.dtype == v.dtype == kv_cache.dtype):
@@ -159,7 +159,7 @@ def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_
     v3.new_keys = keys.data_ptr()
     v3.new_values = values.data_ptr()
     v3.cache_dtype = _FP8.get(kv_cache.dtype, p.dtype)
-    v3.reserved = 0
+    v3.cache_head_dim = kv_cache.shape[4]
 
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream

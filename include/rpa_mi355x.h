@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define RPA_ABI_VERSION 5
+#define RPA_ABI_VERSION 6
 
 /* element type of queries / kv_pages / out */
 #define RPA_DTYPE_BF16 0
@@ -110,7 +110,8 @@ typedef struct RpaParams {
  * ragged_page_attention_v3: write the new tokens' K/V rows into the paged cache, then attend over it.
  * Replaces ejkernel/kernels/_xla/ragged_page_attention_v3/_interface.py:25-96 (program: _kernel.py:127-318).
  * The cache has the layout of kv_pages above, which is what merge_kv (_kernel.py:44-57) produces when head_dim
- * is a multiple of 128: [num_pages, page_size, 2*num_kv_heads / packing, packing, head_dim].
+ * is a multiple of 128: [num_pages, page_size, 2*num_kv_heads / packing, packing, head_dim]; cache_head_dim below
+ * covers the other head_dims.
  */
 typedef struct RpaV3Params {
   RpaParams attn;         /* kv_pages = the cache, updated in place; context_lens = kv_lens (they include the new  */
@@ -124,7 +125,10 @@ typedef struct RpaV3Params {
                           /* to it before P V.  It runs as two passes over                                          */
                           /* the keys (row maximum and sum, then the attention) on the MFMA kernel only, and needs  */
                           /* rpa_v3_workspace_bytes() of workspace.                                                 */
-  int32_t reserved;       /* 0 */
+  int32_t cache_head_dim; /* elements per cache row: align_to(head_dim, 128) as merge_kv pads it (_kernel.py:44-57), or 0  */
+                          /* for head_dim.  With padded rows (head_dim 64 in rows of 128) the cache is                 */
+                          /* [num_pages, page_size, 2*num_kv_heads / packing, packing, cache_head_dim]; the padding    */
+                          /* is neither read nor written.                                                               */
 } RpaV3Params;
 
 /* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */

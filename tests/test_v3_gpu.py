@@ -191,6 +191,53 @@ def test_bf16_random_batches(seed):
             assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
 
 
+@pytest.mark.parametrize("flags", [0, _native.RPA_FLAG_FORCE_GENERIC])
+@pytest.mark.parametrize("D", [64, 192])
+@pytest.mark.parametrize("window", [None, 48])
+def test_cache_rows_padded_to_a_multiple_of_128(D, flags, window):
+    """head_dim 64 lives in cache rows of 128 elements, 192 in rows of 256 (merge_kv pads them): the update writes
+    head_dim elements per row and leaves the padding alone, the attention never reads it (it holds random data).
+    head_dim 64 runs on the MFMA kernel's wave-level loop, 192 on the scalar kernel."""
+    v = small([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], head_dim=D, pages_per_seq=32, sliding_window=window)
+    dalign = -(-D // 128) * 128
+    assert v.kv_cache.shape[-1] == dalign and v.keys.shape[-1] == D
+    before = v.kv_cache.clone()
+    ref_out, ref_cache = oracle(v)
+    out, cache = run_hip(v, flags)
+    assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
+    assert torch.equal(cache[..., D:], before[..., D:]), "the padding was written"
+    assert out.shape == v.queries.shape
+    assert_bf16_parity(to_np(out), ref_out, 176, f"padded rows D={D}")
+
+
+@pytest.mark.parametrize("f8", [pytest.param(torch.float8_e4m3fn, id="e4m3"), pytest.param(torch.float8_e5m2, id="e5m2")])
+def test_8bit_cache_rows_padded_to_a_multiple_of_128(f8):
+    v = to_v3(make_batch([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], num_q_heads=8, num_kv_heads=2, head_dim=64,
+                         page_size=16, pages_per_seq=32, seed=3, device=DEV), seed=3, cache_dtype=f8)
+    assert v.kv_cache.shape[-1] == 128 and v.kv_cache.dtype == f8
+    before = v.kv_cache.clone()
+    ref_out, ref_cache = rpa_v3(*[to_np(a) for a in v.args()], cache_dtype={torch.float8_e4m3fn: "float8_e4m3fn",
+                                torch.float8_e5m2: "float8_e5m2"}[f8], query_dtype="bfloat16", **v.kwargs())
+    out, cache = run_hip(v)
+    assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
+    assert torch.equal(cache[..., 64:].view(torch.uint8), before[..., 64:].view(torch.uint8)), "the padding was written"
+    assert_bf16_parity(to_np(out), ref_out, 176, "8-bit padded rows")
+
+
+@pytest.mark.parametrize("seed", range(300, 316))
+def test_bf16_random_batches_head_dim_64(seed):
+    """Seeded random shapes at head_dim 64 (cache rows padded to 128): the cache bit for bit, outputs within the bound."""
+    b, what = random_rpa_batch(seed, DEV, head_dims=(64,))
+    rows = b.total_valid_tokens
+    for flags in (0, _native.RPA_FLAG_FORCE_GENERIC):
+        v = to_v3(random_rpa_batch(seed, DEV, head_dims=(64,))[0], seed=seed)
+        ref_out, ref_cache = oracle(v)
+        out, cache = run_hip(v, flags)
+        assert np.array_equal(to_np(cache), ref_cache), what
+        if rows:
+            assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
+
+
 # ---------------------------------------------------------------- 8-bit cache (float8_e4m3fn, bf16 queries)
 # The device follows the program's casts (Q / q_scale clipped and cast to the cache dtype, normalised probabilities
 # cast to the cache dtype), so against the restatement the only differences left are float32 evaluation order and
