@@ -186,7 +186,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   // A batch without prefill tiles is pure streaming: it runs fastest with one workgroup per compute unit, so
   // the second half of the grid (dispatched after every unit has one workgroup) leaves at once.
   const int grid_all = static_cast<int>(gridDim.x);
-  const int grid_wgs = total_wg == 0 ? min(grid_all, a.decode_grid) : grid_all;
+  const int grid_wgs = total_wg == 0 ? min(grid_all, a.stream_grid) : grid_all;
   if (static_cast<int>(blockIdx.x) >= grid_wgs) return;
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
@@ -458,7 +458,11 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
   a.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
-  a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 1));
+  // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
+  // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes
+  // in flight.
+  a.stream_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", p.head_dim == 64 ? 2 : 1));
+  a.decode_grid = device_cu_count();
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
@@ -468,7 +472,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities; both launches run
     // every sequence through the wave-level loop.  A wavefront has half the bytes in flight that it has with a
     // 16-bit cache, so both workgroups of a compute unit stream (0.70 ms against 0.84 ms on 256 x 512..8192 keys).
-    a.decode_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 2));
+    a.stream_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 2));
     int rc;
     if (kv_elem == 2) {
       rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)

@@ -22,7 +22,8 @@ struct TileArgs {
   KvLayout kv;        // K / V addressing of the decode loop (prefill tiles assume the interleaved layout)
   int page_shift;     // log2(page_size)
   int uniform_page;   // page_size >= 16: a 16-token sub-tile lies in one page
-  int decode_grid;    // workgroups that take part when the batch has no prefill tiles
+  int decode_grid;    // mixed batches: the workgroups from this one on take the decode stream first
+  int stream_grid;    // workgroups that take part when the batch has no prefill tiles
   int sched_shift;    // the schedule arrays hold every (1 << sched_shift)-th sequence's start (0: every sequence)
   int min_share_tiles; // small batches: tiles per streaming wavefront before more wavefronts are used
   int even_xcd_permille;  // share of the decode stream given to the workgroups on even XCDs, in 1/1000
