@@ -84,6 +84,8 @@ class RpaV3Params(ctypes.Structure):
         ("new_values", ctypes.c_void_p),
         ("cache_dtype", ctypes.c_int32),
         ("cache_head_dim", ctypes.c_int32),
+        ("cache_combined_heads", ctypes.c_int32),
+        ("reserved", ctypes.c_int32),
     ]
 
 

@@ -308,6 +308,10 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (chd < v.attn.head_dim || (static_cast<uint64_t>(chd) * esize) % 16 != 0)
     return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_head_dim=%d: rows hold head_dim=%d elements at least and are a multiple of 16 bytes",
                      v.cache_head_dim, v.attn.head_dim);
+  const int chx2 = v.cache_combined_heads > 0 ? v.cache_combined_heads : 2 * v.attn.num_kv_heads;  // heads per cache token
+  if (chx2 < 2 * v.attn.num_kv_heads)
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "cache_combined_heads=%d: a cache token holds 2 * num_kv_heads = %d rows at least",
+                     v.cache_combined_heads, 2 * v.attn.num_kv_heads);
   if (fp8) {
     if (v.attn.dtype != RPA_DTYPE_BF16 || v.attn.compute != RPA_COMPUTE_BF16)
       return rpa::fail(RPA_ERR_UNSUPPORTED, "an 8-bit cache takes bf16 queries and RPA_COMPUTE_BF16");
@@ -333,7 +337,7 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (rc == RPA_ERR_UNSUPPORTED)
     return rpa::fail(rc, "head_dim=%d rows are not a multiple of 16 bytes", v.attn.head_dim);
   if (rc != RPA_OK) return rpa::fail(rc, "cache update launch failed: %s", hipGetErrorString(hipGetLastError()));
-  if (!fp8 && chd == v.attn.head_dim) return rpa_fwd_launch(&v.attn, hip_stream);
+  if (!fp8 && chd == v.attn.head_dim && chx2 == 2 * v.attn.num_kv_heads) return rpa_fwd_launch(&v.attn, hip_stream);
 
   // 8-bit elements or padded rows: the cache is addressed through its own strides (K row of head j at combined
   // head 2j, its V row at 2j + 1, chd elements each)
@@ -341,7 +345,7 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   rpa::KvLayout kv;
   kv.k_base = static_cast<const char*>(p.kv_pages);
   kv.v_base = kv.k_base + static_cast<size_t>(chd) * esize;
-  kv.stride_b = 2u * p.num_kv_heads * chd * esize;
+  kv.stride_b = static_cast<uint32_t>(chx2) * chd * esize;
   kv.page_b = static_cast<uint64_t>(p.page_size) * kv.stride_b;
   kv.head_b = 2u * chd * esize;
   kv.contiguous = 0;

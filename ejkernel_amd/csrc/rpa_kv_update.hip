@@ -10,7 +10,8 @@
 namespace rpa {
 
 __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const char* __restrict__ new_k,
-                                                              const char* __restrict__ new_v, int row_bytes, int dst_row_bytes) {
+                                                              const char* __restrict__ new_v, int row_bytes, int dst_row_bytes,
+                                                              int dst_heads) {
   const int t = blockIdx.x;
   int nseq = p.num_seqs[0];
   nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
@@ -23,7 +24,7 @@ __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const
   int page = p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + pos / p.page_size];
   page = page < 0 ? 0 : (page >= p.num_pages ? p.num_pages - 1 : page);
   const size_t tok = static_cast<size_t>(page) * p.page_size + pos % p.page_size;
-  char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * 2 * p.num_kv_heads * dst_row_bytes;
+  char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * dst_heads * dst_row_bytes;
   const size_t src_off = static_cast<size_t>(t) * p.num_kv_heads * row_bytes;
   const int pieces_per_row = row_bytes / 16, n = 2 * p.num_kv_heads * pieces_per_row;
   for (int k = threadIdx.x; k < n; k += blockDim.x) {
@@ -39,9 +40,10 @@ int launch_kv_cache_update(const RpaV3Params& v, hipStream_t stream) {
   const int esize = v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 1 : v.cache_dtype == RPA_DTYPE_BF16 ? 2 : 4;
   const int row_bytes = p.head_dim * esize;
   const int dst_row_bytes = (v.cache_head_dim > 0 ? v.cache_head_dim : p.head_dim) * esize;
-  if (row_bytes % 16 != 0 || dst_row_bytes % 16 != 0 || dst_row_bytes < row_bytes) return RPA_ERR_UNSUPPORTED;
+  const int dst_heads = v.cache_combined_heads > 0 ? v.cache_combined_heads : 2 * p.num_kv_heads;
+  if (row_bytes % 16 != 0 || dst_row_bytes % 16 != 0 || dst_row_bytes < row_bytes || dst_heads < 2 * p.num_kv_heads) return RPA_ERR_UNSUPPORTED;
   hipLaunchKernelGGL(kv_cache_update_kernel, dim3(p.total_tokens), dim3(256), 0, stream, p,
-                     static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes, dst_row_bytes);
+                     static_cast<const char*>(v.new_keys), static_cast<const char*>(v.new_values), row_bytes, dst_row_bytes, dst_heads);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 

@@ -13,7 +13,8 @@ head_dim that is a multiple of 128 and an even combined-head count, byte for byt
 ``[num_pages, page_size, 2 * num_kv_heads, head_dim]`` layout of the v2 operation.  A head_dim
 that is no multiple of 128 has its rows padded to one (``merge_kv``, ``_kernel.py:44-57``): the
 kernels then walk the cache with the row pitch of the padded rows and neither read nor write
-the padding.  A padded combined-head count is rejected here.
+the padding.  The same holds for a combined-head count padded to a multiple of the packing
+(an odd ``num_kv_heads`` under an 8-bit cache).
 
 ``distribution[-1]`` is the number of sequences (``_kernel.py:195``).
 
@@ -85,8 +86,8 @@ def _static_validate(q, k, v, kv_cache, kv_lens, block_tables, query_start_loc, 
     if logits_soft_cap is not None and logits_soft_cap == 0.0:
         raise ValueError("soft_cap != 0")
     # limits of this implementation
-    if hx2_per_pack * pack != 2 * hkv:
-        raise ValueError("a cache with padded combined heads is not supported")
+    if hx2_per_pack != -(-2 * hkv // pack):
+        raise ValueError("cache dim 2 must be cdiv(2 * num_kv_heads, packing)")
     if not (k.dtype == v.dtype == kv_cache.dtype):
         raise ValueError("keys, values and kv_cache must share one dtype")  # merge_kv asserts it, the update needs it
     if kv_cache.dtype in _FP8:
@@ -160,6 +161,8 @@ def _launch(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_
     v3.new_values = values.data_ptr()
     v3.cache_dtype = _FP8.get(kv_cache.dtype, p.dtype)
     v3.cache_head_dim = kv_cache.shape[4]
+    v3.cache_combined_heads = kv_cache.shape[2] * kv_cache.shape[3]
+    v3.reserved = 0
 
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream

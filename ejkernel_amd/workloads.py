@@ -80,7 +80,8 @@ def to_v3(batch: Batch, seed: int = 0, cache_dtype: torch.dtype | None = None) -
     """New K/V rows for every query token; the cache shares ``batch.kv_pages``' memory, viewed in five dimensions.
 
     The positions the new tokens will occupy hold random data beforehand, so a missed write shows in the output.
-    A head_dim that is no multiple of 128 gets a cache of its own with rows padded to one (random data in the padding).
+    A head_dim that is no multiple of 128, or a combined-head count that is no multiple of the packing, gets a cache of
+    its own with rows / heads padded to one (random data in the padding).
     With ``cache_dtype`` (an 8-bit float type) the cache is a copy of ``batch.kv_pages`` cast to it, and so are the new rows.
     """
     dev = batch.queries.device
@@ -96,13 +97,14 @@ def to_v3(batch: Batch, seed: int = 0, cache_dtype: torch.dtype | None = None) -
     S = int(batch.num_seqs.reshape(-1)[0])
     pages = batch.kv_pages if cdt == dtype else batch.kv_pages.to(cdt)
     dalign = -(-head_dim // 128) * 128
-    if dalign != head_dim:  # rows padded as merge_kv pads them; the padding holds random data that must not matter
-        padded = _randn_chunked((num_pages, page_size, hx2, dalign), gen, dev, dtype).to(cdt)
-        padded[..., :head_dim] = pages
+    hx2_pad = -(-hx2 // pack) * pack
+    if dalign != head_dim or hx2_pad != hx2:  # rows and combined heads padded as merge_kv pads them; the padding
+        padded = _randn_chunked((num_pages, page_size, hx2_pad, dalign), gen, dev, dtype).to(cdt)  # holds random data
+        padded[:, :, :hx2, :head_dim] = pages
         pages = padded
     return V3Batch(
         queries=batch.queries, keys=keys, values=values,
-        kv_cache=pages.view(num_pages, page_size, hx2 // pack, pack, dalign),
+        kv_cache=pages.view(num_pages, page_size, hx2_pad // pack, pack, dalign),
         kv_lens=batch.context_lens, block_tables=batch.block_tables.reshape(-1).contiguous(),
         query_start_loc=batch.query_start_loc,
         distribution=torch.tensor([0, 0, S], dtype=torch.int32, device=dev), base=batch)

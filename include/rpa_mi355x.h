@@ -129,6 +129,10 @@ typedef struct RpaV3Params {
                           /* for head_dim.  With padded rows (head_dim 64 in rows of 128) the cache is                 */
                           /* [num_pages, page_size, 2*num_kv_heads / packing, packing, cache_head_dim]; the padding    */
                           /* is neither read nor written.                                                               */
+  int32_t cache_combined_heads; /* combined K/V heads per cache token: 2*num_kv_heads rounded up to a multiple of the    */
+                          /* packing as merge_kv pads them (an odd num_kv_heads under an 8-bit cache), or 0 for         */
+                          /* 2*num_kv_heads.  The padding heads are neither read nor written.                           */
+  int32_t reserved;       /* 0 */
 } RpaV3Params;
 
 /* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */

@@ -111,6 +111,11 @@ def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
     p.workspace_bytes = plain
     p.head_dim = 520                                          # beyond the scalar kernel
     assert lib.rpa_v3_launch(ctypes.byref(v), None) == -2 and b"at most 512" in lib.rpa_last_error()
+    p.head_dim = 64
+    v.cache_head_dim = 32                                     # shorter than the rows it holds
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_head_dim" in lib.rpa_last_error()
+    v.cache_head_dim, v.cache_combined_heads = 128, 2         # fewer than 2 * num_kv_heads = 4
+    assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_combined_heads" in lib.rpa_last_error()
 
 
 def test_workspace_bytes_and_errors_without_gpu():

@@ -238,6 +238,23 @@ def test_bf16_random_batches_head_dim_64(seed):
             assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
 
 
+def test_8bit_cache_with_an_odd_number_of_kv_heads_pads_the_combined_heads():
+    """One kv head under packing 4: the cache holds four combined heads per token, K, V and two of padding (merge_kv
+    pads them); the update leaves the padding alone and the attention never reads it."""
+    f8 = torch.float8_e4m3fn
+    v = to_v3(make_batch([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], num_q_heads=8, num_kv_heads=1, head_dim=128,
+                         page_size=16, pages_per_seq=32, seed=3, device=DEV), seed=3, cache_dtype=f8)
+    assert tuple(v.kv_cache.shape[2:]) == (1, 4, 128)
+    before = v.kv_cache.clone()
+    ref_out, ref_cache = rpa_v3(*[to_np(a) for a in v.args()], cache_dtype="float8_e4m3fn", query_dtype="bfloat16",
+                                **v.kwargs())
+    out, cache = run_hip(v)
+    assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
+    assert torch.equal(cache[:, :, :, 2:].view(torch.uint8), before[:, :, :, 2:].view(torch.uint8)), "padding heads written"
+    assert not torch.equal(cache[:, :, :, :2].view(torch.uint8), before[:, :, :, :2].view(torch.uint8))
+    assert_bf16_parity(to_np(out), ref_out, 176, "8-bit cache, one kv head")
+
+
 # ---------------------------------------------------------------- 8-bit cache (float8_e4m3fn, bf16 queries)
 # The device follows the program's casts (Q / q_scale clipped and cast to the cache dtype, normalised probabilities
 # cast to the cache dtype), so against the restatement the only differences left are float32 evaluation order and
@@ -318,9 +335,7 @@ def test_e4m3_random_batches(seed):
     step of that probability times the value row: the restatement reports that allowance per row (zero nearly
     everywhere) and it is added to the bound.  Seeds 1123 and 1341 hold such a row (0.027 and 0.19 from the
     restatement in one (token, head) row each, every other row bit for bit)."""
-    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))
-    if b.meta["num_kv_heads"] % 2:
-        pytest.skip("an odd number of kv heads pads the packed cache: rejected")
+    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))   # an odd number of kv heads pads the packed cache
     rows = b.total_valid_tokens
     v = to_v3(b, seed=seed, cache_dtype=F8 if seed % 2 == 0 else torch.float8_e5m2)
     slack = np.zeros((v.queries.shape[0], v.queries.shape[1]), np.float32)
