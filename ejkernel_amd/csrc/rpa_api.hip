@@ -155,6 +155,7 @@ int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream)
   kv.head_b = static_cast<uint32_t>(p.page_size) * kv.stride_b;
   kv.page_b = static_cast<uint64_t>(p.num_kv_heads) * kv.head_b;
   kv.contiguous = 0;
+  kv.capacity = rpa::paged_capacity(p);
   if (static_cast<uint64_t>(p.page_size) * p.head_dim * esize > 0xffffffffull)
     return rpa::fail(RPA_ERR_UNSUPPORTED, "a cache block of one head exceeds 4 GiB");
   return rpa::dispatch(p, kv, page_attention_tiled(p), static_cast<hipStream_t>(hip_stream));
@@ -230,6 +231,7 @@ int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stre
   kv.stride_b = static_cast<uint32_t>(p.num_kv_heads) * kv.head_b;
   kv.page_b = static_cast<uint64_t>(params->seq_len) * kv.stride_b;
   kv.contiguous = 1;
+  kv.capacity = params->seq_len;
   hipStream_t stream = static_cast<hipStream_t>(hip_stream);
   const bool tiled = page_attention_tiled(p);
   if (params->num_sinks == 0) return rpa::dispatch(p, kv, tiled, stream);
@@ -349,6 +351,7 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   kv.page_b = static_cast<uint64_t>(p.page_size) * kv.stride_b;
   kv.head_b = 2u * chd * esize;
   kv.contiguous = 0;
+  kv.capacity = rpa::paged_capacity(p);
   if (!fp8) return rpa::dispatch(p, kv, rpa::tiled_supported(p), stream);
   const uint64_t base = (rpa_workspace_bytes(&p) + 255) & ~255ull;
   float* stats = reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base);

@@ -151,7 +151,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   // are counted apart from the vector loads of the K/V stream.  The block table is never written by this kernel.
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(reinterpret_cast<uintptr_t>(bt));
   const int t_last = range_hi - 1;
-  const float cap = p.logits_soft_cap;
+  // the reference's cap is a weakly typed scalar: it takes the logits' dtype (bf16) before it divides and multiplies
+  const float cap = kMimic ? rbf(p.logits_soft_cap) : p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
 
   using raw_t = typename std::conditional<kKv != 0, u32x2_t, u32x4_t>::type;  // one lane's piece: eight elements
@@ -364,9 +365,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 
   if (part.partial) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
-    // Partials are written and read with agent-scope relaxed atomics (write-through / cache-bypassing accesses),
-    // so no L2 write-back or invalidate is needed around the ticket: it is enough that this wave's stores have
-    // completed (the workgroup-scope release waits for them) before the ticket is taken.
+    // Who writes, who reads: this wavefront writes its slot; the wavefront that draws the last ticket of the
+    // (sequence, kv head) -- any workgroup, usually on another XCD with another L2 -- reads every slot.  Partials are
+    // written and read with agent-scope relaxed atomics, i.e. write-through stores and cache-bypassing loads that
+    // meet in memory-side storage, so no L2 write-back or invalidate is needed around the ticket.  What the hand-off
+    // needs is order: every store of this wavefront must have completed before its ticket increment can be seen.
+    // The explicit s_waitcnt vmcnt(0) below provides that (on gfx9 stores count in vmcnt, and a store leaves the
+    // counter when it has been acknowledged by the level its scope bits write through to); the fences beside it only
+    // keep the compiler from moving memory operations across.  The reader orders itself by data dependence: its
+    // loads are issued after the ticket value has come back and been compared.
     const size_t slot = static_cast<size_t>(part.slot);
     if (row_valid) {
       uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
@@ -388,6 +395,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       }
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     uint32_t* ctr = a.counters + static_cast<size_t>(s) * p.num_kv_heads + j;
     uint32_t ticket = 0;
     if (lane == 0) ticket = __hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

@@ -75,4 +75,25 @@ __device__ __forceinline__ int seq_of_row(const RpaParams& p, int nseq, int row)
   return p.query_start_loc != nullptr ? find_seq(p.query_start_loc, nseq, row) : row;
 }
 
+// Query rows and key count of sequence s as every kernel uses them: clipped to what the buffers hold, so that
+// malformed device metadata can neither read nor write out of bounds.  Row ranges are clipped to
+// [0, total_tokens] (a start above its end gives an empty sequence) and the key count to [0, kv_capacity], the
+// tokens one sequence's block-table row (or contiguous cache) can address.  The reference's XLA program is safe on
+// such input because XLA clamps every dynamic index; its Pallas path rejects it up front
+// (ejkernel/kernels/_pallas/tpu/ragged_page_attention/_pallas_impl_fwd.py:124-174: q_len <= kv_len,
+// pages_per_seq >= ceil(kv_len / page), cu_q_lens[num_seqs] <= total tokens).
+struct SeqMeta {
+  int q0, q_len, kv_len;
+};
+__device__ __forceinline__ int clip_row(const RpaParams& p, int r) { return min(max(r, 0), p.total_tokens); }
+__device__ __forceinline__ SeqMeta seq_meta(const RpaParams& p, int kv_capacity, int s) {
+  SeqMeta m;
+  m.q0 = clip_row(p, q_start_of(p, s));
+  m.q_len = max(clip_row(p, q_start_of(p, s + 1)) - m.q0, 0);
+  m.kv_len = min(max(p.context_lens[s], 0), kv_capacity);
+  return m;
+}
+// Rows of the ragged batch (rows from here on are written as zeros).
+__device__ __forceinline__ int batch_rows(const RpaParams& p, int nseq) { return clip_row(p, q_start_of(p, nseq)); }
+
 }  // namespace rpa

@@ -26,16 +26,18 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
   T* __restrict__ out = static_cast<T*>(p.out);
 
   const int nseq = seq_count(p);
-  const int total = q_start_of(p, nseq);
+  const int total = batch_rows(p, nseq);
   const size_t row_base = (static_cast<size_t>(row) * p.num_q_heads + static_cast<size_t>(j) * G) * D;
-  if (row >= total) {  // rows past the ragged batch are defined as zero
+  const int s = row < total ? seq_of_row(p, nseq, row) : 0;
+  const SeqMeta sm = seq_meta(p, kvl.capacity, row < total ? s : 0);
+  // rows past the ragged batch are defined as zero (so are rows that malformed row offsets leave without a sequence)
+  if (row >= total || row < sm.q0 || row >= sm.q0 + sm.q_len) {
     for (int i = lane; i < G * D; i += kWave) Elem<T>::store(out + row_base + i, 0.f);
     return;
   }
-  const int s = seq_of_row(p, nseq, row);
-  const int q_len = q_start_of(p, s + 1) - q_start_of(p, s);
-  const int kv_len = p.context_lens[s];
-  const int pos = kv_len - q_len + (row - q_start_of(p, s));
+  const int q_len = sm.q_len;
+  const int kv_len = sm.kv_len;
+  const int pos = kv_len - q_len + (row - sm.q0);
   const int hi = min(pos + 1, kv_len);
   const int lo = max(p.sliding_window > 0 ? max(0, pos - p.sliding_window + 1) : 0, kv_start_of(p, s));
 
@@ -47,7 +49,8 @@ __global__ __launch_bounds__(kWave) void rpa_generic_kernel(RpaParams p, KvLayou
   const float scale = t_is_bf16 ? round_bf16(p.softmax_scale) : p.softmax_scale;
   const float post = p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f);
   const float o_scale = p.v_scale > 0.f ? p.v_scale : 1.f;
-  const float cap = p.logits_soft_cap;
+  // the reference's cap is a weakly typed scalar: it takes the logits' dtype before it divides and multiplies
+  const float cap = kBf16Compute && !v3 ? round_bf16(p.logits_soft_cap) : p.logits_soft_cap;
   const int32_t* __restrict__ bt = p.block_tables + static_cast<size_t>(s) * p.pages_per_seq;
 
   for (int g = 0; g < G; ++g) {

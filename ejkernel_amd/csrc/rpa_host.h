@@ -16,7 +16,12 @@ struct KvLayout {
   uint32_t stride_b;  // between the tokens of a page
   uint32_t head_b;    // between the kv heads of a token
   int32_t contiguous; // 1: no block table, sequence s is page s (page_b = bytes between sequences, slot = position)
+  int32_t capacity;   // tokens one sequence can address: pages_per_seq * page_size, or the contiguous cache's seq_len
 };
+__host__ __device__ inline int32_t paged_capacity(const RpaParams& p) {
+  const int64_t c = static_cast<int64_t>(p.pages_per_seq) * p.page_size;
+  return c > 0x7fffffff ? 0x7fffffff : static_cast<int32_t>(c);
+}
 inline KvLayout interleaved_layout(const RpaParams& p) {
   const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
   KvLayout l;
@@ -26,6 +31,7 @@ inline KvLayout interleaved_layout(const RpaParams& p) {
   l.page_b = static_cast<uint64_t>(p.page_size) * l.stride_b;
   l.head_b = 2u * p.head_dim * esize;
   l.contiguous = 0;
+  l.capacity = paged_capacity(p);
   return l;
 }
 

@@ -1,4 +1,5 @@
-// Cache update of ragged_page_attention_v3 (rows of the cache may be longer than head_dim: the padding stays as it is): token t of sequence s (t in [q_start, q_start + q_len)) is the key /
+// Cache update of ragged_page_attention_v3 (rows of the cache may be longer than head_dim: the padding of an updated
+// token is zeroed, as the reference's scatter of merge_kv's zero-padded rows does): token t of sequence s (t in [q_start, q_start + q_len)) is the key /
 // value at position kv_len - q_len + (t - q_start) of that sequence, and its rows go to
 // cache[block_tables[s, pos / page], pos % page, 2j | 2j + 1, :] for every kv head j
 // (ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:44-57 merge_kv, :207-218 update).
@@ -15,22 +16,26 @@ __global__ __launch_bounds__(256) void kv_cache_update_kernel(RpaParams p, const
   const int t = blockIdx.x;
   int nseq = p.num_seqs[0];
   nseq = nseq < 0 ? 0 : (nseq > p.max_num_seqs ? p.max_num_seqs : nseq);
-  if (t >= p.query_start_loc[nseq]) return;
+  if (t >= batch_rows(p, nseq)) return;
   const int s = find_seq(p.query_start_loc, nseq, t);
-  const int q0 = p.query_start_loc[s], q_len = p.query_start_loc[s + 1] - q0;
-  const int kv_len = p.context_lens[s];
-  const int pos = kv_len - q_len + (t - q0);
-  if (pos < 0 || pos >= kv_len || pos >= p.pages_per_seq * p.page_size) return;
+  const SeqMeta sm = seq_meta(p, paged_capacity(p), s);
+  if (t < sm.q0 || t >= sm.q0 + sm.q_len) return;
+  const int pos = sm.kv_len - sm.q_len + (t - sm.q0);
+  if (pos < 0 || pos >= sm.kv_len) return;
   int page = p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + pos / p.page_size];
   page = page < 0 ? 0 : (page >= p.num_pages ? p.num_pages - 1 : page);
   const size_t tok = static_cast<size_t>(page) * p.page_size + pos % p.page_size;
   char* dst = static_cast<char*>(const_cast<void*>(p.kv_pages)) + tok * dst_heads * dst_row_bytes;
   const size_t src_off = static_cast<size_t>(t) * p.num_kv_heads * row_bytes;
-  const int pieces_per_row = row_bytes / 16, n = 2 * p.num_kv_heads * pieces_per_row;
+  // The whole token record is written: the new K / V rows, and zeros in what merge_kv pads them with (row tails
+  // beyond head_dim, combined heads beyond 2 * num_kv_heads) -- the reference scatters the padded rows.
+  const int pieces_per_row = row_bytes / 16, dst_pieces = dst_row_bytes / 16, n = dst_heads * dst_pieces;
   for (int k = threadIdx.x; k < n; k += blockDim.x) {
-    const int row = k / pieces_per_row, piece = k - row * pieces_per_row;  // row = combined head 2j (K) or 2j + 1 (V)
-    const char* src = ((row & 1) ? new_v : new_k) + src_off + static_cast<size_t>(row >> 1) * row_bytes + 16 * piece;
-    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(row) * dst_row_bytes + 16 * piece) = *reinterpret_cast<const uint4*>(src);
+    const int row = k / dst_pieces, piece = k - row * dst_pieces;  // row = combined head 2j (K) or 2j + 1 (V)
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (row < 2 * p.num_kv_heads && piece < pieces_per_row)
+      v = *reinterpret_cast<const uint4*>(((row & 1) ? new_v : new_k) + src_off + static_cast<size_t>(row >> 1) * row_bytes + 16 * piece);
+    *reinterpret_cast<uint4*>(dst + static_cast<size_t>(row) * dst_row_bytes + 16 * piece) = v;
   }
 }
 

@@ -76,7 +76,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
   const char* kvb = static_cast<const char*>(p.kv_pages);
-  const float cap = p.logits_soft_cap;
+  // the reference's cap is a weakly typed scalar: it takes the logits' dtype (bf16) before it divides and multiplies
+  const float cap = kMimic ? rbf(p.logits_soft_cap) : p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
   const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
   // (A head_dim below the instantiation's runs too: q is padded with zeros and the upper part of every K / V row in

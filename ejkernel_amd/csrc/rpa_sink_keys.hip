@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kSinkWgWaves * kWave) void sink_keys_kernel(RpaPara
   const T* __restrict__ q = static_cast<const T*>(p.queries);
   const bool t_is_bf16 = sizeof(T) == 2;
   const float scale = t_is_bf16 ? round_bf16(p.softmax_scale) : p.softmax_scale;
-  const float cap = p.logits_soft_cap;
+  const float cap = kBf16Compute ? round_bf16(p.logits_soft_cap) : p.logits_soft_cap;  // weakly typed scalar: the logits' dtype first
   const int start = kv_start_of(p, s);
   if (h == 0 && lane == 0) sk.main_start[s] = start + sk.num_sinks;
   const int n_keys = max(0, min(sk.num_sinks, sk.seq_len - start));

@@ -88,7 +88,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   int my_items = 0, my_tiles = 0, my_wg = 0;
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
-    classify(seq_info<C::TT>(p, s, G), t, it, wg);
+    classify(seq_info<C::TT>(a, s, G), t, it, wg);
     my_tiles += t;
     my_items += it;
     my_wg += wg;
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
   int wg_base = block_excl_scan(my_wg, scratch, total_wg);
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
-    classify(seq_info<C::TT>(p, s, G), t, it, wg);
+    classify(seq_info<C::TT>(a, s, G), t, it, wg);
     if ((s & (K - 1)) == 0) {
       item_start[s >> shift] = item_base;
       tile_start[s >> shift] = tile_base;
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       int mine = 0;
       for (int s = s_begin; s < s_end; ++s) {
         int t, it, wg;
-        classify(seq_info<C::TT>(p, s, G), t, it, wg);
+        classify(seq_info<C::TT>(a, s, G), t, it, wg);
         mine += wg > 0;
       }
       int n_pf;
@@ -143,7 +143,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         int* o_cnt = t_cnt + kSortMax;
         for (int s = s_begin; s < s_end; ++s) {
           int t, it, wg;
-          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const SeqInfo si = seq_info<C::TT>(a, s, G);
           classify(si, t, it, wg);
           if (wg > 0) {
             t_seq[at] = s;
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 
   // ---- rows past the ragged batch are zero
   {
-    const int total_rows = q_start_of(p, nseq);
+    const int total_rows = batch_rows(p, nseq);
     const int row_u4 = p.num_q_heads * p.head_dim / 8;  // 16-byte pieces per row
     u32x4_t* o4 = static_cast<u32x4_t*>(p.out);
     for (int row = total_rows + blockIdx.x; row < p.total_tokens; row += gridDim.x)
@@ -204,7 +204,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       const int s_last = min(s + K, nseq) - 1;
       for (; s < s_last; ++s) {
         int t, it, wg;
-        classify(seq_info<C::TT>(p, s, G), t, it, wg);
+        classify(seq_info<C::TT>(a, s, G), t, it, wg);
         const int cnt = __builtin_amdgcn_readfirstlane(kind == 0 ? it : kind == 1 ? t : wg);
         if (x < b + cnt) break;
         b += cnt;
@@ -284,7 +284,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           } else {
             s = find(wg_start, 2, w, s_base);
           }
-          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const SeqInfo si = seq_info<C::TT>(a, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
           const int local = w - s_base;
           const int j = local / n_qt, member = local - j * n_qt;
@@ -304,7 +304,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         for (int w = vwg; w < total_wg; w += gridDim.x) {
           int base;
           const int s = find(wg_start, 2, w, base);
-          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const SeqInfo si = seq_info<C::TT>(a, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
           const int local = w - base;
           const int j = local / n_qt, member = local - j * n_qt;
@@ -322,7 +322,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
       for (int w = worker; w < total_items; w += n_workers) {
         int s_base;
         const int s = find(item_start, 0, w, s_base);
-        const SeqInfo si = seq_info<C::TT>(p, s, G);
+        const SeqInfo si = seq_info<C::TT>(a, s, G);
         const int local = w - s_base;
         const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
         const int row_hi = min(rt * 16 + 16, si.rows);
@@ -364,7 +364,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
         while (x < x_end) {
           int s_base;
           const int s = find(tile_start, 1, x, s_base);
-          const SeqInfo si = seq_info<C::TT>(p, s, G);
+          const SeqInfo si = seq_info<C::TT>(a, s, G);
           const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
           const int local = x - s_base;
           const int j = local / per_head, t0 = local - j * per_head;
@@ -386,18 +386,42 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
 
 // ----------------------------------------------------------------------------- host side
 
-static int env_int(const char* name, int dflt) {
-  const char* v = getenv(name);
-  return v && *v ? atoi(v) : dflt;
+// Experiment knobs (RPA_TUNE_* environment variables), read once per process on the first launch: a launch costs
+// no getenv calls, and a setenv in another host thread cannot race with one.
+struct Tune {
+  int wgs_per_cu;          // RPA_TUNE_WGS_PER_CU: workgroups of the persistent grid per compute unit (1..kTiledMaxWgsPerCu)
+  int decode_wgs_per_cu;   // RPA_TUNE_DECODE_WGS_PER_CU: of these, how many stream a batch without prefill tiles (0 = rule)
+  int min_share_tiles;     // RPA_TUNE_MIN_SHARE_TILES
+  int phase_mode;          // RPA_TUNE_PHASE_MODE
+  int even_xcd_permille;   // RPA_TUNE_EVEN_XCD_PERMILLE
+  int no_mimic;            // RPA_TUNE_NO_MIMIC
+  int no_wave_only;        // RPA_TUNE_NO_WAVE_ONLY
+  int wave_only_rows;      // RPA_TUNE_WAVE_ONLY_ROWS
+};
+static const Tune& tune() {
+  static const Tune t = [] {
+    auto env_int = [](const char* name, int dflt) {
+      const char* v = getenv(name);
+      return v && *v ? atoi(v) : dflt;
+    };
+    Tune x;
+    x.wgs_per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 2)));
+    x.decode_wgs_per_cu = max(0, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 0));
+    x.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
+    x.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
+    x.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
+    x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
+    x.no_wave_only = env_int("RPA_TUNE_NO_WAVE_ONLY", 0);
+    x.wave_only_rows = env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows);
+    return x;
+  }();
+  return t;
 }
 
 // Workgroups of the persistent grid: two per compute unit (two wavefronts per SIMD, so one wavefront's LDS and
 // softmax latency hides behind the other's MFMAs in prefill tiles); the decode stream alone is ~3 % faster with
-// one.  RPA_TUNE_WGS_PER_CU overrides it for experiments (1..kTiledMaxWgsPerCu).
-static int tiled_grid() {
-  const int per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 2)));
-  return device_cu_count() * per_cu;
-}
+// one.
+static int tiled_grid() { return device_cu_count() * tune().wgs_per_cu; }
 
 bool tiled_supported(const RpaParams& p) {
   if (p.flags & RPA_FLAG_FORCE_GENERIC) return false;
@@ -453,15 +477,15 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.pre = pre;
   a.stats = stats;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
-  a.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
+  a.min_share_tiles = tune().min_share_tiles;
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
-  a.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
-  a.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
+  a.phase_mode = tune().phase_mode;
+  a.even_xcd_permille = tune().even_xcd_permille;
   // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
   // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes
   // in flight.
-  a.stream_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", p.head_dim == 64 ? 2 : 1));
+  a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : p.head_dim == 64 ? 2 : 1);
   a.decode_grid = device_cu_count();
   char* ws = static_cast<char*>(p.workspace);
   a.counters = reinterpret_cast<uint32_t*>(ws);
@@ -472,7 +496,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities; both launches run
     // every sequence through the wave-level loop.  A wavefront has half the bytes in flight that it has with a
     // 16-bit cache, so both workgroups of a compute unit stream (0.70 ms against 0.84 ms on 256 x 512..8192 keys).
-    a.stream_grid = device_cu_count() * max(1, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 2));
+    a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
     int rc;
     if (kv_elem == 2) {
       rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)
@@ -487,20 +511,20 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
                              : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
   }
-  const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && env_int("RPA_TUNE_NO_MIMIC", 0) == 0;
+  const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && tune().no_mimic == 0;
   // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
   // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
   // alone gets a register allocation without spills, and short prefill chunks spread over four times as many
   // wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
   const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
   const bool small_batch = p.query_start_loc == nullptr || ((p.flags & RPA_FLAG_PREFILL_TILES) == 0 &&
-                                                            rows <= env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows));
+                                                            rows <= tune().wave_only_rows);
   // Prefill tiles address the cache as [page][slot][2 * kv heads][head_dim]; any other layout (two caches, one
   // contiguous cache per sequence, rows padded beyond head_dim) runs through the wave-level loop alone.
   const KvLayout canon = interleaved_layout(p);
   const bool canonical = kv.k_base == canon.k_base && kv.v_base == canon.v_base && kv.stride_b == canon.stride_b &&
                          kv.head_b == canon.head_b && kv.page_b == canon.page_b && kv.contiguous == 0;
-  const bool wave_only = pre.ml != nullptr || !canonical || (small_batch && env_int("RPA_TUNE_NO_WAVE_ONLY", 0) == 0);
+  const bool wave_only = pre.ml != nullptr || !canonical || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);

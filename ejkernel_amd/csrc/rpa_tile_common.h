@@ -102,19 +102,21 @@ struct SeqInfo {
 };
 
 template <int TT>
-__device__ __forceinline__ SeqInfo seq_info(const RpaParams& p, int s, int G) {
+__device__ __forceinline__ SeqInfo seq_info(const TileArgs& a, int s, int G) {
+  const RpaParams& p = a.p;
   SeqInfo si;
-  si.q0 = q_start_of(p, s);
-  si.q_len = q_start_of(p, s + 1) - si.q0;
-  si.kv_len = p.context_lens[s];
-  si.rows = si.q_len > 0 ? si.q_len * G : 0;
+  const SeqMeta sm = seq_meta(p, a.kv.capacity, s);
+  si.q0 = sm.q0;
+  si.q_len = sm.q_len;
+  si.kv_len = sm.kv_len;
+  si.rows = si.q_len * G;
   si.n_rt = (si.rows + 15) >> 4;
   const int pos_min = si.kv_len - si.q_len;
   si.start = kv_start_of(p, s);
   int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
   lo = max(lo, si.start);
   si.lo_al = lo & ~(TT - 1);
-  si.hi = max(si.kv_len, 0);
+  si.hi = si.kv_len;
   si.eligible = si.n_rt == 1 && si.hi > si.lo_al;  // a sequence without keys stays an item: its rows become zero
   return si;
 }

@@ -141,7 +141,7 @@ def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tens
 
 def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *, softmax_scale,
             logits_soft_cap, compute_dtype, sliding_window, softmax_aux, cfg, flags: int = 0,
-            kv_start=None) -> torch.Tensor:
+            kv_start=None, out=None) -> torch.Tensor:
     lib = _native.load()
     if not queries.is_cuda:
         raise RuntimeError(
@@ -176,7 +176,10 @@ def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_
     if softmax_aux is not None:
         sinks = _sinks_per_q_head(softmax_aux.to(dev), num_q_heads, num_kv_heads)
 
-    out = torch.empty_like(queries)
+    if out is None:
+        out = torch.empty_like(queries)
+    elif out.shape != queries.shape or out.dtype != queries.dtype or out.device != dev or not out.is_contiguous():
+        raise ValueError("out must be a contiguous tensor of the shape, dtype and device of queries")
     p = _native.RpaParams()
     p.queries = queries.data_ptr()
     p.kv_pages = kv_pages.data_ptr()
@@ -252,6 +255,7 @@ class RaggedPageAttention:
         cfg: RaggedPageAttentionConfig,
         _flags: int = 0,
         _kv_start=None,
+        _out=None,
     ):
         """Same parameters as the reference's ``run`` (``:225-318``).
 
@@ -268,7 +272,7 @@ class RaggedPageAttention:
         return _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs,
                        softmax_scale=softmax_scale, logits_soft_cap=logits_soft_cap, compute_dtype=compute_dtype,
                        sliding_window=sliding_window, softmax_aux=softmax_aux, cfg=cfg, flags=_flags,
-                       kv_start=_kv_start)
+                       kv_start=_kv_start, out=_out)
 
     def heuristic_cfg(self, inv=None) -> RaggedPageAttentionConfig:
         """Default configuration (``:320-337``)."""

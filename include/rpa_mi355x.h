@@ -128,10 +128,11 @@ typedef struct RpaV3Params {
   int32_t cache_head_dim; /* elements per cache row: align_to(head_dim, 128) as merge_kv pads it (_kernel.py:44-57), or 0  */
                           /* for head_dim.  With padded rows (head_dim 64 in rows of 128) the cache is                 */
                           /* [num_pages, page_size, 2*num_kv_heads / packing, packing, cache_head_dim]; the padding    */
-                          /* is neither read nor written.                                                               */
+                          /* is never read, and zeroed in the token records the update writes (the reference scatters  */
+                          /* merge_kv's zero-padded rows).                                                              */
   int32_t cache_combined_heads; /* combined K/V heads per cache token: 2*num_kv_heads rounded up to a multiple of the    */
                           /* packing as merge_kv pads them (an odd num_kv_heads under an 8-bit cache), or 0 for         */
-                          /* 2*num_kv_heads.  The padding heads are neither read nor written.                           */
+                          /* 2*num_kv_heads.  The padding heads are never read, and zeroed in the records the update writes. */
   int32_t reserved;       /* 0 */
 } RpaV3Params;
 

@@ -118,7 +118,7 @@ def ragged_decode_strict(query, key, value, sequence_start, sequence_end, softma
                 mb = mask[sl][None, None, :]
                 sc = R(np.einsum("jgd,jkd->jgk", qs, kb, dtype=np.float32))
                 if logits_soft_cap is not None:
-                    cap = np.float32(logits_soft_cap)
+                    cap = R(np.float32(logits_soft_cap))  # weakly typed scalar: the array's dtype first
                     sc = R(R(np.tanh(R(sc / cap))) * cap)
                 if aux is not None:
                     sc = Rm(sc + _bias(aux, np.arange(i * block_size, (i + 1) * block_size))[None, :, :])

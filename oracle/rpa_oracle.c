@@ -148,7 +148,10 @@ static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, 
       for (int k = 0; k < kv_tok; ++k) {
         const int k_pos = kbi * kv_tok + k;
         float x = rb(srow[k], bf);
-        if (a->cap != 0.f) x = rb(rb(tanhf(rb(x / a->cap, bf)), bf) * a->cap, bf); /* :125-126 */
+        if (a->cap != 0.f) { /* :125-126; the Python scalar is weakly typed: it takes the array's dtype first */
+          const float capc = rb(a->cap, bf);
+          x = rb(rb(tanhf(rb(x / capc, bf)), bf) * capc, bf);
+        }
         const int keep = q_pos >= k_pos && k_pos < kv_len && (a->window <= 0 || k_pos > q_pos - a->window);
         x = keep ? x : -INFINITY; /* :138 */
         srow[k] = x;
@@ -192,7 +195,8 @@ static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, 
         const float floor_ = rb(1e-6f, bf);
         den = den > floor_ ? den : floor_;
       } else {
-        den = l[r] > 1e-6f ? l[r] : 1e-6f; /* :174 */
+        const float floor_ = rb(1e-6f, bf); /* :174, the weakly typed 1e-6 in the carry's dtype */
+        den = l[r] > floor_ ? l[r] : floor_;
         if (l[r] != l[r]) den = l[r];
       }
       const size_t dst = ((size_t)row * a->Hq + h) * D;

@@ -193,7 +193,8 @@ def rpa_strict(
 
     kv_tok = page_size * kvblocks
     base_k = np.arange(kv_tok, dtype=np.int64)
-    cap = None if logits_soft_cap is None else np.float32(logits_soft_cap)
+    # a Python scalar is weakly typed: XLA converts it to the array's dtype before the op (cap 23.7 is 23.75 in bf16)
+    cap = None if logits_soft_cap is None else Rc(np.float32(logits_soft_cap))
     neg_inf = np.float32(-np.inf)
 
     with np.errstate(invalid="ignore", over="ignore", divide="ignore"):
@@ -259,7 +260,7 @@ def rpa_strict(
                     denom = np.maximum(denom, Rc(np.float32(1e-6)))
                     res = Rc(Rc(e_m[..., None] * o) / denom[..., None])
                 else:  # :173-177
-                    l = np.maximum(l, np.float32(1e-6))
+                    l = np.maximum(l, Rc(np.float32(1e-6)))
                     res = Rc(o / l[..., None])
                 res = Rq(res)  # :179
                 out[r0 : r0 + qblocks] = res  # dynamic_update_slice clamps the same way :181-185

@@ -212,6 +212,7 @@ def rpa_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_l
             if pos < 0 or pos >= min(kv_len, pps * page):
                 continue
             pg = int(bt[s * pps + pos // page])
+            cache_rows[pg, pos % page] = 0.0  # merge_kv's padding (row tails, combined heads past 2 Hkv) is scattered too
             cache_rows[pg, pos % page, 0:2 * Hkv:2, :D] = keys[q_start + t]
             cache_rows[pg, pos % page, 1:2 * Hkv:2, :D] = values[q_start + t]
     # 2. attention on the updated cache

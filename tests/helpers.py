@@ -116,3 +116,23 @@ def random_rpa_batch(seed, device, head_dims=(64, 128, 256)):
     b = make_batch(q_lens, kv_lens, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, page_size=page, pages_per_seq=pps,
                    seed=seed, device=device, sliding_window=window, logits_soft_cap=cap, max_num_seqs=n + extra)
     return b, f"seed {seed}: {hq}/{hkv} D={D} page={page} q={q_lens} kv={kv_lens} W={window} cap={cap}"
+
+
+def two_key_cap_batch(device="cpu", head_dim=16, dtype=torch.bfloat16):
+    """One query row over two keys with the soft cap 23.7, which bf16 does not hold (the weakly typed scalar becomes
+    23.75 before it divides and multiplies, _xla_impl_fwd.py:125-126).  q . k is 20 for key 0 and 16 for key 1
+    (scale 1), V is 0 and 8.  By hand, every op rounded to bf16: 20 / 23.75 -> 0.84375, tanh -> 0.6875, * 23.75 ->
+    16.375; 16 / 23.75 -> 0.671875, tanh -> 0.5859375, * 23.75 -> 13.9375; p1 = bf16(exp(-2.4375)) = 0.08740234375,
+    l = bf16(1.08740234375) = 1.0859375, o = 8 p1 = 0.69921875, out = bf16(o / l) = 0.64453125.  With the cap left at
+    23.7 the two logits become 16.25 and 13.875 and the output 0.6796875; a device that normalises with the fp32 row sum
+    (1.08740234375) lands on 0.64453125 as well."""
+    b = make_batch([1], [2], num_q_heads=1, num_kv_heads=1, head_dim=head_dim, page_size=4, pages_per_seq=1, seed=0,
+                   dtype=dtype, device=device, logits_soft_cap=23.7, softmax_scale=1.0)
+    pg = int(b.block_tables[0, 0])
+    b.queries.zero_()
+    b.queries[0, 0, 0] = 4.0
+    b.kv_pages[pg].zero_()
+    b.kv_pages[pg, 0, 0, 0] = 5.0   # K of key 0
+    b.kv_pages[pg, 1, 0, 0] = 4.0   # K of key 1
+    b.kv_pages[pg, 1, 1, :] = 8.0   # V of key 1 (V of key 0 is zero)
+    return b, 0.64453125

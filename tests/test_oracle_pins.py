@@ -117,6 +117,17 @@ def test_two_key_soft_cap_closed_form():
     np.testing.assert_allclose(run_strict(b, compute_dtype="float32")[0, 0], want, rtol=2e-6, atol=2e-6)
 
 
+def test_cap_that_bf16_does_not_hold_is_rounded_before_use():
+    """The cap is a weakly typed scalar: in a bf16 program it is 23.75, not 23.7 (closed form worked out by hand in
+    two_key_cap_batch; with 23.7 the output would be 0.6796875)."""
+    from tests.helpers import two_key_cap_batch
+
+    b, want = two_key_cap_batch()
+    assert np.all(run_strict(b)[0, 0] == np.float32(want))
+    assert np.all(_c_strict(b)[0, 0] == np.float32(want))
+    assert abs(run_exact(b)[0, 0, 0] - 8 / (1 + math.exp(23.7 * (math.tanh(20 / 23.7) - math.tanh(16 / 23.7))))) < 1e-12
+
+
 def test_one_key_one_sink_closed_form():
     b = _batch([1], [1], num_q_heads=2, num_kv_heads=1, head_dim=4, pages_per_seq=1, softmax_scale=0.5)
     sink = np.float32([[0.3], [-1.2]])  # per q head

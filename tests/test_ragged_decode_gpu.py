@@ -64,6 +64,33 @@ def test_bf16_starts_windows_and_caps_against_float64(flags, window, cap):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+def test_sequence_end_beyond_the_cache_is_clipped(flags):
+    """sequence_end > seq_len must not read the next sequence's keys (or past the buffers for the last sequence): the
+    reference masks with arange(seq_len) (_xla_impl_fwd.py:50-55), so such an end acts as seq_len; the device clips it.
+    Without a window the two agree on every row."""
+    ends = [300, 64, 320, 17, 200]
+    b = small([0, 5, 100, 0, 7], ends)
+    want = run_hip(b, flags)
+    big_k = torch.zeros((len(ends) + 2, *b.key.shape[1:]), dtype=b.key.dtype, device=DEV)
+    big_v = torch.zeros_like(big_k)
+    big_k[:len(ends)], big_v[:len(ends)] = b.key, b.value
+    big_k[len(ends):] = float("nan")  # what a read past the last sequence would see
+    big_v[len(ends):] = float("nan")
+    end_bad = b.sequence_end.clone()
+    end_bad[2] = 320 + 5000           # already the whole cache: nothing changes
+    end_bad[4] = 2 ** 30              # the last sequence: acts as seq_len = 320
+    out = ragged_decode_attention(b.query, big_k[:len(ends)], big_v[:len(ends)], b.sequence_start, end_bad,
+                                  softmax_scale=b.softmax_scale, _flags=flags)
+    torch.cuda.synchronize()
+    out = to_np(out)
+    assert np.isfinite(out).all()
+    assert np.array_equal(out[:4], want[:4])
+    ref = ragged_decode_exact(to_np(b.query), to_np(b.key), to_np(b.value), to_np(b.sequence_start),
+                              np.array([300, 64, 320, 17, 320], np.int32), softmax_scale=b.softmax_scale)
+    assert_bf16_parity(out, ref, len(ends), "clipped sequence_end")
+
+
+@pytest.mark.parametrize("flags", PATHS)
 def test_float32_against_float64(flags):
     b = small([0, 5, 100, 0], [300, 64, 101, 17], dtype=torch.float32)
     ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=(150, 0))

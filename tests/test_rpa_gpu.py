@@ -13,7 +13,7 @@ from ejkernel_amd import _native
 from ejkernel_amd.modules import RaggedPageAttention, RaggedPageAttentionConfig, ragged_page_attention
 from ejkernel_amd.workloads import Batch, compact_for_host, make_batch, make_workload
 from tests.helpers import (F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, random_rpa_batch,
-                           run_exact, run_strict, to_np)
+                           run_exact, run_strict, to_np, two_key_cap_batch)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -319,6 +319,60 @@ def test_bf16_random_batches(seed):
         mx, mean = err_stats(out, exact, rows)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
         assert not out[rows:].any()
+
+
+@pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("D", [16, 128])
+def test_cap_that_bf16_does_not_hold_is_rounded_before_use(flags, D):
+    """logits_soft_cap = 23.7 acts as 23.75 in the bf16 program (closed form in tests.helpers.two_key_cap_batch; with
+    23.7 unrounded the result would be 0.6796875, nine bf16 steps away).  head_dim 16 runs on the scalar kernel."""
+    b, want = two_key_cap_batch(DEV, head_dim=D)
+    out = to_np(run_hip(b, flags))[0, 0]
+    assert np.abs(out - want).max() <= 2.0 ** -8, out[:4]
+
+
+@pytest.mark.parametrize("flags", PATHS)
+def test_malformed_device_metadata_stays_in_bounds(flags):
+    """A key count beyond what the block-table row can address, a negative one, and row offsets beyond the query
+    buffer are clipped on the device (the reference's XLA program clamps every dynamic index; its Pallas path rejects
+    such input, _pallas_impl_fwd.py:124-174): the rows of the well-formed sequences are bitwise what they are
+    without the damage, nothing outside `out` is written, and the damaged sequences' rows are finite."""
+    q_lens, kv_lens = [4, 1, 1, 50, 1, 3], [200, 255, 40, 50, 100, 64]
+    b = small(q_lens, kv_lens, max_num_seqs=8)
+    T, Hq, D = b.queries.shape
+    base = run_hip(b, flags)
+    # every buffer the damaged lengths could run past is a window into a larger allocation
+    q_big = torch.zeros((T + 4096, Hq, D), dtype=b.queries.dtype, device=DEV)
+    q_big[:T] = b.queries
+    out_big = torch.full((T + 8192, Hq, D), 123.0, dtype=b.queries.dtype, device=DEV)
+    bt_big = torch.zeros((8 + 64, b.block_tables.shape[1]), dtype=torch.int32, device=DEV)
+    bt_big[:8] = b.block_tables
+    bad = Batch(**{**b.__dict__})
+    bad.queries, bad.block_tables = q_big[:T], bt_big[:8]
+    bad.context_lens = b.context_lens.clone()
+    bad.context_lens[1] = 100000        # 16 pages of 16 tokens can address 256 keys
+    bad.context_lens[2] = -7            # no keys: zeros
+    bad.query_start_loc = b.query_start_loc.clone()
+    bad.query_start_loc[6:] = T + 1000  # the last sequence's rows run past the buffer: clipped at T
+    out = RaggedPageAttention().run(*bad.args(), softmax_scale=b.softmax_scale, cfg=RaggedPageAttentionConfig(),
+                                    _flags=flags, _out=out_big[4096:4096 + T])
+    torch.cuda.synchronize()
+    assert bool((out_big[:4096] == 123.0).all()) and bool((out_big[4096 + T:] == 123.0).all()), "wrote outside out"
+    cu = np.concatenate([[0], np.cumsum(q_lens)])
+    for s in (0, 3, 4):
+        assert torch.equal(out[cu[s]:cu[s + 1]], base[cu[s]:cu[s + 1]]), f"well-formed sequence {s} changed"
+    assert torch.isfinite(out.float()).all()
+    assert not out[cu[2]:cu[3]].any(), "a sequence without keys yields zeros"
+    # sequence 1 attends to the 256 keys its pages hold (one more than before)
+    fixed = Batch(**{**b.__dict__})
+    fixed.context_lens = b.context_lens.clone()
+    fixed.context_lens[1] = 256
+    fixed.kv_lens = np.array(kv_lens)
+    fixed.kv_lens[1] = 256
+    assert_bf16_parity(to_np(out[cu[1]:cu[2]]), run_strict(fixed)[cu[1]:cu[2]], 1, "clipped key count")
+    # the last sequence keeps the rows that exist: with kv_len 64 and a (damaged) q_len beyond it, row r sits at
+    # position 64 - q_len + r of the clipped chunk
+    assert out.shape[0] == T
 
 
 # ----------------------------------------------------------------------------- invariants on the device result

@@ -195,8 +195,9 @@ def test_bf16_random_batches(seed):
 @pytest.mark.parametrize("D", [64, 192])
 @pytest.mark.parametrize("window", [None, 48])
 def test_cache_rows_padded_to_a_multiple_of_128(D, flags, window):
-    """head_dim 64 lives in cache rows of 128 elements, 192 in rows of 256 (merge_kv pads them): the update writes
-    head_dim elements per row and leaves the padding alone, the attention never reads it (it holds random data).
+    """head_dim 64 lives in cache rows of 128 elements, 192 in rows of 256 (merge_kv pads them with zeros): the update
+    writes whole token records, padding zeroed as the reference's scatter does (_kernel.py:44-57, :207-218), and leaves
+    other tokens' padding alone; the attention never reads it (it holds random data).
     head_dim 64 runs on the MFMA kernel's wave-level loop, 192 on the scalar kernel."""
     v = small([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], head_dim=D, pages_per_seq=32, sliding_window=window)
     dalign = -(-D // 128) * 128
@@ -205,7 +206,9 @@ def test_cache_rows_padded_to_a_multiple_of_128(D, flags, window):
     ref_out, ref_cache = oracle(v)
     out, cache = run_hip(v, flags)
     assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
-    assert torch.equal(cache[..., D:], before[..., D:]), "the padding was written"
+    written = (cache[..., :D] != before[..., :D]).flatten(2).any(-1)  # [pages, slots]: token records the update wrote
+    assert written.any() and bool((cache[..., D:][written] == 0).all()), "padding of an updated token is zeroed"
+    assert torch.equal(cache[..., D:][~written], before[..., D:][~written]), "padding of other tokens was written"
     assert out.shape == v.queries.shape
     assert_bf16_parity(to_np(out), ref_out, 176, f"padded rows D={D}")
 
@@ -220,7 +223,10 @@ def test_8bit_cache_rows_padded_to_a_multiple_of_128(f8):
                                 torch.float8_e5m2: "float8_e5m2"}[f8], query_dtype="bfloat16", **v.kwargs())
     out, cache = run_hip(v)
     assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
-    assert torch.equal(cache[..., 64:].view(torch.uint8), before[..., 64:].view(torch.uint8)), "the padding was written"
+    c8, b8 = cache.view(torch.uint8), before.view(torch.uint8)
+    written = (c8[..., :64] != b8[..., :64]).flatten(2).any(-1)
+    assert written.any() and bool((c8[..., 64:][written] == 0).all()), "padding of an updated token is zeroed"
+    assert torch.equal(c8[..., 64:][~written], b8[..., 64:][~written]), "padding of other tokens was written"
     assert_bf16_parity(to_np(out), ref_out, 176, "8-bit padded rows")
 
 
@@ -240,7 +246,7 @@ def test_bf16_random_batches_head_dim_64(seed):
 
 def test_8bit_cache_with_an_odd_number_of_kv_heads_pads_the_combined_heads():
     """One kv head under packing 4: the cache holds four combined heads per token, K, V and two of padding (merge_kv
-    pads them); the update leaves the padding alone and the attention never reads it."""
+    pads them with zeros); the update zeroes the padding heads of the tokens it writes and the attention never reads them."""
     f8 = torch.float8_e4m3fn
     v = to_v3(make_batch([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], num_q_heads=8, num_kv_heads=1, head_dim=128,
                          page_size=16, pages_per_seq=32, seed=3, device=DEV), seed=3, cache_dtype=f8)
@@ -250,8 +256,10 @@ def test_8bit_cache_with_an_odd_number_of_kv_heads_pads_the_combined_heads():
                                 **v.kwargs())
     out, cache = run_hip(v)
     assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
-    assert torch.equal(cache[:, :, :, 2:].view(torch.uint8), before[:, :, :, 2:].view(torch.uint8)), "padding heads written"
-    assert not torch.equal(cache[:, :, :, :2].view(torch.uint8), before[:, :, :, :2].view(torch.uint8))
+    c8, b8 = cache.view(torch.uint8), before.view(torch.uint8)
+    written = (c8[:, :, :, :2] != b8[:, :, :, :2]).flatten(2).any(-1)
+    assert written.any() and bool((c8[:, :, :, 2:][written] == 0).all()), "padding heads of an updated token are zeroed"
+    assert torch.equal(c8[:, :, :, 2:][~written], b8[:, :, :, 2:][~written]), "padding heads of other tokens were written"
     assert_bf16_parity(to_np(out), ref_out, 176, "8-bit cache, one kv head")
 
 

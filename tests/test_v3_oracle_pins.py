@@ -85,6 +85,38 @@ def test_cache_update_closed_form():
     assert (new != cache).any()
 
 
+@pytest.mark.parametrize("dtype,Hkv", [("bfloat16", 2), ("float8_e4m3fn", 1)])
+def test_padding_of_updated_tokens_is_zeroed_as_merge_kv_pads_it(dtype, Hkv):
+    """head_dim 64 in rows of 128 and (8-bit cache, one kv head) two combined heads padded to four, the cache filled
+    with non-zero values everywhere: the literal restatement scatters merge_kv's zero-padded rows (_kernel.py:44-57,
+    :207-218), so an updated token's padding becomes zero and every other byte of the cache stays; the efficient
+    restatement must give the same cache bit for bit."""
+    rng = np.random.default_rng(21)
+    q_lens, kv_lens = [3, 1, 0], [7, 9, 5]
+    D, page, pps = 64, 4, 4
+    pack = 2 if dtype == "bfloat16" else 4
+    hx2 = -(-2 * Hkv // pack) * pack
+    R = rpa_oracle._rounder(dtype)
+    q, k, v, _, lens, bt, qsl, dist = make(rng, q_lens, kv_lens, Hq=4, Hkv=Hkv, D=D, page=page, pps=pps)
+    k, v = R(k), R(v)
+    P = 4 * pps + 3
+    cache = R(1.0 + rng.random((P, page, hx2 // pack, pack, 128)).astype(np.float32))  # no zero anywhere
+    kw = dict(cache_dtype=dtype, query_dtype="bfloat16")
+    _, c_lit = rpa_v3_literal(q, k, v, cache, lens, bt, qsl, dist, **kw)
+    _, c_fast = rpa_v3(q, k, v, cache, lens, bt, qsl, dist, **kw)
+    assert np.array_equal(c_lit, c_fast)
+    rows = c_fast.reshape(P, page, hx2, 128)
+    before = cache.reshape(P, page, hx2, 128)
+    touched = np.zeros((P, page), bool)
+    for s, (ql, kl) in enumerate(zip(q_lens, kv_lens)):
+        for t in range(ql):
+            pos = kl - ql + t
+            touched[bt[s * pps + pos // page], pos % page] = True
+    assert touched.sum() == sum(q_lens)
+    assert not rows[touched][:, :, D:].any() and not rows[touched][:, 2 * Hkv:].any()
+    assert np.array_equal(rows[~touched], before[~touched])
+
+
 @pytest.mark.parametrize("window,cap", [(None, None), (5, None), (None, 8.0)])
 def test_attention_matches_the_dense_float64_oracle_on_the_updated_cache(window, cap):
     rng = np.random.default_rng(5)
