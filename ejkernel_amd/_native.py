@@ -26,6 +26,8 @@ EXPORTED_SYMBOLS = (
     "rpa_workspace_bytes",
     "rpa_workspace_init",
     "rpa_fwd_launch",
+    "rpa_fwd_launch_static",
+    "rpa_static_scratch_bytes",
     "rpa_v3_launch",
     "rpa_v3_workspace_bytes",
     "rpa_page_attention_workspace_bytes",
@@ -181,6 +183,10 @@ def load() -> ctypes.CDLL:
     lib.rpa_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     lib.rpa_fwd_launch.restype = ctypes.c_int
     lib.rpa_fwd_launch.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
+    lib.rpa_fwd_launch_static.restype = ctypes.c_int
+    lib.rpa_fwd_launch_static.argtypes = [ctypes.POINTER(RpaParams), ctypes.c_void_p]
+    lib.rpa_static_scratch_bytes.restype = ctypes.c_uint64
+    lib.rpa_static_scratch_bytes.argtypes = []
     lib.rpa_v3_workspace_bytes.restype = ctypes.c_uint64
     lib.rpa_v3_workspace_bytes.argtypes = [ctypes.POINTER(RpaV3Params)]
     lib.rpa_v3_launch.restype = ctypes.c_int

@@ -7,6 +7,7 @@
 #include <atomic>
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 
 #include "rpa_host.h"
 
@@ -96,6 +97,71 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
 
 namespace rpa {
 static int dispatch(const RpaParams& p, const KvLayout& kv, bool tiled, hipStream_t stream, const PreState& pre = PreState());
+}
+
+// ---- rpa_fwd_launch_static: the forward pass for callers that cannot allocate.
+//
+// The kernels' scratch (split tickets, prefill queue counters, partial attention states of split (sequence, kv head)s)
+// lives in a file-scope device array instead of a caller-supplied workspace.  Every GPU the library runs on holds its
+// own copy of the array until the process ends; its address on a GPU comes from hipGetSymbolAddress, looked up once per
+// device with that device current, and that pointer -- never the array's name, which in host code is only a handle --
+// is what the kernels receive.
+namespace rpa {
+constexpr uint64_t kStaticScratchBytes = 34ull << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+static std::mutex g_scratch_mu;
+static std::atomic<void*> g_scratch_ptr[64];  // per device; null until the first call there
+
+// Address of this device's copy of `scratch`; the first call on a device looks it up and clears the ticket region
+// (the loader zero-fills the array and every launch leaves the tickets at zero again, so this is belt and braces for
+// a process that aborted a launch half way).  Enqueue-only, no allocation.
+static int static_scratch(hipStream_t stream, void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(RPA_ERR_LAUNCH, "hipGetDevice failed or device index above 63");
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+      const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || p == nullptr)
+        return fail(RPA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+      hipLaunchKernelGGL(zero_fill_kernel, dim3(64), dim3(256), 0, stream, static_cast<uint4*>(p),
+                         static_cast<size_t>(kWorkspaceTicketBytes / 16));
+      if (hipGetLastError() != hipSuccess) return fail(RPA_ERR_LAUNCH, "clearing the static scratch tickets failed");
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
+    }
+  }
+  *out = p;
+  return RPA_OK;
+}
+}  // namespace rpa
+
+uint64_t rpa_static_scratch_bytes(void) { return rpa::kStaticScratchBytes; }
+
+int rpa_fwd_launch_static(const RpaParams* params, void* hip_stream) {
+  if (params == nullptr) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "params is null");
+  RpaParams p = *params;
+  int rc = rpa::validate(p, true);
+  if (rc != RPA_OK) return rc;
+  const bool tiled = rpa::tiled_supported(p);
+  p.workspace = nullptr;
+  p.workspace_bytes = 0;
+  if (tiled) {
+    const uint64_t need = rpa_workspace_bytes(&p);
+    if (need > rpa::kStaticScratchBytes)
+      return rpa::fail(RPA_ERR_WORKSPACE,
+                       "this shape needs %llu bytes of scratch, the static scratch of rpa_fwd_launch_static holds %llu: "
+                       "use rpa_fwd_launch with a workspace",
+                       (unsigned long long)need, (unsigned long long)rpa::kStaticScratchBytes);
+    void* ptr = nullptr;
+    rc = rpa::static_scratch(static_cast<hipStream_t>(hip_stream), &ptr);
+    if (rc != RPA_OK) return rc;
+    p.workspace = ptr;
+    p.workspace_bytes = rpa::kStaticScratchBytes;
+  }
+  return rpa::dispatch(p, rpa::interleaved_layout(p), tiled, static_cast<hipStream_t>(hip_stream));
 }
 
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream) {

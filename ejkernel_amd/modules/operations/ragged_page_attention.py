@@ -141,7 +141,7 @@ def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tens
 
 def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, *, softmax_scale,
             logits_soft_cap, compute_dtype, sliding_window, softmax_aux, cfg, flags: int = 0,
-            kv_start=None, out=None) -> torch.Tensor:
+            kv_start=None, out=None, static_scratch=False) -> torch.Tensor:
     lib = _native.load()
     if not queries.is_cuda:
         raise RuntimeError(
@@ -208,11 +208,14 @@ def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_
 
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream
-        nbytes = int(lib.rpa_workspace_bytes(ctypes.byref(p)))
-        ws = _workspace(dev, nbytes, stream_ptr)
-        p.workspace = ws.data_ptr()
-        p.workspace_bytes = ws.numel()
-        rc = lib.rpa_fwd_launch(ctypes.byref(p), ctypes.c_void_p(stream_ptr))
+        if static_scratch:  # the entry point that allocates nothing: scratch inside the library, no workspace
+            rc = lib.rpa_fwd_launch_static(ctypes.byref(p), ctypes.c_void_p(stream_ptr))
+        else:
+            nbytes = int(lib.rpa_workspace_bytes(ctypes.byref(p)))
+            ws = _workspace(dev, nbytes, stream_ptr)
+            p.workspace = ws.data_ptr()
+            p.workspace_bytes = ws.numel()
+            rc = lib.rpa_fwd_launch(ctypes.byref(p), ctypes.c_void_p(stream_ptr))
     if rc != 0:
         msg = _native.last_error()
         if rc == -1:
@@ -256,6 +259,7 @@ class RaggedPageAttention:
         _flags: int = 0,
         _kv_start=None,
         _out=None,
+        _static_scratch: bool = False,
     ):
         """Same parameters as the reference's ``run`` (``:225-318``).
 
@@ -272,7 +276,7 @@ class RaggedPageAttention:
         return _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs,
                        softmax_scale=softmax_scale, logits_soft_cap=logits_soft_cap, compute_dtype=compute_dtype,
                        sliding_window=sliding_window, softmax_aux=softmax_aux, cfg=cfg, flags=_flags,
-                       kv_start=_kv_start, out=_out)
+                       kv_start=_kv_start, out=_out, static_scratch=_static_scratch)
 
     def heuristic_cfg(self, inv=None) -> RaggedPageAttentionConfig:
         """Default configuration (``:320-337``)."""

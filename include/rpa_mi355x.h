@@ -146,6 +146,19 @@ int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stre
 /* Enqueues the forward pass on `hip_stream` (a hipStream_t; NULL = default stream). */
 int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
 
+/*
+ * rpa_fwd_launch for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  `workspace` / `workspace_bytes` of
+ * the params are ignored: the kernels' scratch (split tickets, queue counters, partial attention states) is a
+ * device array inside the library, rpa_static_scratch_bytes() = 34 MiB per GPU, held until the process ends.  The
+ * call allocates and frees nothing and never synchronises; results are those of rpa_fwd_launch, bit for bit.
+ * Shapes whose rpa_workspace_bytes() exceeds the array are rejected with RPA_ERR_WORKSPACE (head_dim 256 on the
+ * MFMA kernel, today).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU, on
+ * whatever streams, race -- serialise them (one stream, or events between streams).
+ */
+uint64_t rpa_static_scratch_bytes(void);
+int rpa_fwd_launch_static(const RpaParams* params, void* hip_stream);
+
 /* Bytes of workspace rpa_v3_launch needs (rpa_workspace_bytes() of `attn`, plus the row statistics of an 8-bit
  * cache). */
 uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims);
