@@ -1,0 +1,330 @@
+"""Generates rpa_prefill_pipe_asm.inc: the key loop of the software-pipelined prefill tile as one instruction stream.
+
+The tile of rpa_prefill_pipe.h runs one wavefront per SIMD, so matrix and vector work only overlap when one
+instruction stream interleaves them, and that stream keeps about 400 registers in fixed places (output accumulators
+and MFMA operands in accumulation registers, logits and probabilities in ordinary ones).  Left to the compiler, the
+same loop moved accumulators between the two register files every half and spilled; here it is written out with
+fixed registers.  The C++ side binds its variables to the same registers with physical-register constraints, so the
+compiler still sees every value that enters or leaves.  `python gen_prefill_pipe_asm.py` rewrites the .inc file; a
+CPU test compares the committed file with this script's output.
+
+Register map (one wavefront):
+  a[0:127]    O^T accumulators, row tile m, column block c: a[32 m + 4 c : +3]                     (out)
+  a[128:143]  row sums, row tile m: a[128 + 4 m : +3]                                             (out)
+  a[144:175]  K operands of one half, sub-tile u, k-step ks: a[144 + 4 (4 u + ks) : +3]
+  a[176:207]  V^T operands of one half, column block c: a[176 + 4 c : +3]
+  v[0:31]     logits / exp2 arguments, buffer A: row tile m, sub-tile u: v[4 (2 m + u) : +3]
+  v[32:63]    the same, buffer B (halves alternate between the buffers)
+  v[64:127]   Q operands, row tile m, k-step ks: v[64 + 4 (4 m + ks) : +3]                        (in)
+  v[128:143]  P^T operands, row tile m: v[128 + 4 m : +3]
+  v[144:147]  eight bf16 ones (operand of the row-sum MFMA)
+  v[148:151]  -m log2(e) per row tile, the offset of the exp2 argument                            (out)
+  v[152:155]  maximum exp2 argument of the half per row tile
+  v[156:159]  masked halves: first visible key of the lane's rows relative to the lane's first key of the half
+  v[160:163]  visible keys of the lane's rows minus one (0 with an unreachable first key: none)   (in)
+  v[164:167]  LDS address of the K operand reads per k-step (stage of the next tile);  v168  of the V^T reads
+  v169        factor of the exp2 argument: log2(e) times the fp32 logit scale                     (in)
+  v170, v195:199  temporaries;  v171  -inf
+  v[172:175]  threshold of the exp2 arguments per row tile: -inf before a row's first key         (out)
+  v176        the threshold once a row has a reference point
+  v[178:181]  first visible key of the lane's rows minus 4 g (absolute)                           (in)
+  v[182:185]  LDS address of the K operand reads per k-step in stage 0;  v186  of the V^T reads   (in)
+  v[187:189]  fetch: the lane's row in a K block, in a V block, byte offset of its V piece        (in)
+  v[190:193]  fetch: byte offset of the lane's 16-byte piece in a K row, per block of four rows   (in)
+  s[36:43]    halves of this wavefront, tiles, first key of the range, all_lo, all_hi (a half starting at a0 needs no
+              mask iff all_lo < a0 <= all_hi), last key of the range, 16 * wavefront, LDS address of the wavefront's
+              part of stage 0                                                                     (in)
+  s[44:51]    block table row (64 bit), cache base of the kv head's K rows (64 bit), bytes per token, bytes per page,
+              log2(page size), pages - 1                                                          (in)
+  s[52:79]    temporaries
+"""
+
+from __future__ import annotations
+
+import os
+
+MRT, NKS, CB = 4, 4, 8
+ROWB = 256
+STAGE_B = 32768   # K tile + V tile
+NSTG = 3
+LAZY_LOG2E = 16.0 * 1.4426950408889634
+
+O = lambda m, c: f"a[{32 * m + 4 * c}:{32 * m + 4 * c + 3}]"
+L = lambda m: f"a[{128 + 4 * m}:{128 + 4 * m + 3}]"
+KOP = lambda u, ks: f"a[{144 + 4 * (4 * u + ks)}:{144 + 4 * (4 * u + ks) + 3}]"
+VRAW2 = lambda c, u: f"a[{176 + 4 * c + 2 * u}:{176 + 4 * c + 2 * u + 1}]"
+VRAW = lambda c: f"a[{176 + 4 * c}:{176 + 4 * c + 3}]"
+SQ = lambda base, m, u: f"v[{base + 4 * (2 * m + u)}:{base + 4 * (2 * m + u) + 3}]"
+SE = lambda base, m, u, r: f"v{base + 4 * (2 * m + u) + r}"
+QOP = lambda m, ks: f"v[{64 + 4 * (4 * m + ks)}:{64 + 4 * (4 * m + ks) + 3}]"
+PW = lambda m: f"v[{128 + 4 * m}:{128 + 4 * m + 3}]"
+PWE = lambda m, k: f"v{128 + 4 * m + k}"
+ONES = "v[144:147]"
+MNEG = lambda m: f"v{148 + m}"
+TMAX = lambda m: f"v{152 + m}"
+MLO = lambda m: f"v{156 + m}"
+MSPAN = lambda m: f"v{160 + m}"
+KADDR = lambda ks: f"v{164 + ks}"
+VADDR = "v168"
+CFAC = "v169"
+T0 = "v170"
+NINF = "v171"
+MTHR = lambda m: f"v{172 + m}"
+THRC = "v176"
+ROWLO = lambda m: f"v{178 + m}"
+KBASE = lambda ks: f"v{182 + ks}"
+VBASE = "v186"
+LROW, VROW, VPIECE = "v187", "v188", "v189"
+KPIECE = lambda n: f"v{190 + n}"
+T1, T2, T3, T4, T5 = "v195", "v196", "v197", "v198", "v199"
+MFMA = "v_mfma_f32_16x16x32_bf16"
+
+# scalar inputs
+S_HB, S_NT, S_RLO, S_ALLLO, S_ALLHI, S_TLAST, S_WAVE16, S_LDSW = (f"s{36 + k}" for k in range(8))
+S_BTLO, S_BTHI, S_KVLO, S_KVHI, S_STRIDE, S_PAGEB, S_PSHIFT, S_NP1 = (f"s{44 + k}" for k in range(8))
+# scalar temporaries
+S_HH, S_T, S_A0, S_CUR, S_NXT, S_FBUF = "s52", "s53", "s54", "s55", "s56", "s57"   # loop state; stage byte offsets
+S_R = "s[60:63]"                                                                   # buffer resource of a fetch
+S_R0, S_R1, S_R2, S_R3 = "s60", "s61", "s62", "s63"
+S_X0, S_X1, S_X2, S_X3, S_X4, S_X5 = "s64", "s65", "s66", "s67", "s68", "s69"
+S_P = "s[70:71]"
+S_PMASK = "s72"
+S_TT = "s73"
+
+
+def kload(h: int) -> list[str]:
+    """K operands of a half with parity h from the stage that v[164:167] point into."""
+    return [f"ds_read_b128 {KOP(u, ks)}, {KADDR(ks)} offset:{h * 32 * ROWB + u * 16 * ROWB}" for u in range(2) for ks in range(NKS)]
+
+
+def vload(h: int) -> list[str]:
+    """V^T operands of a half with parity h: per column block the keys 4g..4g+3 of both 16-key sub-tiles."""
+    return [f"ds_read_b64_tr_b16 {VRAW2(c, u)}, {VADDR} offset:{(8 * h + 4 * u) * 1024 + c * 128}" for c in range(CB) for u in range(2)]
+
+
+def qk(n: int, nxt: int) -> str:
+    """MFMA n (0..31) of S^T = K Q^T: k-step outermost, so consecutive MFMAs feed different accumulators."""
+    ks, u, m = n >> 3, (n >> 2) & 1, n & 3
+    c = "0" if ks == 0 else SQ(nxt, m, u)
+    return f"{MFMA} {SQ(nxt, m, u)}, {KOP(u, ks)}, {QOP(m, ks)}, {c}"
+
+
+def sm1_pair(cur: int, m: int, e: int, mask: bool, rnd: bool) -> list[str]:
+    """Elements e, e + 1 of row tile m: logit -> exp2 argument in place, running maximum."""
+    u, r = e >> 2, e & 3
+    x0, x1 = SE(cur, m, u, r), SE(cur, m, u, r + 1)
+    out = []
+    if mask:
+        for x, cst in ((x0, 16 * u + r), (x1, 16 * u + r + 1)):
+            out += [f"v_sub_u32 {T0}, {cst}, {MLO(m)}", f"v_cmp_le_u32 vcc, {T0}, {MSPAN(m)}", f"v_cndmask_b32 {x}, {NINF}, {x}, vcc"]
+    if rnd:
+        out += [f"v_cvt_pk_bf16_f32 {T0}, {x0}, {x1}", f"v_lshlrev_b32 {x0}, 16, {T0}", f"v_and_b32 {x1}, 0xffff0000, {T0}"]
+    out += [f"v_fma_f32 {x0}, {x0}, {CFAC}, {MNEG(m)}", f"v_fma_f32 {x1}, {x1}, {CFAC}, {MNEG(m)}"]
+    out += [f"v_max_f32 {TMAX(m)}, {x0}, {x1}" if e == 0 else f"v_max3_f32 {TMAX(m)}, {TMAX(m)}, {x0}, {x1}"]
+    return out
+
+
+def block_a(h: int, mask: bool, rnd: bool) -> list[str]:
+    """[QK(next half) | SM1(this half)]: 32 slots of one MFMA and half a pair's vector work."""
+    cur, nxt = (0, 32) if h == 0 else (32, 0)
+    out = ["s_waitcnt lgkmcnt(0)"] + vload(h)
+    if mask:
+        out += [f"v_subrev_u32 {MLO(m)}, {S_A0}, {ROWLO(m)}" for m in range(MRT)]
+    for n in range(32):
+        out.append(qk(n, nxt))
+        if n % 2 == 0:
+            out += sm1_pair(cur, n >> 3, n & 7, mask, rnd)
+    return out
+
+
+def sm2_exp(cur: int, m: int, k: int) -> list[str]:
+    u, r = k >> 1, 2 * (k & 1)
+    return [f"v_exp_f32 {SE(cur, m, u, r)}, {SE(cur, m, u, r)}", f"v_exp_f32 {SE(cur, m, u, r + 1)}, {SE(cur, m, u, r + 1)}"]
+
+
+def sm2_pack(cur: int, m: int, k: int) -> list[str]:
+    u, r = k >> 1, 2 * (k & 1)
+    return [f"v_cvt_pk_bf16_f32 {PWE(m, k)}, {SE(cur, m, u, r)}, {SE(cur, m, u, r + 1)}"]
+
+
+def sm2_tile(cur: int, m: int) -> list[list[str]]:
+    """P of row tile m = exp2 of its eight arguments, packed to bf16, in four groups of instructions.  The result of
+    a transcendental instruction may not be read by the very next instruction (the hardware does not wait), so the
+    pack of a pair follows the next pair's exponentials."""
+    return [sm2_exp(cur, m, 0), sm2_exp(cur, m, 1) + sm2_pack(cur, m, 0), sm2_exp(cur, m, 2) + sm2_pack(cur, m, 1),
+            sm2_exp(cur, m, 3) + sm2_pack(cur, m, 2) + ["s_nop 0"] + sm2_pack(cur, m, 3)]
+
+
+def block_b(h: int) -> list[str]:
+    """[SM2 | PV]: the exponentials of row tile m + 1 under the 9 MFMAs of row tile m."""
+    cur = 0 if h == 0 else 32
+    out = kload(h) + ["s_waitcnt lgkmcnt(8)"]
+    for grp in sm2_tile(cur, 0):
+        out += grp
+    out.append("s_nop 1")
+    for m in range(MRT):
+        out.append(f"{MFMA} {L(m)}, {ONES}, {PW(m)}, {L(m)}")
+        nxt = sm2_tile(cur, m + 1) if m + 1 < MRT else None
+        for c in range(CB):
+            out.append(f"{MFMA} {O(m, c)}, {VRAW(c)}, {PW(m)}, {O(m, c)}")
+            # P of the next row tile, its last pack two MFMAs ahead of the MFMA that reads it (a vector write needs
+            # two wait states before an MFMA reads the register)
+            if nxt is not None and c in (0, 2, 4, 5):
+                out += nxt[(0, 2, 4, 5).index(c)]
+    return out
+
+
+def rescale(h: int, tag: str) -> list[str]:
+    """Vote; where some row's exp2 argument exceeds its threshold (or the row sees its first key), move that row's
+    reference point up by the row maximum: shift the exp2 arguments, scale row sum and outputs by exp2(-shift)."""
+    cur = 0 if h == 0 else 32
+    out = [f"v_cmp_gt_f32 vcc, {TMAX(0)}, {MTHR(0)}"]
+    for m in range(1, MRT):
+        out += [f"v_cmp_gt_f32 {S_P}, {TMAX(m)}, {MTHR(m)}", f"s_or_b64 vcc, vcc, {S_P}"]
+    out.append(f"s_cbranch_vccz .Lpp_noresc_{tag}_%=")
+    for m in range(MRT):
+        x = TMAX(m)
+        # maximum over the four lanes that hold one row (lanes l, l ^ 16, l ^ 32, l ^ 48)
+        out += [f"v_mov_b32 {T1}, {x}", f"v_mov_b32 {T2}, {x}", "s_nop 1", f"v_permlane16_swap_b32 {T1}, {T2}", "s_nop 1",
+                f"v_max_f32 {T3}, {T1}, {T2}", f"v_mov_b32 {T1}, {T3}", f"v_mov_b32 {T2}, {T3}", "s_nop 1",
+                f"v_permlane32_swap_b32 {T1}, {T2}", "s_nop 1", f"v_max_f32 {T3}, {T1}, {T2}"]
+        out += [f"v_cmp_gt_f32 vcc, {T3}, {MTHR(m)}", f"s_cbranch_vccz .Lpp_skip{m}_{tag}_%="]
+        out += [f"v_cndmask_b32 {T4}, 0, {T3}, vcc",                       # shift: the row maximum where the row moves
+                f"v_exp_f32_e64 {T5}, -{T3}",
+                f"v_cmp_neq_f32 {S_P}, {MTHR(m)}, {NINF}",
+                f"v_cndmask_b32_e64 {T5}, 0, {T5}, {S_P}",                 # a row without a reference point: outputs are zero
+                f"v_cndmask_b32 {T5}, 1.0, {T5}, vcc",                     # alpha
+                f"v_cndmask_b32 {MTHR(m)}, {MTHR(m)}, {THRC}, vcc"]
+        out += [f"v_sub_f32 {SE(cur, m, u, r)}, {SE(cur, m, u, r)}, {T4}" for u in range(2) for r in range(4)]
+        out.append(f"v_sub_f32 {MNEG(m)}, {MNEG(m)}, {T4}")
+        regs = [128 + 4 * m + k for k in range(4)] + [32 * m + k for k in range(32)]
+        for q in range(0, len(regs), 4):
+            grp = regs[q:q + 4]
+            tmp = [T1, T2, T3, T4]
+            out += [f"v_accvgpr_read_b32 {t}, a{a}" for t, a in zip(tmp, grp)]
+            out += [f"v_mul_f32 {t}, {t}, {T5}" for t in tmp]
+            out += [f"v_accvgpr_write_b32 a{a}, {t}" for t, a in zip(tmp, grp)]
+        out.append(f".Lpp_skip{m}_{tag}_%=:")
+    out.append(f".Lpp_noresc_{tag}_%=:")
+    return out
+
+
+def fetch(tag: str) -> list[str]:
+    """This wavefront's part (16 K rows, 16 V rows) of the tile whose first key is in S_TT, into the stage at byte
+    offset S_FBUF.  Keys past the range repeat the last one; the 16 keys share a page (pages of at least 16 keys)."""
+    out = [f"s_add_i32 {S_X0}, {S_TT}, {S_WAVE16}",            # first key of the group
+           f"s_and_b32 {S_X1}, {S_TLAST}, -16",
+           f"s_min_i32 {S_X1}, {S_X1}, {S_X0}",                 # base key: same page as every key fetched
+           f"s_sub_i32 {S_X2}, {S_X0}, {S_X1}",                 # d
+           f"s_sub_i32 {S_X3}, {S_TLAST}, {S_X1}",              # last row that exists, relative to the base
+           f"s_lshr_b32 {S_X4}, {S_X1}, {S_PSHIFT}", f"s_lshl_b32 {S_X4}, {S_X4}, 2",
+           f"s_add_u32 {S_X4}, {S_BTLO}, {S_X4}", f"s_addc_u32 {S_X5}, {S_BTHI}, 0",
+           f"s_load_dword {S_X0}, s[68:69], 0x0",
+           f"v_add_u32 {T1}, {S_X2}, {LROW}", f"v_add_u32 {T2}, {S_X2}, {VROW}"]
+    vo = ["v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207"]
+    for n in range(4):
+        out += [f"v_add_u32 {T3}, {4 * n}, {T1}", f"v_min_i32 {T3}, {S_X3}, {T3}", f"v_mad_u32_u24 {vo[n]}, {T3}, {S_STRIDE}, {KPIECE(n)}",
+                f"v_add_u32 {T3}, {4 * n}, {T2}", f"v_min_i32 {T3}, {S_X3}, {T3}", f"v_mad_u32_u24 {vo[4 + n]}, {T3}, {S_STRIDE}, {VPIECE}"]
+    out += ["s_waitcnt lgkmcnt(0)",
+            f"s_max_i32 {S_X0}, {S_X0}, 0", f"s_min_i32 {S_X0}, {S_X0}, {S_NP1}",
+            f"s_mul_hi_u32 {S_X5}, {S_X0}, {S_PAGEB}", f"s_mul_i32 {S_X4}, {S_X0}, {S_PAGEB}",
+            f"s_and_b32 {S_X1}, {S_X1}, {S_PMASK}", f"s_mul_i32 {S_X1}, {S_X1}, {S_STRIDE}",
+            f"s_add_u32 {S_X4}, {S_X4}, {S_X1}", f"s_addc_u32 {S_X5}, {S_X5}, 0",
+            f"s_add_u32 {S_R0}, {S_X4}, {S_KVLO}", f"s_addc_u32 {S_R1}, {S_X5}, {S_KVHI}",
+            f"s_and_b32 {S_R1}, {S_R1}, 0xffff",
+            f"s_add_i32 {S_X0}, {S_LDSW}, {S_FBUF}"]
+    for n in range(4):
+        out += [f"s_add_i32 m0, {S_X0}, {n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[n]}, {S_R}, 0 offen lds",
+                f"s_add_i32 m0, {S_X0}, {16384 + n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[4 + n]}, {S_R}, 0 offen lds"]
+    return out
+
+
+def publish(tag: str, t_reg: str) -> list[str]:
+    """Publishes tile t + 1 (this wavefront's part has landed; after the barrier everybody's) and refills the stage
+    of tile t - 1 with tile t + 2.  S_FBUF is the byte offset of that stage."""
+    return ["s_waitcnt vmcnt(0)", "s_barrier",
+            f"s_add_i32 {S_X0}, {t_reg}, 2", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_nofetch_{tag}_%=",
+            f"s_lshl_b32 {S_TT}, {S_X0}, 6", f"s_add_i32 {S_TT}, {S_TT}, {S_RLO}"] + fetch(tag) + [f".Lpp_nofetch_{tag}_%=:"]
+
+
+def half(h: int, rnd: bool) -> list[str]:
+    tag = f"h{h}"
+    out = [f"s_cmp_gt_i32 {S_A0}, {S_ALLLO}", f"s_cbranch_scc0 .Lpp_mask_{tag}_%=",
+           f"s_cmp_le_i32 {S_A0}, {S_ALLHI}", f"s_cbranch_scc0 .Lpp_mask_{tag}_%="]
+    out += block_a(h, False, rnd) + [f"s_branch .Lpp_adone_{tag}_%=", f".Lpp_mask_{tag}_%=:"] + block_a(h, True, rnd) + [f".Lpp_adone_{tag}_%=:"]
+    out += rescale(h, tag)
+    if h == 0:
+        out += [f"s_add_i32 {S_X0}, {S_T}, 1", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_nopub_%="]
+        out += publish("loop", S_T) + [".Lpp_nopub_%=:"]
+    out += block_b(h)
+    out += [f"s_add_i32 {S_HH}, {S_HH}, 1", f"s_add_i32 {S_A0}, {S_A0}, 32", f"s_cmp_eq_u32 {S_HH}, {S_HB}", "s_cbranch_scc1 .Lpp_done_%="]
+    return out
+
+
+def rotate_stages() -> list[str]:
+    """Start of a tile: stage offsets of this tile, the next one and the one to refill; operand addresses."""
+    out = [f"s_mov_b32 {S_FBUF}, {S_CUR}",      # after this tile's barrier the previous tile's stage is refilled ...
+           f"s_mov_b32 {S_CUR}, {S_NXT}",
+           f"s_add_i32 {S_NXT}, {S_NXT}, {STAGE_B}", f"s_cmp_eq_u32 {S_NXT}, {NSTG * STAGE_B}", f"s_cselect_b32 {S_NXT}, 0, {S_NXT}"]
+    out += [f"v_add_u32 {VADDR}, {S_CUR}, {VBASE}"] + [f"v_add_u32 {KADDR(ks)}, {S_NXT}, {KBASE(ks)}" for ks in range(NKS)]
+    return out
+
+
+def loop(rnd: bool) -> list[str]:
+    out = ["s_mov_b32 s58, m0"]  # the compiler's m0 is restored at the end
+    # ---- set-up
+    out += [f"v_accvgpr_write_b32 a{k}, 0" for k in range(144)]
+    out += [f"v_mov_b32 {MNEG(m)}, 0" for m in range(MRT)] + [f"v_mov_b32 {NINF}, 0xff800000"]
+    out += [f"v_mov_b32 {MTHR(m)}, {NINF}" for m in range(MRT)]
+    out += [f"v_mov_b32 {THRC}, 0x{float_bits(LAZY_LOG2E):08x}"] + [f"v_mov_b32 v{144 + k}, 0x3f803f80" for k in range(4)]
+    out += [f"s_mov_b32 {S_R2}, 0x7fffffff", f"s_mov_b32 {S_R3}, 0x00020000",
+            f"s_lshl_b32 {S_PMASK}, 1, {S_PSHIFT}", f"s_add_i32 {S_PMASK}, {S_PMASK}, -1",
+            f"s_mov_b32 {S_HH}, 0", f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_A0}, {S_RLO}",
+            f"s_cmp_eq_u32 {S_HB}, 0", "s_cbranch_scc1 .Lpp_done_%="]
+    # stage state as if tile -1 were in progress: the first rotation makes tile 0 current
+    out += [f"s_mov_b32 {S_CUR}, {(NSTG - 1) * STAGE_B}", f"s_mov_b32 {S_NXT}, 0"]
+    # logits of the first half, K operands of the second (both in tile 0, stage 0)
+    out += [f"v_mov_b32 {KADDR(ks)}, {KBASE(ks)}" for ks in range(NKS)]
+    out += kload(0) + ["s_waitcnt lgkmcnt(0)"] + [qk(n, 0) for n in range(32)] + ["s_nop 7", "s_nop 7"] + kload(1)
+    out.append(".Lpp_tile_%=:")
+    out += rotate_stages()
+    out += half(0, rnd) + half(1, rnd)
+    out += [f"s_add_i32 {S_T}, {S_T}, 1", "s_branch .Lpp_tile_%="]
+    # ---- tiles past this wavefront's last half: it still takes part in their barriers and fetches
+    out += [".Lpp_done_%=:",
+            f"s_add_i32 {S_X5}, {S_HH}, 1", f"s_lshr_b32 {S_T}, {S_X5}, 1",
+            # the stage to refill at tile t's barrier is that of tile t - 1
+            f"s_add_i32 {S_X0}, {S_T}, {NSTG - 1}", f"s_mul_hi_u32 {S_X1}, {S_X0}, 0xaaaaaaab", f"s_lshr_b32 {S_X1}, {S_X1}, 1",
+            f"s_mul_i32 {S_X1}, {S_X1}, {NSTG}", f"s_sub_i32 {S_X0}, {S_X0}, {S_X1}", f"s_mul_i32 {S_FBUF}, {S_X0}, {STAGE_B}",
+            ".Lpp_tail_%=:",
+            f"s_add_i32 {S_X0}, {S_T}, 1", f"s_cmp_ge_i32 {S_X0}, {S_NT}", "s_cbranch_scc1 .Lpp_end_%="]
+    out += publish("tail", S_T)
+    out += [f"s_add_i32 {S_T}, {S_T}, 1",
+            f"s_add_i32 {S_FBUF}, {S_FBUF}, {STAGE_B}", f"s_cmp_eq_u32 {S_FBUF}, {NSTG * STAGE_B}", f"s_cselect_b32 {S_FBUF}, 0, {S_FBUF}",
+            "s_branch .Lpp_tail_%=", ".Lpp_end_%=:", "s_waitcnt lgkmcnt(0)", "s_mov_b32 m0, s58", "s_nop 7", "s_nop 7"]
+    return out
+
+
+def float_bits(x: float) -> int:
+    import struct
+    return struct.unpack("<I", struct.pack("<f", x))[0]
+
+
+def macro(name: str, lines: list[str]) -> str:
+    body = " \\\n".join(f'  "{ln}\\n\\t"' for ln in lines)
+    return f"#define {name} \\\n{body}\n"
+
+
+def render() -> str:
+    parts = ["// Generated by gen_prefill_pipe_asm.py -- do not edit; see that file for the register map.\n#pragma once\n"]
+    parts.append(macro("RPA_PPA_LOOP_ROUND", loop(True)))
+    parts.append(macro("RPA_PPA_LOOP_PLAIN", loop(False)))
+    return "\n".join(parts)
+
+
+INC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "rpa_prefill_pipe_asm.inc")
+
+if __name__ == "__main__":
+    with open(INC, "w") as f:
+        f.write(render())
+    print(f"wrote {INC}")

@@ -1,0 +1,371 @@
+// Workgroup-level attention tile for large prefill batches at head_dim 128: one wavefront per SIMD, software-pipelined.
+//
+// One workgroup (4 wavefronts, the only one on its compute unit: up to 512 registers per lane) owns 256 consecutive
+// rows of one (sequence, kv head) -- 64 rows = 4 MFMA row tiles per wavefront, so every K / V operand read from LDS
+// feeds four MFMAs -- and walks the keys those rows can see in tiles of 64, fetched into LDS stages as in
+// rpa_prefill.h (same layouts: K rows swizzled, V by 32-byte column units for the transposing read).
+//
+// With one wavefront per SIMD nothing but the wavefront's own instruction order overlaps matrix and vector work, so the
+// loop is written as that order.  Per 32-key half h the work is
+//     QK(h)   S^T = K Q^T                                   32 MFMAs
+//     SM1(h)  exp2 arguments t = s c - m c and their maxima  vector
+//     SM2(h)  P = exp2(t) rounded to bf16                    vector
+//     PV(h)   row sums and O^T += V^T P^T                    36 MFMAs
+// and the stream runs  [QK(h+1) | SM1(h)]  [SM2(h) | PV(h)]: the matrix pipe works on the next half's logits while
+// the vector unit prepares this half's softmax, then on this half's P V while the vector unit exponentiates, one row
+// tile ahead.  Each "|" is an explicit interleave -- one MFMA, a few vector instructions, fenced by scheduling
+// barriers -- because the compiler's own order keeps the two kinds apart.  Both phases are bound by the matrix pipe
+// when the interleave holds (512 and 576 cycles of MFMA against about 400 and 460 cycles of vector issue).
+// LDS operands are requested one phase ahead (V of half h at the start of [QK|SM1], K of half h+2 at the start of
+// [SM2|PV]); the tile that a half needs is published by one barrier per tile, placed between the two phases of a
+// tile's first half, and the stage freed by it is refilled at once, NSTG - 1 tiles ahead of its use.
+//
+// Halves that need per-key masks (causal diagonal, window edge, end of the range, first visible key) or a soft cap
+// run the same stream with those steps added (`kGeneral`).  A wavefront stops computing after the last half its rows
+// can see and keeps taking part in fetches and barriers; halves left of a wavefront's window but inside the
+// workgroup's range are walked with every key masked.
+#pragma once
+
+#include <type_traits>
+
+#include "rpa_prefill.h"
+
+namespace rpa {
+
+#ifndef RPA_PP_NSTG
+#define RPA_PP_NSTG 3
+#endif
+#ifndef RPA_PP_ROUND
+#define RPA_PP_ROUND 1
+#endif
+
+struct PipeCfg {
+  static constexpr int D = 128;
+  static constexpr int MRT = 4;                     // 16-row tiles per wavefront
+  static constexpr int NKS = D / 32;                // k-steps of the QK^T contraction
+  static constexpr int CB = D / 16;                 // MFMA column blocks of the output
+  static constexpr int TK = 64;                     // keys per tile (two halves of 32)
+  static constexpr int ROWB = D * 2;                // LDS bytes per K row
+  static constexpr int WROWS = 16 * MRT;            // rows per wavefront
+  static constexpr int WGROWS = kWgWaves * WROWS;   // rows per workgroup: 256
+  static constexpr int TILE_B = TK * ROWB;          // one K (or V) tile: 16 KiB
+  static constexpr int NSTG = RPA_PP_NSTG;          // LDS stages
+  static constexpr int LDS = 2 * NSTG * TILE_B;
+  static constexpr int PR = D / 8;                  // 16-byte pieces per row
+  static constexpr int RB = kWave / PR;             // rows one wave-wide load covers: 4
+  static constexpr int HB = TK / RB / kWgWaves;     // K (and V) load instructions per wavefront and tile: 4
+  static constexpr int GROUP = RB * HB;             // rows of the K and of the V tile a wavefront moves: 16
+  static constexpr int LOADS = 2 * HB;              // load instructions per wavefront and tile
+  // Logits are rounded to bf16 before the softmax where the reference rounds them (_xla_impl_fwd.py:119-124).
+  static constexpr bool ROUND = RPA_PP_ROUND != 0;
+  static __device__ __forceinline__ int swz(int row) { return row & 15; }
+};
+
+
+typedef __attribute__((ext_vector_type(32))) float f32x32_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) int i32x4_t;
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+
+#include "rpa_prefill_pipe_asm.inc"
+
+// What the key loop takes and leaves, each member bound to the registers the instruction stream uses for it
+// (register map in gen_prefill_pipe_asm.py).
+struct PipeIo {
+  f32x32_t o0, o1, o2, o3;  // out: O^T accumulators of the four row tiles
+  f32x16_t l;               // out: row sums
+  f32x4_t mneg, mthr;       // out: exp2 offset and threshold per row tile
+  f32x32_t q0, q1;          // in: Q operands
+  i32x4_t mspan, rowlo;     // in: per-lane bounds of the visible keys
+  i32x4_t kbase, kpiece;    // in: LDS addresses of the K operand reads; fetch: piece offsets in a K row
+  i32x4_t misc;             // in: LDS address of the V^T reads, fetch: row in a K block, in a V block, V piece offset
+  float cfac;               // in: factor of the exp2 argument
+  i32x8_t s0, s1;           // in: scalars (see the register map)
+};
+
+#define RPA_PPA_CLOBBERS                                                                                                  \
+  "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17",    \
+  "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33", "v34", \
+  "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", \
+  "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v128", "v129", "v130", "v131",    \
+  "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145",        \
+  "v146", "v147", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v164", "v165", "v166", "v167",        \
+  "v168", "v170", "v171", "v176", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204",        \
+  "v205", "v206", "v207", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154",        \
+  "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168",        \
+  "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182",        \
+  "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192", "a193", "a194", "a195", "a196",        \
+  "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", "s52", "s53", "s54", "s55",    \
+  "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", \
+  "s73", "vcc", "scc", "memory"
+
+// The key loop of one tile for one wavefront.  LDS stages 0 and 1 hold the first two K/V tiles (or the only one) and
+// have been published by a barrier; the stream runs every later barrier and fetch of the tile itself.
+template <bool kRound>
+__device__ __forceinline__ void pipe_key_loop(PipeIo& R) {
+#define RPA_PPA_OPERANDS                                                                                                  \
+  : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={a[128:143]}"(R.l),          \
+    "={v[148:151]}"(R.mneg), "={v[172:175]}"(R.mthr)                                                                   \
+  : "{v[64:95]}"(R.q0), "{v[96:127]}"(R.q1), "{v[160:163]}"(R.mspan), "{v[178:181]}"(R.rowlo), "{v[182:185]}"(R.kbase), \
+    "{v[186:189]}"(R.misc), "{v[190:193]}"(R.kpiece), "{v169}"(R.cfac), "{s[36:43]}"(R.s0), "{s[44:51]}"(R.s1)         \
+  : RPA_PPA_CLOBBERS
+  if constexpr (kRound) asm volatile(RPA_PPA_LOOP_ROUND RPA_PPA_OPERANDS);
+  else asm volatile(RPA_PPA_LOOP_PLAIN RPA_PPA_OPERANDS);
+#undef RPA_PPA_OPERANDS
+}
+
+template <bool kMimic>
+__device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
+                                                  int qt) {
+  using C = PipeCfg;
+  constexpr int MRT = C::MRT;
+  const RpaParams& p = a.p;
+  const int tid = threadIdx.x;
+  const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+  const int i = lane & 15, g = lane >> 4;
+  const int G = p.num_q_heads / p.num_kv_heads;
+  const int W = p.sliding_window;
+  const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
+  bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
+  const char* kvb = static_cast<const char*>(p.kv_pages);
+  const float cap = kMimic ? rbf(p.logits_soft_cap) : p.logits_soft_cap;
+  const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
+  const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
+  constexpr int hd = C::D;
+
+  // ---- key range of the workgroup's rows
+  const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
+  const int wg_pos_min = pos0 + wg_row_lo / G, wg_pos_max = pos0 + (wg_row_hi - 1) / G;
+  const int range_hi = min(si.kv_len, wg_pos_max + 1);
+  const int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
+  const int t_last = range_hi - 1;
+
+  // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
+  const int w_row_lo = wg_row_lo + wave * C::WROWS;
+  int pos_n[MRT];
+  auto row_of = [&](int m, int opaque0, bool& valid, int& head, size_t& q_off) {
+    const int R = w_row_lo + 16 * m + i + opaque0;
+    valid = R < si.rows;
+    const int qi = valid ? R / G : 0;
+    head = j * G + (valid ? R - qi * G : 0);
+    q_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * hd;
+    return qi;
+  };
+  bf16x8_t qreg[MRT][C::NKS];
+  const float scale = rbf(p.softmax_scale);
+  const float post_scale = logit_scale(p);
+  // Without a soft cap the fp32 logit scale of the unscaled-q arithmetic is folded into the exp2 argument.
+  const bool fold_scale = !kMimic && cap == 0.f;
+  const float sf = fold_scale ? post_scale : 1.f, sf_log2e = sf * kLog2e;
+  // One interval test per half: no row tile of this wavefront needs a per-key mask iff all_lo < a0 <= all_hi.
+  int all_lo = -0x7fffffff, all_hi = 0x7fffffff;
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    bool valid;
+    int head;
+    size_t q_off;
+    const int qi = row_of(m, 0, valid, head, q_off);
+    pos_n[m] = valid ? pos0 + qi : -1;
+    const int tr_lo = w_row_lo + 16 * m, tr_hi = min(tr_lo + 16, si.rows);
+    const bool t_any = tr_hi > tr_lo;
+    const int t_pos_lo = pos0 + tr_lo / G, t_pos_hi = pos0 + (max(tr_hi, tr_lo + 1) - 1) / G;
+    // the row tile sees all 32 keys from a0 on iff nomask_lo < a0 <= nomask_hi (a tile without rows never does)
+    const int nomask_hi = t_any ? min(t_pos_lo - 31, range_hi - 32) : -0x7fffffff;
+    const int nomask_lo = max(W > 0 ? t_pos_hi - W : -0x7fffffff, si.start - 1);
+    all_lo = max(all_lo, nomask_lo);
+    all_hi = min(all_hi, nomask_hi);
+#pragma unroll
+    for (int ks = 0; ks < C::NKS; ++ks) {
+      u32x4_t raw = {0u, 0u, 0u, 0u};
+      if (valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
+      u32x4_t sc;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
+                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
+      qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
+    }
+  }
+  const bool w_any = w_row_lo < si.rows;
+  const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;
+  const int w_act_hi = min(range_hi - 1, w_pos_hi);  // last key this wavefront's rows can see
+
+  f32x4_t o_acc[MRT][C::CB];
+  f32x4_t l_acc[MRT];
+  // Softmax reference point m per row, kept as the exp2 offset -m log2(e) (0 while the row has seen no key) and as
+  // the threshold for exp2 arguments: kLazy log2(e) once there is a reference point, -inf before.
+  float m_thr[MRT], m_neg[MRT];
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    m_thr[m] = -INFINITY;
+    m_neg[m] = 0.f;
+    l_acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int c = 0; c < C::CB; ++c) o_acc[m][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  }
+
+  // ---- cooperative fetch (as in rpa_prefill.h): one wave-wide direct-to-LDS load moves 4 rows; wavefront w moves
+  // rows [16 w, 16 w + 16) of the K tile and of the V tile.
+  const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * hd) * 2u;
+  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
+  const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
+      reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
+  const int l_row = lane / C::PR, l_slot = lane % C::PR;
+  const int v_row = (lane >> 1) % C::RB;
+  const uint32_t v_src = 16u * static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1));  // byte offset in the row
+  uint32_t pre_off[C::HB];
+#pragma unroll
+  for (int n = 0; n < C::HB; ++n) {
+    const int t_local = C::GROUP * wave + C::RB * n + l_row;
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ C::swz(t_local));
+  }
+  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + hd * 2;
+  const bool group_in_page = p.page_size >= C::GROUP;
+  auto fetch_tile = [&](int tile, int buf) {
+    const int t_first = tile + C::GROUP * wave;
+    char* dst = lds + 2 * buf * C::TILE_B + C::HB * wave * 1024;
+    if (group_in_page && t_first + C::GROUP - 1 <= t_last) {
+      const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
+      const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+      const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(sbase), 0, 0x7fffffff, 0x00020000);
+#pragma unroll
+      for (int n = 0; n < C::HB; ++n) {
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + n * 1024), 16,
+                                                 pre_off[n], 0, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024),
+                                                 16, v_pre_off + n * C::RB * stride_b, 0, 0, 0);
+      }
+      return;
+    }
+    // last tile of the range or small pages: per block, keys past the range repeat the last one (masked)
+#pragma unroll
+    for (int n = 0; n < C::HB; ++n) {
+      const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
+      const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
+      const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
+                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+      const int tok = min(t_c + l_row, t_last);
+      const int t_local = C::GROUP * wave + C::RB * n + l_row;
+      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * static_cast<uint32_t>(l_slot ^ C::swz(t_local));
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
+                                       (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
+      const int v_tok = min(t_c + v_row, t_last);
+      __builtin_amdgcn_global_load_lds(
+          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_src + hd * 2),
+          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+    }
+  };
+  // Wait until at most `tiles_ahead` later tiles of this wavefront's loads are outstanding (they complete in order).
+  auto wait_fetch = [&](int tiles_ahead) {
+    static_assert(C::LOADS == 8 && C::NSTG >= 3 && C::NSTG <= 4, "extend the immediates below");
+    switch (tiles_ahead) {
+      case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;   // vmcnt(0)
+      case 1: __builtin_amdgcn_s_waitcnt(0x0F78); break;   // vmcnt(8)
+      default: __builtin_amdgcn_s_waitcnt(0x4F70); break;  // vmcnt(16)
+    }
+  };
+
+  if (range_hi > range_lo) {
+    const int n_tiles = (range_hi - range_lo + C::TK - 1) / C::TK;
+    // halves this wavefront computes: [0, hb); a half starts at range_lo + 32 * index
+    const int hb = __builtin_amdgcn_readfirstlane(
+        w_any && w_act_hi >= range_lo ? min(2 * n_tiles, ((w_act_hi - range_lo) >> 5) + 1) : 0);
+
+    PipeIo R;
+    const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));  // LDS pointers are 32-bit offsets
+    // LDS addresses of the operand reads in stage 0: K per k-step; V^T, with the transposing read: in each group of 16
+    // lanes, lanes 4e..4e+3 point at 16 consecutive elements of key e of a 4-key block (see rpa_prefill.h)
+#pragma unroll
+    for (int ks = 0; ks < C::NKS; ++ks) R.kbase[ks] = lds_base + i * C::ROWB + 16 * ((4 * ks + g) ^ C::swz(i));
+    const int v_key = 4 * g + (i >> 2);
+    R.misc[0] = lds_base + C::TILE_B + (v_key / C::RB) * 1024 + (v_key % C::RB) * 32 + 8 * (i & 3);
+    // fetch: the lane's row in a 4-row block and its 16-byte piece, K (swizzled by the row in the tile) and V
+    R.misc[1] = l_row;
+    R.misc[2] = v_row;
+    R.misc[3] = static_cast<int>(v_src) + hd * 2;
+#pragma unroll
+    for (int n = 0; n < C::HB; ++n) R.kpiece[n] = 16 * (l_slot ^ C::swz(C::RB * n + l_row));
+    // Per-lane bounds of the keys row tile m may see (none for a row past the end: an unreachable first key)
+#pragma unroll
+    for (int m = 0; m < MRT; ++m) {
+      const int hi = min(pos_n[m], range_hi - 1);
+      const int lo = max(W > 0 ? pos_n[m] - W + 1 : -0x40000000, si.start);
+      R.rowlo[m] = (hi < lo ? 0x40000000 : lo) - 4 * g;
+      R.mspan[m] = max(hi - lo, 0);
+    }
+    R.cfac = sf_log2e;
+#pragma unroll
+    for (int m = 0; m < MRT; ++m)
+#pragma unroll
+      for (int ks = 0; ks < C::NKS; ++ks)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float f = __uint_as_float(__builtin_bit_cast(u32x4_t, qreg[m][ks])[e]);
+          if (m < 2) R.q0[4 * (4 * m + ks) + e] = f;
+          else R.q1[4 * (4 * (m - 2) + ks) + e] = f;
+        }
+    const uint64_t bt_addr = reinterpret_cast<uint64_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq);
+    const uint64_t kv_addr = reinterpret_cast<uint64_t>(kvb) + static_cast<uint64_t>(2 * j * hd * 2);
+    auto sgpr = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+    R.s0 = i32x8_t{hb, sgpr(n_tiles), sgpr(range_lo), sgpr(all_lo), sgpr(all_hi), sgpr(t_last), 16 * wave,
+                   sgpr(lds_base) + C::HB * wave * 1024};
+    R.s1 = i32x8_t{sgpr(static_cast<int>(bt_addr)), sgpr(static_cast<int>(bt_addr >> 32)), sgpr(static_cast<int>(kv_addr)),
+                   sgpr(static_cast<int>(kv_addr >> 32)), sgpr(static_cast<int>(stride_b)), sgpr(static_cast<int>(page_b)),
+                   sgpr(a.page_shift), sgpr(p.num_pages - 1)};
+
+    __syncthreads();  // every wavefront has left the previous item's tiles
+    for (int t = 0; t < min(C::NSTG - 1, n_tiles); ++t) fetch_tile(range_lo + t * C::TK, t);
+    wait_fetch(min(n_tiles - 1, C::NSTG - 2));
+    __syncthreads();  // publishes tile 0
+    pipe_key_loop<kMimic && C::ROUND>(R);
+#pragma unroll
+    for (int m = 0; m < MRT; ++m) {
+      l_acc[m][0] = R.l[4 * m];
+      m_neg[m] = R.mneg[m];
+      m_thr[m] = R.mthr[m];
+#pragma unroll
+      for (int c = 0; c < C::CB; ++c)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          o_acc[m][c][r] = (m == 0 ? R.o0 : m == 1 ? R.o1 : m == 2 ? R.o2 : R.o3)[4 * c + r];
+    }
+  }
+
+  // ---- normalise (with optional sinks) and store
+#pragma unroll
+  for (int m = 0; m < MRT; ++m) {
+    bool valid;
+    int head;
+    size_t q_off;
+    int opaque0 = 0;
+    asm volatile("" : "+v"(opaque0));
+    row_of(m, opaque0, valid, head, q_off);
+    if (!valid) continue;
+    const float l_run = l_acc[m][0];
+    const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+    float num_scale = 1.f, denom = l_run;
+    if (p.sinks != nullptr && p.num_sinks > 0) {
+      const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
+      float smax = -INFINITY;
+      for (int k = 0; k < p.num_sinks; ++k) smax = fmaxf(smax, sk[k]);
+      const float mt = fmaxf(m_row, smax);
+      float ssum = 0.f;
+      for (int k = 0; k < p.num_sinks; ++k) ssum += expf(sk[k] - mt);
+      num_scale = m_row == -INFINITY ? 0.f : expf(m_row - mt);
+      denom = num_scale * l_run + ssum;
+    }
+    const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
+    bf16_t* orow = out + q_off;
+    // MFMA c holds head_dim elements 16 c + 4 g + r of this lane's row
+#pragma unroll
+    for (int c = 0; c < C::CB; ++c) {
+      u32x2_t w;
+      w[0] = pack_bf16x2(o_acc[m][c][0] * inv, o_acc[m][c][1] * inv);
+      w[1] = pack_bf16x2(o_acc[m][c][2] * inv, o_acc[m][c][3] * inv);
+      *reinterpret_cast<u32x2_t*>(orow + 16 * c + 4 * g) = w;
+    }
+  }
+}
+
+}  // namespace rpa

@@ -29,6 +29,7 @@
 
 #include "rpa_decode.h"
 #include "rpa_prefill.h"
+#include "rpa_prefill_pipe.h"
 
 namespace rpa {
 
@@ -52,8 +53,22 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 // for every batch, slow for large prefill batches).  That leaves the decode loop a register allocation of its own, about
 // 2 % faster on decode batches, and spreads short prefill chunks over more wavefronts, which is why the host picks
 // this instantiation for small batches; it is also the one that merges an attention state in a.pre into every row.
+// Prefill tiles of the instantiation: four row tiles per wavefront at head_dim 128 select the software-pipelined tile
+// of rpa_prefill_pipe.h, which runs one workgroup per compute unit (one wavefront per SIMD, up to 512 registers).
+template <int D, int MRT>
+constexpr bool kPipeTile = D == 128 && MRT == 4;
+template <int D, int MRT>
+constexpr int kWavesPerSimd = kPipeTile<D, MRT> ? 1 : 2;
+
+template <int D, int MRT, bool kMimic>
+__device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt) {
+  if constexpr (kPipeTile<D, MRT>) prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
+  else prefill_tile<D, MRT, kMimic>(a, lds, si, s, j, qt);
+}
+
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
-__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2))) void rpa_tile_kernel(TileArgs a) {
+__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D, MRT>, kWavesPerSimd<D, MRT>)))
+void rpa_tile_kernel(TileArgs a) {
   constexpr int DD = D < 128 ? 128 : D;  // head_dim 64: the wave-level loop works 128 wide, prefill tiles 64 wide
   using C = Cfg<DD, NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -288,7 +303,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
           const int local = w - s_base;
           const int j = local / n_qt, member = local - j * n_qt;
-          prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, n_qt - 1 - member);
+          run_prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, n_qt - 1 - member);
         }
         if (tid == 0) {
           const uint32_t done = __hip_atomic_fetch_add(&qctr[8], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -310,7 +325,7 @@ __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(2, 2
           const int j = local / n_qt, member = local - j * n_qt;
           const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
           const int qt = (member + 5 * round0) % n_qt;
-          prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
+          run_prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
         }
       }
       // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
@@ -397,6 +412,8 @@ struct Tune {
   int no_mimic;            // RPA_TUNE_NO_MIMIC
   int no_wave_only;        // RPA_TUNE_NO_WAVE_ONLY
   int wave_only_rows;      // RPA_TUNE_WAVE_ONLY_ROWS
+  int pipe;                // RPA_TUNE_PIPE: 0 = never use the software-pipelined prefill tile (head_dim 128)
+  int pipe_stream_wgs;     // RPA_TUNE_PIPE_STREAM_WGS: workgroups (of one per compute unit) that take the decode stream first
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -413,6 +430,8 @@ static const Tune& tune() {
     x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
     x.no_wave_only = env_int("RPA_TUNE_NO_WAVE_ONLY", 0);
     x.wave_only_rows = env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows);
+    x.pipe = env_int("RPA_TUNE_PIPE", 0);
+    x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
     return x;
   }();
   return t;
@@ -450,7 +469,8 @@ template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv =
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<(D < 128 ? 128 : D), NT, kMimic>;
   using PC = PCfg<D, MRT>;
-  const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE, static_cast<size_t>(PC::LDS));
+  const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE,
+                          static_cast<size_t>(kPipeTile<D, MRT> ? PipeCfg::LDS : PC::LDS));
   const size_t lds = sched_bytes((a.p.max_num_seqs + (1 << a.sched_shift) - 1) >> a.sched_shift) + data;
   // More than 64 KiB of dynamic LDS has to be allowed once per kernel (and device); the call is idempotent.
   static std::atomic<uint64_t> allowed[64];
@@ -532,8 +552,21 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   }
   if (p.head_dim == 64)
     return mimic ? launch_cfg<64, 2, 4, true>(a, grid, stream) : launch_cfg<64, 2, 4, false>(a, grid, stream);
-  if (p.head_dim <= 128)
+  if (p.head_dim <= 128) {
+    // The software-pipelined tile fetches 16 keys per page look-up, has no soft cap and folds a positive logit scale
+    // into the exp2 argument; everything else takes the plain tile.
+    const bool pipe_ok = p.page_size >= 16 && p.logits_soft_cap == 0.f &&
+                         (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
+    if (tune().pipe != 0 && pipe_ok) {
+      // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
+      // number on every XCD) take the decode stream first and join the prefill queues when it is done
+      const int g1 = device_cu_count();
+      a.stream_grid = g1;
+      a.decode_grid = max(0, g1 - tune().pipe_stream_wgs);
+      return mimic ? launch_cfg<128, 2, 4, true>(a, g1, stream) : launch_cfg<128, 2, 4, false>(a, g1, stream);
+    }
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
+  }
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);
 }
 
