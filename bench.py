@@ -22,12 +22,20 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
-# HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter passes (scaled by a plain 1 GiB device copy); a
-# workload without a counter run reports null.
-MEASURED_TRAFFIC_BYTES = {
-    "decode_llama3_8b": (2184963 * 2.0 + 18447 * 1.0) * 1024,
-    "mixed_prefill_decode": (2148880 * 2.0 + 85691 * 1.0) * 1024,
-}
+# HBM bytes per launch as the FETCH_SIZE / WRITE_SIZE counter passes measured them (each counter scaled by what it reads
+# for a plain device copy of known size): profiles/hbm_traffic.json, written by `python -m ejkernel_amd.hbm_traffic`
+# from the counter files of a profile run.  A workload without an entry reports null.
+def measured_traffic_bytes(workload: str):
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            entry = json.load(f).get(workload)
+        return None if entry is None else float(entry["bytes"])
+    except (OSError, ValueError, KeyError):
+        return None
+
+
+# The configurations of the benchmark besides the headline one, measured in the same run (entries of "configs").
+EXTRA_CONFIGS = ["decode_small", "mixed_prefill_decode", "mixed_prefill_only", "gemma2_local", "decode_long_context"]
 
 
 def parse():
@@ -52,6 +60,8 @@ def parse():
     ap.add_argument("--cpu-seqs", type=int, default=0, help="sequences in the CPU sample (0 = pick for ~10-30 s)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-parity", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="only the headline workload: skip the other benchmark configurations (the \"configs\" array)")
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB MiB --steps times (a kernel of "
                          "known traffic, used to scale the FETCH_SIZE / WRITE_SIZE counters)")
@@ -289,6 +299,95 @@ def page_attention_main(args):
     print(json.dumps(line))
 
 
+def time_steps(step, steps, warmup):
+    """`warmup` untimed calls, then `steps` calls bracketed by synchronisation: wall time per step, the per-call
+    durations between HIP events on the stream the op launches on (torch's current one), and the last output."""
+    import torch
+
+    out = None
+    for _ in range(warmup):
+        out = step()
+    torch.cuda.synchronize()
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(steps)]
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        starts[i].record()
+        out = step()
+        ends[i].record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall * 1e3 / steps, sorted(s.elapsed_time(e) for s, e in zip(starts, ends)), out
+
+
+def roofline_of(counts, ev_ms):
+    """The roofline object of a workload: the bound its algorithmic bytes and flops put it under at MI355X's peaks,
+    priced with the average kernel duration."""
+    from ejkernel_amd.roofline import HBM_PEAK_GBPS, MFMA_BF16_PEAK_TFLOPS
+
+    kernel_ms = sum(ev_ms) / len(ev_ms)
+    gbps = counts["bytes"] / (kernel_ms * 1e-3) / 1e9
+    tflops = counts["flops"] / (kernel_ms * 1e-3) / 1e12
+    if counts["bytes"] / (HBM_PEAK_GBPS * 1e9) >= counts["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12):
+        roof = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS}
+    else:
+        roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
+    roof.update({"traffic": None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
+                 "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
+                 "algorithmic_flops": counts["flops"], "tflops": tflops, "gbps": gbps})
+    return roof
+
+
+def measure_config(name, steps, warmup, want_parity):
+    """One entry of "configs": the named workload at full size, timed like the headline one and checked against the
+    CPU restatement on a small sample of its sequences."""
+    import torch
+
+    from ejkernel_amd.modules import ragged_page_attention
+    from ejkernel_amd.roofline import algorithmic_counts
+    from ejkernel_amd.workloads import make_workload
+
+    batch = make_workload(name, device="cuda:0")
+    m = batch.meta
+    counts = algorithmic_counts(batch.q_lens, batch.kv_lens, num_q_heads=m["num_q_heads"], num_kv_heads=m["num_kv_heads"],
+                                head_dim=m["head_dim"], page_size=m["page_size"], sliding_window=batch.sliding_window)
+
+    def step():
+        return ragged_page_attention(*batch.args(), **batch.kwargs())
+
+    ms_per_step, ev_ms, out = time_steps(step, steps, warmup)
+    roof = roofline_of(counts, ev_ms)
+    roof["traffic"] = measured_traffic_bytes(name)
+    entry = {"workload": name, "ms_per_step": ms_per_step, "kernel_ms_avg": roof["kernel_ms_avg"],
+             "tokens_per_s": counts["tokens"] / (ms_per_step * 1e-3), "roofline": roof,
+             "host_overhead_ms": ms_per_step - roof["kernel_ms_avg"]}
+    if name == "decode_small":
+        # the launch-bound configuration: the same call replayed from a HIP graph, where no host code runs per step
+        g = torch.cuda.CUDAGraph()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step()
+            side.synchronize()
+            with torch.cuda.graph(g, stream=side):
+                step()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        reps = max(steps, 50)
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            g.replay()
+        torch.cuda.synchronize()
+        entry["graph_replay_ms"] = (time.perf_counter() - t0) * 1e3 / reps
+    if want_parity:
+        entry["parity"] = cpu_sample_and_parity(batch, out, False, True, 0, budget_s=2.0)["parity"]
+    del batch, out
+    torch.cuda.empty_cache()
+    return entry
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -345,36 +444,12 @@ def main():
             return ragged_page_attention_v3(*v3.args(), **v3.kwargs())[0]
         return ragged_page_attention(*batch.args(), **batch.kwargs())
 
-    for _ in range(args.warmup):
-        out = step()
-    torch.cuda.synchronize()
-    starts = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    ends = [torch.cuda.Event(enable_timing=True) for _ in range(args.steps)]
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        starts[i].record()  # the op launches on torch's current stream, the one these events are recorded on
-        out = step()
-        ends[i].record()
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-    ev_ms = sorted(s.elapsed_time(e) for s, e in zip(starts, ends))
+    ms_per_step, ev_ms, out = time_steps(step, args.steps, args.warmup)
     kernel_ms = sum(ev_ms) / len(ev_ms)
-    ms_per_step = wall * 1e3 / args.steps
     tokens = counts["tokens"]
-
-    gbps = counts["bytes"] / (kernel_ms * 1e-3) / 1e9
-    tflops = counts["flops"] / (kernel_ms * 1e-3) / 1e12
-    hbm_time = counts["bytes"] / (HBM_PEAK_GBPS * 1e9)
-    mfma_time = counts["flops"] / (MFMA_BF16_PEAK_TFLOPS * 1e12)
-    if hbm_time >= mfma_time:
-        roof = {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": gbps / HBM_PEAK_GBPS}
-    else:
-        roof = {"bound": "mfma", "achieved": tflops, "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": tflops / MFMA_BF16_PEAK_TFLOPS}
-    roof.update({"traffic": MEASURED_TRAFFIC_BYTES.get(args.workload) if args.scale == 1.0 and v3 is None else None, "kernel_ms_avg": kernel_ms, "kernel_ms_min": ev_ms[0],
-                 "kernel_ms_median": ev_ms[len(ev_ms) // 2], "algorithmic_bytes": counts["bytes"],
-                 "algorithmic_flops": counts["flops"], "tflops": tflops, "gbps": gbps})
+    roof = roofline_of(counts, ev_ms)
+    roof["traffic"] = measured_traffic_bytes(args.workload) if args.scale == 1.0 and v3 is None else None
+    gbps, tflops = roof["gbps"], roof["tflops"]
 
     line = {
         "metric": "ragged paged-attn tokens/s" if v3 is None else "ragged paged-attn v3 (cache update + attention) tokens/s", "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
@@ -393,6 +468,10 @@ def main():
             # which only differ at the positions it overwrites itself.
             line.update(cpu_sample_and_parity_v3(batch, v3, out, not args.no_cpu_baseline, not args.no_parity,
                                                  args.cpu_seqs))
+    if (not args.no_configs and args.workload == "decode_llama3_8b" and args.op == "rpa" and args.scale == 1.0):
+        del batch, out
+        torch.cuda.empty_cache()
+        line["configs"] = [measure_config(name, args.steps, args.warmup, not args.no_parity) for name in EXTRA_CONFIGS]
     print(json.dumps(line))
 
 

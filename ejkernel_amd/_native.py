@@ -19,6 +19,8 @@ RPA_COMPUTE_BF16, RPA_COMPUTE_F32 = 0, 1
 RPA_FLAG_FORCE_GENERIC = 1
 RPA_FLAG_FP32_LOGITS = 2
 RPA_FLAG_PREFILL_TILES = 4
+RPA_FLAG_PIPE_TILES = 8
+RPA_FLAG_PLAIN_TILES = 16
 
 EXPORTED_SYMBOLS = (
     "rpa_abi_version",

@@ -24,7 +24,7 @@ Register map (one wavefront):
   v[160:163]  visible keys of the lane's rows minus one (0 with an unreachable first key: none)   (in)
   v[164:167]  LDS address of the K operand reads per k-step (stage of the next tile);  v168  of the V^T reads
   v169        factor of the exp2 argument: log2(e) times the fp32 logit scale                     (in)
-  v170, v195:199  temporaries;  v171  -inf
+  v170, v195:199  temporaries;  v171  -inf;  v[200:215]  fetch: byte offsets of the lane's pieces
   v[172:175]  threshold of the exp2 arguments per row tile: -inf before a row's first key         (out)
   v176        the threshold once a row has a reference point
   v[178:181]  first visible key of the lane's rows minus 4 g (absolute)                           (in)
@@ -46,7 +46,7 @@ import os
 MRT, NKS, CB = 4, 4, 8
 ROWB = 256
 STAGE_B = 32768   # K tile + V tile
-NSTG = 3
+NSTG = 4
 LAZY_LOG2E = 16.0 * 1.4426950408889634
 
 O = lambda m, c: f"a[{32 * m + 4 * c}:{32 * m + 4 * c + 3}]"
@@ -78,6 +78,15 @@ LROW, VROW, VPIECE = "v187", "v188", "v189"
 KPIECE = lambda n: f"v{190 + n}"
 T1, T2, T3, T4, T5 = "v195", "v196", "v197", "v198", "v199"
 MFMA = "v_mfma_f32_16x16x32_bf16"
+PROF = os.environ.get("RPA_PPA_PROF", "") != ""   # experiment: cycle counts of the loop's regions in s[76:83]
+
+
+def stamp(k: int) -> list[str]:
+    """Experiment builds: s[84:85] = now; region k (0..7) gets the cycles since the previous stamp."""
+    if not PROF:
+        return []
+    return ["s_memtime s[84:85]", "s_waitcnt lgkmcnt(0)", f"s_sub_u32 s86, s84, s87", f"s_add_u32 s{76 + k}, s{76 + k}, s86", "s_mov_b32 s87, s84"]
+
 
 # scalar inputs
 S_HB, S_NT, S_RLO, S_ALLLO, S_ALLHI, S_TLAST, S_WAVE16, S_LDSW = (f"s{36 + k}" for k in range(8))
@@ -90,6 +99,8 @@ S_X0, S_X1, S_X2, S_X3, S_X4, S_X5 = "s64", "s65", "s66", "s67", "s68", "s69"
 S_P = "s[70:71]"
 S_PMASK = "s72"
 S_TT = "s73"
+S_PG, S_TB, S_D, S_LIM = "s89", "s90", "s91", "s92"   # a prepared fetch: page, base key, offset of the group, last row
+S_PEND, S_SITE = "s74", "s75"   # fetch of the tile in S_TT pending (this wavefront's site number, or 0); site number
 
 
 def kload(h: int) -> list[str]:
@@ -109,19 +120,23 @@ def qk(n: int, nxt: int) -> str:
     return f"{MFMA} {SQ(nxt, m, u)}, {KOP(u, ks)}, {QOP(m, ks)}, {c}"
 
 
-def sm1_pair(cur: int, m: int, e: int, mask: bool, rnd: bool) -> list[str]:
-    """Elements e, e + 1 of row tile m: logit -> exp2 argument in place, running maximum."""
+def sm1_pair(cur: int, m: int, e: int, mask: bool, rnd: bool) -> tuple[list[str], list[str]]:
+    """Elements e, e + 1 of row tile m: logit -> exp2 argument in place, running maximum.  Two groups of
+    instructions, for the two MFMA slots of the pair: an MFMA occupies the matrix pipe for 16 cycles and the issue port
+    for about 8, so three vector instructions behind every MFMA cost nothing, six behind every other one do."""
     u, r = e >> 2, e & 3
     x0, x1 = SE(cur, m, u, r), SE(cur, m, u, r + 1)
-    out = []
+    first, second = [], []
     if mask:
         for x, cst in ((x0, 16 * u + r), (x1, 16 * u + r + 1)):
-            out += [f"v_sub_u32 {T0}, {cst}, {MLO(m)}", f"v_cmp_le_u32 vcc, {T0}, {MSPAN(m)}", f"v_cndmask_b32 {x}, {NINF}, {x}, vcc"]
+            first += [f"v_sub_u32 {T0}, {cst}, {MLO(m)}", f"v_cmp_le_u32 vcc, {T0}, {MSPAN(m)}", f"v_cndmask_b32 {x}, {NINF}, {x}, vcc"]
     if rnd:
-        out += [f"v_cvt_pk_bf16_f32 {T0}, {x0}, {x1}", f"v_lshlrev_b32 {x0}, 16, {T0}", f"v_and_b32 {x1}, 0xffff0000, {T0}"]
-    out += [f"v_fma_f32 {x0}, {x0}, {CFAC}, {MNEG(m)}", f"v_fma_f32 {x1}, {x1}, {CFAC}, {MNEG(m)}"]
-    out += [f"v_max_f32 {TMAX(m)}, {x0}, {x1}" if e == 0 else f"v_max3_f32 {TMAX(m)}, {TMAX(m)}, {x0}, {x1}"]
-    return out
+        first += [f"v_cvt_pk_bf16_f32 {T0}, {x0}, {x1}", f"v_lshlrev_b32 {x0}, 16, {T0}", f"v_and_b32 {x1}, 0xffff0000, {T0}"]
+    second += [f"v_fma_f32 {x0}, {x0}, {CFAC}, {MNEG(m)}", f"v_fma_f32 {x1}, {x1}, {CFAC}, {MNEG(m)}"]
+    second += [f"v_max_f32 {TMAX(m)}, {x0}, {x1}" if e == 0 else f"v_max3_f32 {TMAX(m)}, {TMAX(m)}, {x0}, {x1}"]
+    if not first:  # nothing to round or mask: one instruction group, split evenly
+        first, second = second[:2], second[2:]
+    return first, second
 
 
 def block_a(h: int, mask: bool, rnd: bool) -> list[str]:
@@ -132,8 +147,7 @@ def block_a(h: int, mask: bool, rnd: bool) -> list[str]:
         out += [f"v_subrev_u32 {MLO(m)}, {S_A0}, {ROWLO(m)}" for m in range(MRT)]
     for n in range(32):
         out.append(qk(n, nxt))
-        if n % 2 == 0:
-            out += sm1_pair(cur, n >> 3, n & 7, mask, rnd)
+        out += sm1_pair(cur, n >> 3, (n & 7) & ~1, mask, rnd)[n & 1]
     return out
 
 
@@ -148,29 +162,32 @@ def sm2_pack(cur: int, m: int, k: int) -> list[str]:
 
 
 def sm2_tile(cur: int, m: int) -> list[list[str]]:
-    """P of row tile m = exp2 of its eight arguments, packed to bf16, in four groups of instructions.  The result of
-    a transcendental instruction may not be read by the very next instruction (the hardware does not wait), so the
-    pack of a pair follows the next pair's exponentials."""
-    return [sm2_exp(cur, m, 0), sm2_exp(cur, m, 1) + sm2_pack(cur, m, 0), sm2_exp(cur, m, 2) + sm2_pack(cur, m, 1),
-            sm2_exp(cur, m, 3) + sm2_pack(cur, m, 2) + ["s_nop 0"] + sm2_pack(cur, m, 3)]
+    """P of row tile m = exp2 of its eight arguments, packed to bf16, as nine groups of instructions for the gaps
+    behind the nine MFMAs of the row tile before it.  The result of a transcendental instruction may not be read by
+    the very next instruction (the hardware does not wait), and a register written by a vector instruction may not be
+    read by an MFMA within two wait states: the pack of a pair follows the first exponential of the next pair, and
+    the last pack is followed by two idle states."""
+    e = [sm2_exp(cur, m, k) for k in range(4)]
+    p = [sm2_pack(cur, m, k) for k in range(4)]
+    return [[e[0][0]], [e[0][1]], [e[1][0]] + p[0], [e[1][1]], [e[2][0]] + p[1], [e[2][1]], [e[3][0]] + p[2], [e[3][1]],
+            p[3] + ["s_nop 1"]]
 
 
 def block_b(h: int) -> list[str]:
-    """[SM2 | PV]: the exponentials of row tile m + 1 under the 9 MFMAs of row tile m."""
+    """[SM2 | PV]: the exponentials of row tile m + 1 in the gaps behind the 9 MFMAs of row tile m."""
     cur = 0 if h == 0 else 32
     out = kload(h) + ["s_waitcnt lgkmcnt(8)"]
-    for grp in sm2_tile(cur, 0):
+    first = sm2_tile(cur, 0)
+    first[8] = ["s_nop 0"] + first[8]  # no MFMA between the last exponential and the pack that reads it
+    for grp in first:
         out += grp
-    out.append("s_nop 1")
     for m in range(MRT):
+        nxt = sm2_tile(cur, m + 1) if m + 1 < MRT else [[] for _ in range(9)]
         out.append(f"{MFMA} {L(m)}, {ONES}, {PW(m)}, {L(m)}")
-        nxt = sm2_tile(cur, m + 1) if m + 1 < MRT else None
+        out += nxt[0]
         for c in range(CB):
             out.append(f"{MFMA} {O(m, c)}, {VRAW(c)}, {PW(m)}, {O(m, c)}")
-            # P of the next row tile, its last pack two MFMAs ahead of the MFMA that reads it (a vector write needs
-            # two wait states before an MFMA reads the register)
-            if nxt is not None and c in (0, 2, 4, 5):
-                out += nxt[(0, 2, 4, 5).index(c)]
+            out += nxt[c + 1]
     return out
 
 
@@ -178,9 +195,10 @@ def rescale(h: int, tag: str) -> list[str]:
     """Vote; where some row's exp2 argument exceeds its threshold (or the row sees its first key), move that row's
     reference point up by the row maximum: shift the exp2 arguments, scale row sum and outputs by exp2(-shift)."""
     cur = 0 if h == 0 else 32
-    out = [f"v_cmp_gt_f32 vcc, {TMAX(0)}, {MTHR(0)}"]
-    for m in range(1, MRT):
-        out += [f"v_cmp_gt_f32 {S_P}, {TMAX(m)}, {MTHR(m)}", f"s_or_b64 vcc, vcc, {S_P}"]
+    # (a row without a reference point has threshold -inf: the difference is +inf, or NaN when it has no key yet either,
+    # which the maxima drop)
+    out = [f"v_sub_f32 {tmp}, {TMAX(m)}, {MTHR(m)}" for m, tmp in enumerate((T1, T2, T3, T4))]
+    out += [f"v_max3_f32 {T1}, {T1}, {T2}, {T3}", f"v_max_f32 {T1}, {T1}, {T4}", f"v_cmp_lt_f32 vcc, 0, {T1}"]
     out.append(f"s_cbranch_vccz .Lpp_noresc_{tag}_%=")
     for m in range(MRT):
         x = TMAX(m)
@@ -209,56 +227,101 @@ def rescale(h: int, tag: str) -> list[str]:
     return out
 
 
+VO = [f"v{200 + k}" for k in range(8)]     # fetch: byte offsets of the lane's pieces in a group of 16 whole rows (4 K, 4 V blocks)
+VOX = [f"v{208 + k}" for k in range(8)]    # the same for a group that reaches past the last key
+
+
+def fetch_setup() -> list[str]:
+    """Per-lane byte offsets of a fetch whose 16 rows all exist (every tile but the last of a range)."""
+    out = []
+    for n in range(4):
+        out += [f"v_add_u32 {T3}, {4 * n}, {LROW}", f"v_mad_u32_u24 {VO[n]}, {T3}, {S_STRIDE}, {KPIECE(n)}",
+                f"v_add_u32 {T3}, {4 * n}, {VROW}", f"v_mad_u32_u24 {VO[4 + n]}, {T3}, {S_STRIDE}, {VPIECE}"]
+    return out
+
+
+def fetch_prepare() -> list[str]:
+    """For the tile whose first key is in S_TT: the group's base key, how far the group lies behind it, the last row
+    that exists; requests the page of the base key (the group's 16 keys share it: pages of at least 16 keys)."""
+    return [f"s_add_i32 {S_X0}, {S_TT}, {S_WAVE16}",            # first key of the group
+            f"s_and_b32 {S_TB}, {S_TLAST}, -16",
+            f"s_min_i32 {S_TB}, {S_TB}, {S_X0}",                 # base key: same page as every key fetched
+            f"s_sub_i32 {S_D}, {S_X0}, {S_TB}",
+            f"s_sub_i32 {S_LIM}, {S_TLAST}, {S_TB}",            # last row that exists, relative to the base
+            f"s_lshr_b32 {S_X4}, {S_TB}, {S_PSHIFT}", f"s_lshl_b32 {S_X4}, {S_X4}, 2",
+            f"s_add_u32 {S_X4}, {S_BTLO}, {S_X4}", f"s_addc_u32 {S_X5}, {S_BTHI}, 0",
+            f"s_load_dword {S_PG}, s[68:69], 0x0"]
+
+
 def fetch(tag: str) -> list[str]:
-    """This wavefront's part (16 K rows, 16 V rows) of the tile whose first key is in S_TT, into the stage at byte
-    offset S_FBUF.  Keys past the range repeat the last one; the 16 keys share a page (pages of at least 16 keys)."""
-    out = [f"s_add_i32 {S_X0}, {S_TT}, {S_WAVE16}",            # first key of the group
-           f"s_and_b32 {S_X1}, {S_TLAST}, -16",
-           f"s_min_i32 {S_X1}, {S_X1}, {S_X0}",                 # base key: same page as every key fetched
-           f"s_sub_i32 {S_X2}, {S_X0}, {S_X1}",                 # d
-           f"s_sub_i32 {S_X3}, {S_TLAST}, {S_X1}",              # last row that exists, relative to the base
-           f"s_lshr_b32 {S_X4}, {S_X1}, {S_PSHIFT}", f"s_lshl_b32 {S_X4}, {S_X4}, 2",
-           f"s_add_u32 {S_X4}, {S_BTLO}, {S_X4}", f"s_addc_u32 {S_X5}, {S_BTHI}, 0",
-           f"s_load_dword {S_X0}, s[68:69], 0x0",
-           f"v_add_u32 {T1}, {S_X2}, {LROW}", f"v_add_u32 {T2}, {S_X2}, {VROW}"]
-    vo = ["v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207"]
+    """This wavefront's part (16 K rows, 16 V rows) of the prepared tile into the stage at byte offset S_FBUF.  Keys
+    past the range repeat the last one."""
+    out = ["s_waitcnt lgkmcnt(0)",
+           f"s_max_i32 {S_X0}, {S_PG}, 0", f"s_min_i32 {S_X0}, {S_X0}, {S_NP1}",
+           f"s_mul_hi_u32 {S_X5}, {S_X0}, {S_PAGEB}", f"s_mul_i32 {S_X4}, {S_X0}, {S_PAGEB}",
+           f"s_and_b32 {S_X1}, {S_TB}, {S_PMASK}", f"s_mul_i32 {S_X1}, {S_X1}, {S_STRIDE}",
+           f"s_add_u32 {S_X4}, {S_X4}, {S_X1}", f"s_addc_u32 {S_X5}, {S_X5}, 0",
+           f"s_add_u32 {S_R0}, {S_X4}, {S_KVLO}", f"s_addc_u32 {S_R1}, {S_X5}, {S_KVHI}",
+           f"s_and_b32 {S_R1}, {S_R1}, 0xffff",
+           f"s_add_i32 {S_X0}, {S_LDSW}, {S_FBUF}",
+           f"s_cmp_lt_i32 {S_LIM}, 15", f"s_cbranch_scc1 .Lpp_fx_{tag}_%=",
+           f"s_cmp_lg_u32 {S_D}, 0", f"s_cbranch_scc1 .Lpp_fx_{tag}_%="]
+
+    def loads(vo):
+        o = []
+        for n in range(4):
+            o += [f"s_add_i32 m0, {S_X0}, {n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[n]}, {S_R}, 0 offen lds",
+                  f"s_add_i32 m0, {S_X0}, {16384 + n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[4 + n]}, {S_R}, 0 offen lds"]
+        return o
+
+    out += loads(VO) + [f"s_branch .Lpp_fd_{tag}_%=", f".Lpp_fx_{tag}_%=:"]
+    out += [f"v_add_u32 {T1}, {S_D}, {LROW}", f"v_add_u32 {T2}, {S_D}, {VROW}"]
     for n in range(4):
-        out += [f"v_add_u32 {T3}, {4 * n}, {T1}", f"v_min_i32 {T3}, {S_X3}, {T3}", f"v_mad_u32_u24 {vo[n]}, {T3}, {S_STRIDE}, {KPIECE(n)}",
-                f"v_add_u32 {T3}, {4 * n}, {T2}", f"v_min_i32 {T3}, {S_X3}, {T3}", f"v_mad_u32_u24 {vo[4 + n]}, {T3}, {S_STRIDE}, {VPIECE}"]
-    out += ["s_waitcnt lgkmcnt(0)",
-            f"s_max_i32 {S_X0}, {S_X0}, 0", f"s_min_i32 {S_X0}, {S_X0}, {S_NP1}",
-            f"s_mul_hi_u32 {S_X5}, {S_X0}, {S_PAGEB}", f"s_mul_i32 {S_X4}, {S_X0}, {S_PAGEB}",
-            f"s_and_b32 {S_X1}, {S_X1}, {S_PMASK}", f"s_mul_i32 {S_X1}, {S_X1}, {S_STRIDE}",
-            f"s_add_u32 {S_X4}, {S_X4}, {S_X1}", f"s_addc_u32 {S_X5}, {S_X5}, 0",
-            f"s_add_u32 {S_R0}, {S_X4}, {S_KVLO}", f"s_addc_u32 {S_R1}, {S_X5}, {S_KVHI}",
-            f"s_and_b32 {S_R1}, {S_R1}, 0xffff",
-            f"s_add_i32 {S_X0}, {S_LDSW}, {S_FBUF}"]
-    for n in range(4):
-        out += [f"s_add_i32 m0, {S_X0}, {n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[n]}, {S_R}, 0 offen lds",
-                f"s_add_i32 m0, {S_X0}, {16384 + n * 1024}", "s_nop 0", f"buffer_load_dwordx4 {vo[4 + n]}, {S_R}, 0 offen lds"]
+        out += [f"v_add_u32 {T3}, {4 * n}, {T1}", f"v_min_i32 {T3}, {S_LIM}, {T3}", f"v_mad_u32_u24 {VOX[n]}, {T3}, {S_STRIDE}, {KPIECE(n)}",
+                f"v_add_u32 {T3}, {4 * n}, {T2}", f"v_min_i32 {T3}, {S_LIM}, {T3}", f"v_mad_u32_u24 {VOX[4 + n]}, {T3}, {S_STRIDE}, {VPIECE}"]
+    out += loads(VOX) + [f".Lpp_fd_{tag}_%=:"]
     return out
 
 
 def publish(tag: str, t_reg: str) -> list[str]:
-    """Publishes tile t + 1 (this wavefront's part has landed; after the barrier everybody's) and refills the stage
-    of tile t - 1 with tile t + 2.  S_FBUF is the byte offset of that stage."""
-    return ["s_waitcnt vmcnt(0)", "s_barrier",
-            f"s_add_i32 {S_X0}, {t_reg}, 2", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_nofetch_{tag}_%=",
-            f"s_lshl_b32 {S_TT}, {S_X0}, 6", f"s_add_i32 {S_TT}, {S_TT}, {S_RLO}"] + fetch(tag) + [f".Lpp_nofetch_{tag}_%=:"]
+    """Publishes tile t + 1: this wavefront's part of it has landed (its loads complete in order; those of tile
+    t + 2 may still be in flight), after the barrier everybody's.  Every wavefront is then past its last read of
+    tile t - 1, whose stage (byte offset S_FBUF) takes tile t + NSTG - 1: the fetch is left pending for the wavefront's
+    site of the tile, so that the four wavefronts do not issue their loads at the same moment (a compute unit accepts
+    one 1-KiB load per 16 cycles or so, and a wavefront is held while its load waits)."""
+    return [f"s_add_i32 {S_X0}, {t_reg}, 2", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_w0_{tag}_%=",
+            "s_waitcnt vmcnt(8)", f"s_branch .Lpp_w1_{tag}_%=", f".Lpp_w0_{tag}_%=:", "s_waitcnt vmcnt(0)", f".Lpp_w1_{tag}_%=:"] + \
+        (stamp(6) if tag == "loop" else []) + ["s_barrier"] + (stamp(7) if tag == "loop" else []) + [
+            f"s_add_i32 {S_X0}, {t_reg}, {NSTG - 1}", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_nofetch_{tag}_%=",
+            f"s_lshl_b32 {S_TT}, {S_X0}, 6", f"s_add_i32 {S_TT}, {S_TT}, {S_RLO}", f"s_mov_b32 {S_PEND}, {S_SITE}"] + fetch_prepare() + [
+            f".Lpp_nofetch_{tag}_%=:"]
 
 
-def half(h: int, rnd: bool) -> list[str]:
+def site(k: int, tag: str) -> list[str]:
+    """Fetch site k of a tile (0: behind the barrier, 1: end of the first half, 2: middle of the second half, 3: end of
+    the tile): the wavefront whose site this is issues its pending fetch.  k < 0: whoever has one pending."""
+    test = [f"s_cmp_eq_u32 {S_PEND}, {k + 1}"] if k >= 0 else [f"s_cmp_lg_u32 {S_PEND}, 0"]
+    return test + [f"s_cbranch_scc0 .Lpp_nosite_{tag}_%="] + fetch(tag) + [f"s_mov_b32 {S_PEND}, 0", f".Lpp_nosite_{tag}_%=:"]
+
+
+def half(h: int, rnd: bool) -> tuple[list[str], list[str]]:
+    """One half; the second list is its masked block A, kept out of line behind the loop."""
     tag = f"h{h}"
     out = [f"s_cmp_gt_i32 {S_A0}, {S_ALLLO}", f"s_cbranch_scc0 .Lpp_mask_{tag}_%=",
            f"s_cmp_le_i32 {S_A0}, {S_ALLHI}", f"s_cbranch_scc0 .Lpp_mask_{tag}_%="]
-    out += block_a(h, False, rnd) + [f"s_branch .Lpp_adone_{tag}_%=", f".Lpp_mask_{tag}_%=:"] + block_a(h, True, rnd) + [f".Lpp_adone_{tag}_%=:"]
-    out += rescale(h, tag)
+    out += stamp(0)
+    out += block_a(h, False, rnd) + stamp(1) + [f".Lpp_adone_{tag}_%=:"]
+    cold = [f".Lpp_mask_{tag}_%=:"] + block_a(h, True, rnd) + stamp(2) + [f"s_branch .Lpp_adone_{tag}_%="]
+    out += rescale(h, tag) + stamp(3)
     if h == 0:
         out += [f"s_add_i32 {S_X0}, {S_T}, 1", f"s_cmp_ge_i32 {S_X0}, {S_NT}", f"s_cbranch_scc1 .Lpp_nopub_%="]
-        out += publish("loop", S_T) + [".Lpp_nopub_%=:"]
-    out += block_b(h)
+        out += publish("loop", S_T) + [".Lpp_nopub_%=:"] + site(0, "s0") + stamp(4)
+    else:
+        out += site(2, "s2")
+    out += block_b(h) + stamp(5)
+    out += site(1 if h == 0 else 3, "s1" if h == 0 else "s3")
     out += [f"s_add_i32 {S_HH}, {S_HH}, 1", f"s_add_i32 {S_A0}, {S_A0}, 32", f"s_cmp_eq_u32 {S_HH}, {S_HB}", "s_cbranch_scc1 .Lpp_done_%="]
-    return out
+    return out, cold
 
 
 def rotate_stages() -> list[str]:
@@ -272,6 +335,8 @@ def rotate_stages() -> list[str]:
 
 def loop(rnd: bool) -> list[str]:
     out = ["s_mov_b32 s58, m0"]  # the compiler's m0 is restored at the end
+    if PROF:
+        out += [f"s_mov_b32 s{76 + k}, 0" for k in range(8)] + ["s_memtime s[84:85]", "s_waitcnt lgkmcnt(0)", "s_mov_b32 s87, s84", "s_mov_b32 s88, s84"]
     # ---- set-up
     out += [f"v_accvgpr_write_b32 a{k}, 0" for k in range(144)]
     out += [f"v_mov_b32 {MNEG(m)}, 0" for m in range(MRT)] + [f"v_mov_b32 {NINF}, 0xff800000"]
@@ -280,7 +345,10 @@ def loop(rnd: bool) -> list[str]:
     out += [f"s_mov_b32 {S_R2}, 0x7fffffff", f"s_mov_b32 {S_R3}, 0x00020000",
             f"s_lshl_b32 {S_PMASK}, 1, {S_PSHIFT}", f"s_add_i32 {S_PMASK}, {S_PMASK}, -1",
             f"s_mov_b32 {S_HH}, 0", f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_A0}, {S_RLO}",
-            f"s_cmp_eq_u32 {S_HB}, 0", "s_cbranch_scc1 .Lpp_done_%="]
+            f"s_mov_b32 {S_PEND}, 0", f"s_lshr_b32 {S_SITE}, {S_WAVE16}, 4", f"s_add_i32 {S_SITE}, {S_SITE}, 1",
+            ]
+    out += fetch_setup()
+    out += [f"s_cmp_eq_u32 {S_HB}, 0", "s_cbranch_scc1 .Lpp_done_%="]
     # stage state as if tile -1 were in progress: the first rotation makes tile 0 current
     out += [f"s_mov_b32 {S_CUR}, {(NSTG - 1) * STAGE_B}", f"s_mov_b32 {S_NXT}, 0"]
     # logits of the first half, K operands of the second (both in tile 0, stage 0)
@@ -288,20 +356,24 @@ def loop(rnd: bool) -> list[str]:
     out += kload(0) + ["s_waitcnt lgkmcnt(0)"] + [qk(n, 0) for n in range(32)] + ["s_nop 7", "s_nop 7"] + kload(1)
     out.append(".Lpp_tile_%=:")
     out += rotate_stages()
-    out += half(0, rnd) + half(1, rnd)
+    h0, cold0 = half(0, rnd)
+    h1, cold1 = half(1, rnd)
+    out += h0 + h1
     out += [f"s_add_i32 {S_T}, {S_T}, 1", "s_branch .Lpp_tile_%="]
+    out += cold0 + cold1
     # ---- tiles past this wavefront's last half: it still takes part in their barriers and fetches
-    out += [".Lpp_done_%=:",
+    out += [".Lpp_done_%=:"] + site(-1, "sx") + [
             f"s_add_i32 {S_X5}, {S_HH}, 1", f"s_lshr_b32 {S_T}, {S_X5}, 1",
             # the stage to refill at tile t's barrier is that of tile t - 1
-            f"s_add_i32 {S_X0}, {S_T}, {NSTG - 1}", f"s_mul_hi_u32 {S_X1}, {S_X0}, 0xaaaaaaab", f"s_lshr_b32 {S_X1}, {S_X1}, 1",
-            f"s_mul_i32 {S_X1}, {S_X1}, {NSTG}", f"s_sub_i32 {S_X0}, {S_X0}, {S_X1}", f"s_mul_i32 {S_FBUF}, {S_X0}, {STAGE_B}",
+            f"s_add_i32 {S_X0}, {S_T}, {NSTG - 1}", f"s_and_b32 {S_X0}, {S_X0}, {NSTG - 1}", f"s_mul_i32 {S_FBUF}, {S_X0}, {STAGE_B}",
             ".Lpp_tail_%=:",
             f"s_add_i32 {S_X0}, {S_T}, 1", f"s_cmp_ge_i32 {S_X0}, {S_NT}", "s_cbranch_scc1 .Lpp_end_%="]
-    out += publish("tail", S_T)
+    out += publish("tail", S_T) + site(-1, "st")
     out += [f"s_add_i32 {S_T}, {S_T}, 1",
             f"s_add_i32 {S_FBUF}, {S_FBUF}, {STAGE_B}", f"s_cmp_eq_u32 {S_FBUF}, {NSTG * STAGE_B}", f"s_cselect_b32 {S_FBUF}, 0, {S_FBUF}",
             "s_branch .Lpp_tail_%=", ".Lpp_end_%=:", "s_waitcnt lgkmcnt(0)", "s_mov_b32 m0, s58", "s_nop 7", "s_nop 7"]
+    if PROF:
+        out += []
     return out
 
 

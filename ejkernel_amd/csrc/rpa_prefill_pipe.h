@@ -33,7 +33,7 @@
 namespace rpa {
 
 #ifndef RPA_PP_NSTG
-#define RPA_PP_NSTG 3
+#define RPA_PP_NSTG 4
 #endif
 #ifndef RPA_PP_ROUND
 #define RPA_PP_ROUND 1
@@ -81,7 +81,19 @@ struct PipeIo {
   i32x4_t misc;             // in: LDS address of the V^T reads, fetch: row in a K block, in a V block, V piece offset
   float cfac;               // in: factor of the exp2 argument
   i32x8_t s0, s1;           // in: scalars (see the register map)
+#ifdef RPA_PP_PROF
+  i32x8_t prof;
+#endif
 };
+
+// Experiment builds (-DRPA_PP_PROF, with an .inc file generated under RPA_PPA_PROF=1): cycle counts of the loop's regions.
+#ifdef RPA_PP_PROF
+#define RPA_PPA_PROF_OUT , "={s[76:83]}"(R.prof)
+#define RPA_PPA_PROF_CLOBBERS , "s84", "s85", "s86", "s87", "s88"
+#else
+#define RPA_PPA_PROF_OUT
+#define RPA_PPA_PROF_CLOBBERS
+#endif
 
 #define RPA_PPA_CLOBBERS                                                                                                  \
   "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17",    \
@@ -91,13 +103,13 @@ struct PipeIo {
   "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145",        \
   "v146", "v147", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v164", "v165", "v166", "v167",        \
   "v168", "v170", "v171", "v176", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204",        \
-  "v205", "v206", "v207", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154",        \
+  "v205", "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154",        \
   "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168",        \
   "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182",        \
   "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192", "a193", "a194", "a195", "a196",        \
   "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", "s52", "s53", "s54", "s55",    \
   "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", \
-  "s73", "vcc", "scc", "memory"
+  "s73", "s74", "s75", "s89", "s90", "s91", "s92", "vcc", "scc", "memory"
 
 // The key loop of one tile for one wavefront.  LDS stages 0 and 1 hold the first two K/V tiles (or the only one) and
 // have been published by a barrier; the stream runs every later barrier and fetch of the tile itself.
@@ -105,10 +117,10 @@ template <bool kRound>
 __device__ __forceinline__ void pipe_key_loop(PipeIo& R) {
 #define RPA_PPA_OPERANDS                                                                                                  \
   : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={a[128:143]}"(R.l),          \
-    "={v[148:151]}"(R.mneg), "={v[172:175]}"(R.mthr)                                                                   \
+    "={v[148:151]}"(R.mneg), "={v[172:175]}"(R.mthr) RPA_PPA_PROF_OUT                                                  \
   : "{v[64:95]}"(R.q0), "{v[96:127]}"(R.q1), "{v[160:163]}"(R.mspan), "{v[178:181]}"(R.rowlo), "{v[182:185]}"(R.kbase), \
     "{v[186:189]}"(R.misc), "{v[190:193]}"(R.kpiece), "{v169}"(R.cfac), "{s[36:43]}"(R.s0), "{s[44:51]}"(R.s1)         \
-  : RPA_PPA_CLOBBERS
+  : RPA_PPA_CLOBBERS RPA_PPA_PROF_CLOBBERS
   if constexpr (kRound) asm volatile(RPA_PPA_LOOP_ROUND RPA_PPA_OPERANDS);
   else asm volatile(RPA_PPA_LOOP_PLAIN RPA_PPA_OPERANDS);
 #undef RPA_PPA_OPERANDS
@@ -120,6 +132,10 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
   using C = PipeCfg;
   constexpr int MRT = C::MRT;
   const RpaParams& p = a.p;
+#ifdef RPA_PP_PROF2
+  const uint64_t pt0 = __builtin_readcyclecounter();
+  uint32_t prof2_loop = 0, prof2_halves = 0;
+#endif
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int i = lane & 15, g = lane >> 4;
@@ -318,7 +334,21 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     for (int t = 0; t < min(C::NSTG - 1, n_tiles); ++t) fetch_tile(range_lo + t * C::TK, t);
     wait_fetch(min(n_tiles - 1, C::NSTG - 2));
     __syncthreads();  // publishes tile 0
+#ifdef RPA_PP_PROF2
+    const uint64_t pl0 = __builtin_readcyclecounter();
+#endif
     pipe_key_loop<kMimic && C::ROUND>(R);
+#ifdef RPA_PP_PROF2
+    prof2_loop = static_cast<uint32_t>(__builtin_readcyclecounter() - pl0);
+    prof2_halves = hb;
+#endif
+#ifdef RPA_PP_PROF
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+      uint32_t* dst = reinterpret_cast<uint32_t*>(a.partial_o) + (blockIdx.x * kWgWaves + threadIdx.x / kWave) * 16;
+      for (int k = 0; k < 8; ++k) dst[k] += static_cast<uint32_t>(R.prof[k]);
+      dst[8] += 1;
+    }
+#endif
 #pragma unroll
     for (int m = 0; m < MRT; ++m) {
       l_acc[m][0] = R.l[4 * m];
@@ -366,6 +396,17 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
       *reinterpret_cast<u32x2_t*>(orow + 16 * c + 4 * g) = w;
     }
   }
+#ifdef RPA_PP_PROF2
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    uint32_t* dst = reinterpret_cast<uint32_t*>(a.partial_o) + (blockIdx.x * kWgWaves + threadIdx.x / kWave) * 16;
+    dst[0] += static_cast<uint32_t>(__builtin_readcyclecounter() - pt0);
+    dst[1] += prof2_loop;
+    dst[2] += prof2_halves;
+    dst[3] += 1;
+    if (dst[4] == 0) dst[4] = static_cast<uint32_t>(pt0);  // start of the first tile
+    dst[5] = static_cast<uint32_t>(__builtin_readcyclecounter());  // end of the last
+  }
+#endif
 }
 
 }  // namespace rpa

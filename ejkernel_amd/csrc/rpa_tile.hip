@@ -414,6 +414,7 @@ struct Tune {
   int wave_only_rows;      // RPA_TUNE_WAVE_ONLY_ROWS
   int pipe;                // RPA_TUNE_PIPE: 0 = never use the software-pipelined prefill tile (head_dim 128)
   int pipe_stream_wgs;     // RPA_TUNE_PIPE_STREAM_WGS: workgroups (of one per compute unit) that take the decode stream first
+  int pipe_min_tokens_per_seq;  // RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ: average query tokens per sequence from which it is used
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -430,7 +431,8 @@ static const Tune& tune() {
     x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
     x.no_wave_only = env_int("RPA_TUNE_NO_WAVE_ONLY", 0);
     x.wave_only_rows = env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows);
-    x.pipe = env_int("RPA_TUNE_PIPE", 0);
+    x.pipe = env_int("RPA_TUNE_PIPE", 1);
+    x.pipe_min_tokens_per_seq = max(1, env_int("RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ", 128));
     x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
     return x;
   }();
@@ -537,7 +539,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   // alone gets a register allocation without spills, and short prefill chunks spread over four times as many
   // wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
   const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
-  const bool small_batch = p.query_start_loc == nullptr || ((p.flags & RPA_FLAG_PREFILL_TILES) == 0 &&
+  const bool small_batch = p.query_start_loc == nullptr || ((p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) == 0 &&
                                                             rows <= tune().wave_only_rows);
   // Prefill tiles address the cache as [page][slot][2 * kv heads][head_dim]; any other layout (two caches, one
   // contiguous cache per sequence, rows padded beyond head_dim) runs through the wave-level loop alone.
@@ -553,11 +555,17 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   if (p.head_dim == 64)
     return mimic ? launch_cfg<64, 2, 4, true>(a, grid, stream) : launch_cfg<64, 2, 4, false>(a, grid, stream);
   if (p.head_dim <= 128) {
-    // The software-pipelined tile fetches 16 keys per page look-up, has no soft cap and folds a positive logit scale
-    // into the exp2 argument; everything else takes the plain tile.
+    // The software-pipelined tile (one workgroup per compute unit) fetches 16 keys per page look-up, has no soft cap
+    // and folds a positive logit scale into the exp2 argument.  It pays for batches of long chunks; a batch that mixes
+    // chunks with many decode sequences is bound by its decode stream, which needs a streaming workgroup on every
+    // compute unit beside the prefill tiles (two workgroups per unit: the plain tile).  The host cannot see the lengths,
+    // so it goes by the average number of query tokens per sequence.
     const bool pipe_ok = p.page_size >= 16 && p.logits_soft_cap == 0.f &&
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
-    if (tune().pipe != 0 && pipe_ok) {
+    const bool pipe_wanted = (p.flags & RPA_FLAG_PLAIN_TILES) == 0 &&
+                             ((p.flags & RPA_FLAG_PIPE_TILES) != 0 ||
+                              (tune().pipe != 0 && static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs));
+    if (pipe_wanted && pipe_ok) {
       // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
       // number on every XCD) take the decode stream first and join the prefill queues when it is done
       const int g1 = device_cu_count();

@@ -53,6 +53,10 @@ extern "C" {
 #define RPA_FLAG_PREFILL_TILES 4u /* long chunks run as 128-row workgroup tiles whatever the size of the batch (by   */
                                   /* default batches of up to 20480 (token, query head) rows run them as 16-row      */
                                   /* wave-level items, which fills the device better when the tiles would be few)    */
+#define RPA_FLAG_PIPE_TILES 8u    /* head_dim 128: prefill tiles of 256 rows, one workgroup per compute unit, key loop  */
+                                  /* software-pipelined (by default chosen for batches of long chunks: at least 128    */
+                                  /* query tokens per sequence on average); implies RPA_FLAG_PREFILL_TILES            */
+#define RPA_FLAG_PLAIN_TILES 16u  /* never those: prefill tiles of 128 rows, two workgroups per compute unit          */
 
 typedef struct RpaParams {
   /* ---- device buffers (argument names follow ragged_page_attention.py:540-547) ---- */

@@ -193,3 +193,31 @@ def test_no_cpu_fallback():
     b = _b()
     with pytest.raises(RuntimeError, match="no CPU implementation"):
         ragged_page_attention(*b.args())
+
+
+def test_generated_instruction_stream_is_up_to_date():
+    """csrc/rpa_prefill_pipe_asm.inc is what csrc/gen_prefill_pipe_asm.py writes (the key loop of the software-pipelined
+    prefill tile is generated; the committed file must not drift from its generator)."""
+    import importlib.util
+    from pathlib import Path
+
+    csrc = Path(_native.__file__).resolve().parent / "csrc"
+    spec = importlib.util.spec_from_file_location("gen_prefill_pipe_asm", csrc / "gen_prefill_pipe_asm.py")
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    assert not gen.PROF, "unset RPA_PPA_PROF for this test"
+    assert (csrc / "rpa_prefill_pipe_asm.inc").read_text() == gen.render()
+
+
+def test_hbm_traffic_file_is_well_formed():
+    """profiles/hbm_traffic.json (read by bench.py for roofline.traffic): bytes = scaled counters, per workload."""
+    import json
+    from pathlib import Path
+
+    from ejkernel_amd.workloads import WORKLOADS
+
+    data = json.loads((Path(_native.__file__).resolve().parent.parent / "profiles" / "hbm_traffic.json").read_text())
+    for name, e in data.items():
+        assert name in WORKLOADS
+        want = (e["fetch_size_kib"] * e["fetch_scale"] + e["write_size_kib"] * e["write_scale"]) * 1024.0
+        assert abs(e["bytes"] - want) <= 1e-6 * want

@@ -20,7 +20,9 @@ DEV = "cuda:0"
 
 # the MFMA kernel as the library picks it (small batches: without prefill tiles), the MFMA kernel with prefill tiles
 # forced, and the scalar kernel
-PATHS = [pytest.param(0, id="tiled"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles"),
+PATHS = [pytest.param(0, id="tiled"),
+         pytest.param(_native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, id="tiles"),
+         pytest.param(_native.RPA_FLAG_PIPE_TILES, id="pipe"),  # head_dim 128, pages of 16 keys or more; else as "tiles"
          pytest.param(_native.RPA_FLAG_FORCE_GENERIC, id="generic")]
 
 
@@ -200,9 +202,12 @@ def test_bf16_fp32_logit_arithmetic_on_prefill_tiles(D, window, cap):
     rounding of the probabilities and of the output."""
     b = small([300, 1, 70, 130, 3], [300, 300, 100, 517, 90], num_q_heads=8, num_kv_heads=2, head_dim=D,
               page_size=16, pages_per_seq=36, sliding_window=window, logits_soft_cap=cap)
-    out = to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_FP32_LOGITS))
-    mx, mean = err_stats(out, run_exact(b), b.total_valid_tokens)
-    assert np.isfinite(out).all() and mx <= 2e-2 and mean <= 1e-3, f"D={D} W={window} cap={cap}: max-abs {mx:.4g} mean-abs {mean:.4g}"
+    exact = run_exact(b)
+    for tiles in (_native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_PIPE_TILES):
+        out = to_np(run_hip(b, tiles | _native.RPA_FLAG_FP32_LOGITS))
+        mx, mean = err_stats(out, exact, b.total_valid_tokens)
+        assert np.isfinite(out).all() and mx <= 2e-2 and mean <= 1e-3, \
+            f"D={D} W={window} cap={cap} tiles={tiles}: max-abs {mx:.4g} mean-abs {mean:.4g}"
 
 
 @pytest.mark.parametrize("hq,hkv,D", [(8, 2, 128), (16, 2, 256), (8, 2, 64)])
@@ -311,7 +316,8 @@ def test_bf16_random_batches(seed):
     rows = b.total_valid_tokens
     strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
     finite = np.isfinite(strict).all(axis=(1, 2))
-    for flags in (0, _native.RPA_FLAG_PREFILL_TILES, _native.RPA_FLAG_FORCE_GENERIC):
+    for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_PIPE_TILES,
+                  _native.RPA_FLAG_FORCE_GENERIC):
         out = to_np(run_hip(b, flags))
         assert np.isfinite(out[:rows]).all(), what
         if finite.any():

@@ -21,7 +21,9 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 # the MFMA kernel as the library picks it (small batches: without prefill tiles), the MFMA kernel with prefill tiles
 # forced, and the scalar kernel
-PATHS = [pytest.param(0, id="tiled"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles"),
+PATHS = [pytest.param(0, id="tiled"),
+         pytest.param(_native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, id="tiles"),
+         pytest.param(_native.RPA_FLAG_PIPE_TILES, id="pipe"),  # head_dim 128, pages of 16 keys or more; else as "tiles"
          pytest.param(_native.RPA_FLAG_FORCE_GENERIC, id="generic")]
 
 
@@ -182,7 +184,8 @@ def test_bf16_random_batches(seed):
     bound of the restatement (two bf16 steps of the value where that is larger)."""
     b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))
     rows = b.total_valid_tokens
-    for flags in (0, _native.RPA_FLAG_PREFILL_TILES, _native.RPA_FLAG_FORCE_GENERIC):
+    for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_PIPE_TILES,
+                  _native.RPA_FLAG_FORCE_GENERIC):
         v = to_v3(random_rpa_batch(seed, DEV, head_dims=(128, 256))[0], seed=seed)   # the call updates the cache in place
         ref_out, ref_cache = oracle(v)
         out, cache = run_hip(v, flags)
