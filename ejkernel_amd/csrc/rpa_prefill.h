@@ -13,9 +13,8 @@
 // operand read from LDS feeds MRT MFMAs, Q stays in registers, and each lane owns one row per row
 // tile, so the online softmax is lane-local as in the decode loop.  The row sums come from one
 // extra MFMA against a vector of ones (they add exactly the bf16 probabilities that enter P V).
-// Logits stay in fp32 here unless a soft cap follows (the decode loop rounds them to bf16 as the reference does; on
-// prefill tiles that rounding only costs vector instructions: against the reference restatement the mean
-// error moves from 4e-4 to 5.5e-4 of a 2e-3 budget).  The K operands of a half are requested one
+// Logits are rounded to bf16 where the reference rounds them (kMimic; _xla_impl_fwd.py:119-124), as in the decode
+// loop -- except at head_dim 64, see below; the arithmetic of ragged_page_attention_v3 keeps them in fp32.  The K operands of a half are requested one
 // half ahead and the barrier that publishes the next tile sits before the last P V of a tile, so
 // LDS latency and barrier skew hide behind matrix work.  Halves of a step that lie entirely in a
 // wavefront's causal future, left of its window or before the sequence's first visible key are
@@ -403,6 +402,18 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
               for (int r = 0; r < 4; ++r)  // the cap's own bf16 roundings make it sensitive to its input: round that too
                 sv[u][r] = soft_cap<kMimic>(kMimic ? rbf(sv[u][r]) : sv[u][r], cap, inv_cap);
+          }
+          else if (kMimic && D >= 128) {
+            // the reference's logits are bf16 (_xla_impl_fwd.py:119-124): round them, two per conversion (head_dim 64
+            // keeps fp32 logits: its tiles are bound by vector instructions and the rounding costs them 16 %)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; r += 2) {
+                const uint32_t pk = pack_bf16x2(sv[u][r], sv[u][r + 1]);
+                sv[u][r] = __uint_as_float(pk << 16);
+                sv[u][r + 1] = __uint_as_float(pk & 0xffff0000u);
+              }
           }
           // a row tile that sees none of these keys goes through the mask with every key dropped: P = 0
           const bool need_mask = a0 <= clear_lo[m] || a0 > clear_hi[m];

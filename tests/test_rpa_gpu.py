@@ -321,7 +321,7 @@ def test_bf16_random_batches(seed):
         out = to_np(run_hip(b, flags))
         assert np.isfinite(out[:rows]).all(), what
         if finite.any():
-            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}", exact=exact[finite])
+            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}")
         mx, mean = err_stats(out, exact, rows)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
         assert not out[rows:].any()
