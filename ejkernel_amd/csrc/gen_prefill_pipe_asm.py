@@ -8,76 +8,79 @@ fixed registers.  The C++ side binds its variables to the same registers with ph
 compiler still sees every value that enters or leaves.  `python gen_prefill_pipe_asm.py` rewrites the .inc file; a
 CPU test compares the committed file with this script's output.
 
-Register map (one wavefront):
-  a[0:127]    O^T accumulators, row tile m, column block c: a[32 m + 4 c : +3]                     (out)
-  a[128:143]  row sums, row tile m: a[128 + 4 m : +3]                                             (out)
-  a[144:175]  K operands of one half, sub-tile u, k-step ks: a[144 + 4 (4 u + ks) : +3]
-  a[176:207]  V^T operands of one half, column block c: a[176 + 4 c : +3]
-  v[0:31]     logits / exp2 arguments, buffer A: row tile m, sub-tile u: v[4 (2 m + u) : +3]
+Register map (one wavefront; i = lane % 32, g = lane / 32; the 64 rows are two groups of 32, "rg"):
+  a[0:127]    O^T accumulators (32x32 MFMA tiles), row group rg, block of 32 output elements blk:
+              a[16 (4 rg + blk) : +15]; register 4 q + r of a tile holds element 32 blk + 8 q + 4 g + r of row i    (out)
+  a[128:159]  K operands of one half, k-step ks (16 elements of head_dim): a[128 + 4 ks : +3]
+  a[160:191]  V^T operands of one half, 16-key step s, block blk: a[160 + 4 (4 s + blk) : +3]
+  v[0:31]     logits / exp2 arguments, buffer A: row group rg: v[16 rg : +15]; register 4 q + r holds key 8 q + 4 g + r
   v[32:63]    the same, buffer B (halves alternate between the buffers)
-  v[64:127]   Q operands, row tile m, k-step ks: v[64 + 4 (4 m + ks) : +3]                        (in)
-  v[128:143]  P^T operands, row tile m: v[128 + 4 m : +3]
-  v[144:147]  eight bf16 ones (operand of the row-sum MFMA)
-  v[148:151]  -m log2(e) per row tile, the offset of the exp2 argument                            (out)
-  v[152:155]  maximum exp2 argument of the half per row tile
-  v[156:159]  masked halves: first visible key of the lane's rows relative to the lane's first key of the half
-  v[160:163]  visible keys of the lane's rows minus one (0 with an unreachable first key: none)   (in)
-  v[164:167]  LDS address of the K operand reads per k-step (stage of the next tile);  v168  of the V^T reads
+  v[64:127]   Q operands, row group rg, k-step ks: v[64 + 4 (8 rg + ks) : +3]                     (in)
+  v[128:143]  P^T operands, row group rg, key step s: v[128 + 4 (2 rg + s) : +3]
+  v[144:145]  row sums of the lane's keys per row group (the two lanes of a row add up at the end) (out)
+  v146        two bf16 ones (operand of the row-sum dot product)
+  v[148:149]  -m log2(e) per row group, the offset of the exp2 argument                           (out)
+  v[152:153]  maximum exp2 argument of the half per row group
+  v[156:157]  masked halves: first visible key of the lane's rows relative to the lane's first key of the half
+  v[160:161]  visible keys of the lane's rows minus one (0 with an unreachable first key: none)   (in)
+  v168        LDS address of the V^T operand reads (stage of this tile)
   v169        factor of the exp2 argument: log2(e) times the fp32 logit scale                     (in)
   v170, v195:199  temporaries;  v171  -inf;  v[200:215]  fetch: byte offsets of the lane's pieces
-  v[172:175]  threshold of the exp2 arguments per row tile: -inf before a row's first key         (out)
+  v[172:173]  threshold of the exp2 arguments per row group: -inf before a row's first key        (out)
   v176        the threshold once a row has a reference point
-  v[178:181]  first visible key of the lane's rows minus 4 g (absolute)                           (in)
-  v[182:185]  LDS address of the K operand reads per k-step in stage 0;  v186  of the V^T reads   (in)
+  v[178:179]  first visible key of the lane's rows minus 4 g (absolute)                           (in)
+  v186        LDS address of the V^T operand reads in stage 0                                    (in)
   v[187:189]  fetch: the lane's row in a K block, in a V block, byte offset of its V piece        (in)
   v[190:193]  fetch: byte offset of the lane's 16-byte piece in a K row, per block of four rows   (in)
+  v[216:223]  LDS address of the K operand reads per k-step (stage of the next tile)
+  v[224:231]  the same in stage 0                                                                (in)
   s[36:43]    halves of this wavefront, tiles, first key of the range, all_lo, all_hi (a half starting at a0 needs no
               mask iff all_lo < a0 <= all_hi), last key of the range, 16 * wavefront, LDS address of the wavefront's
               part of stage 0                                                                     (in)
   s[44:51]    block table row (64 bit), cache base of the kv head's K rows (64 bit), bytes per token, bytes per page,
               log2(page size), pages - 1                                                          (in)
-  s[52:79]    temporaries
+  s[52:75], s[89:92]  temporaries
 """
 
 from __future__ import annotations
 
 import os
 
-MRT, NKS, CB = 4, 4, 8
+NRG, NKS, NBLK = 2, 8, 4   # row groups of 32 rows, k-steps of 16 elements, blocks of 32 output elements
 ROWB = 256
 STAGE_B = 32768   # K tile + V tile
 NSTG = 4
 LAZY_LOG2E = 16.0 * 1.4426950408889634
 
-O = lambda m, c: f"a[{32 * m + 4 * c}:{32 * m + 4 * c + 3}]"
-L = lambda m: f"a[{128 + 4 * m}:{128 + 4 * m + 3}]"
-KOP = lambda u, ks: f"a[{144 + 4 * (4 * u + ks)}:{144 + 4 * (4 * u + ks) + 3}]"
-VRAW2 = lambda c, u: f"a[{176 + 4 * c + 2 * u}:{176 + 4 * c + 2 * u + 1}]"
-VRAW = lambda c: f"a[{176 + 4 * c}:{176 + 4 * c + 3}]"
-SQ = lambda base, m, u: f"v[{base + 4 * (2 * m + u)}:{base + 4 * (2 * m + u) + 3}]"
-SE = lambda base, m, u, r: f"v{base + 4 * (2 * m + u) + r}"
-QOP = lambda m, ks: f"v[{64 + 4 * (4 * m + ks)}:{64 + 4 * (4 * m + ks) + 3}]"
-PW = lambda m: f"v[{128 + 4 * m}:{128 + 4 * m + 3}]"
-PWE = lambda m, k: f"v{128 + 4 * m + k}"
-ONES = "v[144:147]"
-MNEG = lambda m: f"v{148 + m}"
-TMAX = lambda m: f"v{152 + m}"
-MLO = lambda m: f"v{156 + m}"
-MSPAN = lambda m: f"v{160 + m}"
-KADDR = lambda ks: f"v{164 + ks}"
+O = lambda rg, blk: f"a[{16 * (4 * rg + blk)}:{16 * (4 * rg + blk) + 15}]"
+KOP = lambda ks: f"a[{128 + 4 * ks}:{128 + 4 * ks + 3}]"
+VRAW2 = lambda s, blk, t: f"a[{160 + 4 * (4 * s + blk) + 2 * t}:{160 + 4 * (4 * s + blk) + 2 * t + 1}]"
+VRAW = lambda s, blk: f"a[{160 + 4 * (4 * s + blk)}:{160 + 4 * (4 * s + blk) + 3}]"
+SQ = lambda base, rg: f"v[{base + 16 * rg}:{base + 16 * rg + 15}]"
+SE = lambda base, rg, q, r: f"v{base + 16 * rg + 4 * q + r}"
+QOP = lambda rg, ks: f"v[{64 + 4 * (8 * rg + ks)}:{64 + 4 * (8 * rg + ks) + 3}]"
+PW = lambda rg, s: f"v[{128 + 4 * (2 * rg + s)}:{128 + 4 * (2 * rg + s) + 3}]"
+PWE = lambda rg, s, k: f"v{128 + 4 * (2 * rg + s) + k}"
+LSUM = lambda rg: f"v{144 + rg}"
+ONES2 = "v146"
+MNEG = lambda rg: f"v{148 + rg}"
+TMAX = lambda rg: f"v{152 + rg}"
+MLO = lambda rg: f"v{156 + rg}"
+MSPAN = lambda rg: f"v{160 + rg}"
+KADDR = lambda ks: f"v{216 + ks}"
 VADDR = "v168"
 CFAC = "v169"
 T0 = "v170"
 NINF = "v171"
-MTHR = lambda m: f"v{172 + m}"
+MTHR = lambda rg: f"v{172 + rg}"
 THRC = "v176"
-ROWLO = lambda m: f"v{178 + m}"
-KBASE = lambda ks: f"v{182 + ks}"
+ROWLO = lambda rg: f"v{178 + rg}"
+KBASE = lambda ks: f"v{224 + ks}"
 VBASE = "v186"
 LROW, VROW, VPIECE = "v187", "v188", "v189"
 KPIECE = lambda n: f"v{190 + n}"
 T1, T2, T3, T4, T5 = "v195", "v196", "v197", "v198", "v199"
-MFMA = "v_mfma_f32_16x16x32_bf16"
+MFMA = "v_mfma_f32_32x32x16_bf16"
 PROF = os.environ.get("RPA_PPA_PROF", "") != ""   # experiment: cycle counts of the loop's regions in s[76:83]
 
 
@@ -104,90 +107,97 @@ S_PEND, S_SITE = "s74", "s75"   # fetch of the tile in S_TT pending (this wavefr
 
 
 def kload(h: int) -> list[str]:
-    """K operands of a half with parity h from the stage that v[164:167] point into."""
-    return [f"ds_read_b128 {KOP(u, ks)}, {KADDR(ks)} offset:{h * 32 * ROWB + u * 16 * ROWB}" for u in range(2) for ks in range(NKS)]
+    """K operands of a half with parity h from the stage that v[216:223] point into: lane (i, g) reads elements
+    16 ks + 8 g .. + 7 of key row i."""
+    return [f"ds_read_b128 {KOP(ks)}, {KADDR(ks)} offset:{h * 32 * ROWB}" for ks in range(NKS)]
 
 
 def vload(h: int) -> list[str]:
-    """V^T operands of a half with parity h: per column block the keys 4g..4g+3 of both 16-key sub-tiles."""
-    return [f"ds_read_b64_tr_b16 {VRAW2(c, u)}, {VADDR} offset:{(8 * h + 4 * u) * 1024 + c * 128}" for c in range(CB) for u in range(2)]
+    """V^T operands of a half with parity h: for key step s and block blk the keys 16 s + 8 t + 4 g .. + 3 (t = 0, 1)
+    of output elements 32 blk + i, by two transposing reads (in each group of 16 lanes, lanes 4e..4e+3 address 16
+    consecutive elements of key e; lane x receives element x of the four keys)."""
+    return [f"ds_read_b64_tr_b16 {VRAW2(s, blk, t)}, {VADDR} offset:{(8 * h + 4 * s + 2 * t) * 1024 + blk * 256}"
+            for s in range(2) for blk in range(NBLK) for t in range(2)]
 
 
 def qk(n: int, nxt: int) -> str:
-    """MFMA n (0..31) of S^T = K Q^T: k-step outermost, so consecutive MFMAs feed different accumulators."""
-    ks, u, m = n >> 3, (n >> 2) & 1, n & 3
-    c = "0" if ks == 0 else SQ(nxt, m, u)
-    return f"{MFMA} {SQ(nxt, m, u)}, {KOP(u, ks)}, {QOP(m, ks)}, {c}"
+    """MFMA n (0..15) of S^T = K Q^T: k-step outermost, the two row groups in turn."""
+    ks, rg = n >> 1, n & 1
+    c = "0" if ks == 0 else SQ(nxt, rg)
+    return f"{MFMA} {SQ(nxt, rg)}, {KOP(ks)}, {QOP(rg, ks)}, {c}"
 
 
-def sm1_pair(cur: int, m: int, e: int, mask: bool, rnd: bool) -> tuple[list[str], list[str]]:
-    """Elements e, e + 1 of row tile m: logit -> exp2 argument in place, running maximum.  Two groups of
-    instructions, for the two MFMA slots of the pair: an MFMA occupies the matrix pipe for 16 cycles and the issue port
-    for about 8, so three vector instructions behind every MFMA cost nothing, six behind every other one do."""
-    u, r = e >> 2, e & 3
-    x0, x1 = SE(cur, m, u, r), SE(cur, m, u, r + 1)
-    first, second = [], []
+def sm1_pair(cur: int, p: int, mask: bool, rnd: bool) -> list[str]:
+    """Pair p (0..15) of the half: elements (rg, q, r), (rg, q, r + 1) with rg = p / 8, q = (p % 8) / 2, r = 2 (p % 2):
+    logit -> exp2 argument in place, running maximum of the row group."""
+    rg, q, r = p >> 3, (p & 7) >> 1, 2 * (p & 1)
+    x0, x1 = SE(cur, rg, q, r), SE(cur, rg, q, r + 1)
+    out = []
     if mask:
-        for x, cst in ((x0, 16 * u + r), (x1, 16 * u + r + 1)):
-            first += [f"v_sub_u32 {T0}, {cst}, {MLO(m)}", f"v_cmp_le_u32 vcc, {T0}, {MSPAN(m)}", f"v_cndmask_b32 {x}, {NINF}, {x}, vcc"]
+        for x, cst in ((x0, 8 * q + r), (x1, 8 * q + r + 1)):
+            out += [f"v_sub_u32 {T0}, {cst}, {MLO(rg)}", f"v_cmp_le_u32 vcc, {T0}, {MSPAN(rg)}", f"v_cndmask_b32 {x}, {NINF}, {x}, vcc"]
     if rnd:
-        first += [f"v_cvt_pk_bf16_f32 {T0}, {x0}, {x1}", f"v_lshlrev_b32 {x0}, 16, {T0}", f"v_and_b32 {x1}, 0xffff0000, {T0}"]
-    second += [f"v_fma_f32 {x0}, {x0}, {CFAC}, {MNEG(m)}", f"v_fma_f32 {x1}, {x1}, {CFAC}, {MNEG(m)}"]
-    second += [f"v_max_f32 {TMAX(m)}, {x0}, {x1}" if e == 0 else f"v_max3_f32 {TMAX(m)}, {TMAX(m)}, {x0}, {x1}"]
-    if not first:  # nothing to round or mask: one instruction group, split evenly
-        first, second = second[:2], second[2:]
-    return first, second
-
-
-def block_a(h: int, mask: bool, rnd: bool) -> list[str]:
-    """[QK(next half) | SM1(this half)]: 32 slots of one MFMA and half a pair's vector work."""
-    cur, nxt = (0, 32) if h == 0 else (32, 0)
-    out = ["s_waitcnt lgkmcnt(0)"] + vload(h)
-    if mask:
-        out += [f"v_subrev_u32 {MLO(m)}, {S_A0}, {ROWLO(m)}" for m in range(MRT)]
-    for n in range(32):
-        out.append(qk(n, nxt))
-        out += sm1_pair(cur, n >> 3, (n & 7) & ~1, mask, rnd)[n & 1]
+        out += [f"v_cvt_pk_bf16_f32 {T0}, {x0}, {x1}", f"v_lshlrev_b32 {x0}, 16, {T0}", f"v_and_b32 {x1}, 0xffff0000, {T0}"]
+    out += [f"v_fma_f32 {x0}, {x0}, {CFAC}, {MNEG(rg)}", f"v_fma_f32 {x1}, {x1}, {CFAC}, {MNEG(rg)}"]
+    out += [f"v_max_f32 {TMAX(rg)}, {x0}, {x1}" if (p & 7) == 0 else f"v_max3_f32 {TMAX(rg)}, {TMAX(rg)}, {x0}, {x1}"]
     return out
 
 
-def sm2_exp(cur: int, m: int, k: int) -> list[str]:
-    u, r = k >> 1, 2 * (k & 1)
-    return [f"v_exp_f32 {SE(cur, m, u, r)}, {SE(cur, m, u, r)}", f"v_exp_f32 {SE(cur, m, u, r + 1)}, {SE(cur, m, u, r + 1)}"]
+def block_a(h: int, mask: bool, rnd: bool) -> list[str]:
+    """[QK(next half) | SM1(this half)]: 16 slots of one MFMA (32 cycles of the matrix pipe, about 8 of the issue port)
+    and one pair's vector work (six instructions, about 25 cycles)."""
+    cur, nxt = (0, 32) if h == 0 else (32, 0)
+    out = ["s_waitcnt lgkmcnt(0)"] + vload(h)
+    if mask:
+        out += [f"v_subrev_u32 {MLO(rg)}, {S_A0}, {ROWLO(rg)}" for rg in range(NRG)]
+    for n in range(16):
+        out.append(qk(n, nxt))
+        out += sm1_pair(cur, n, mask, rnd)
+    return out
 
 
-def sm2_pack(cur: int, m: int, k: int) -> list[str]:
-    u, r = k >> 1, 2 * (k & 1)
-    return [f"v_cvt_pk_bf16_f32 {PWE(m, k)}, {SE(cur, m, u, r)}, {SE(cur, m, u, r + 1)}"]
+def sm2_exp(cur: int, rg: int, s: int, k: int) -> list[str]:
+    """The exponentials of pair k (0..3) of P(rg, s): elements q = 2 s + k / 2, r = 2 (k % 2), + 1."""
+    q, r = 2 * s + (k >> 1), 2 * (k & 1)
+    return [f"v_exp_f32 {SE(cur, rg, q, r)}, {SE(cur, rg, q, r)}", f"v_exp_f32 {SE(cur, rg, q, r + 1)}, {SE(cur, rg, q, r + 1)}"]
 
 
-def sm2_tile(cur: int, m: int) -> list[list[str]]:
-    """P of row tile m = exp2 of its eight arguments, packed to bf16, as nine groups of instructions for the gaps
-    behind the nine MFMAs of the row tile before it.  The result of a transcendental instruction may not be read by
-    the very next instruction (the hardware does not wait), and a register written by a vector instruction may not be
-    read by an MFMA within two wait states: the pack of a pair follows the first exponential of the next pair, and
-    the last pack is followed by two idle states."""
-    e = [sm2_exp(cur, m, k) for k in range(4)]
-    p = [sm2_pack(cur, m, k) for k in range(4)]
-    return [[e[0][0]], [e[0][1]], [e[1][0]] + p[0], [e[1][1]], [e[2][0]] + p[1], [e[2][1]], [e[3][0]] + p[2], [e[3][1]],
-            p[3] + ["s_nop 1"]]
+def sm2_pack(cur: int, rg: int, s: int, k: int) -> list[str]:
+    q, r = 2 * s + (k >> 1), 2 * (k & 1)
+    return [f"v_cvt_pk_bf16_f32 {PWE(rg, s, k)}, {SE(cur, rg, q, r)}, {SE(cur, rg, q, r + 1)}"]
+
+
+def rowsum(rg: int, s: int, k: int) -> list[str]:
+    return [f"v_dot2_f32_bf16 {LSUM(rg)}, {PWE(rg, s, k)}, {ONES2}, {LSUM(rg)}"]
 
 
 def block_b(h: int) -> list[str]:
-    """[SM2 | PV]: the exponentials of row tile m + 1 in the gaps behind the 9 MFMAs of row tile m."""
+    """[SM2 | PV]: P^T operand (rg, s) = exp2 of eight arguments per lane, packed to bf16; its four MFMAs (one per
+    block of 32 output elements) run while the vector unit prepares the next operand and adds up its row sums.
+    Rules the order obeys: the result of a transcendental instruction may not be read by the very next instruction
+    (the hardware does not wait); a register written by a vector instruction may not be read by an MFMA within two
+    wait states; and a vector instruction that touches a register an MFMA in flight reads waits for that MFMA, so
+    the row sums of an operand are added before its MFMAs start, not beside them."""
     cur = 0 if h == 0 else 32
+    groups = [(rg, s) for rg in range(NRG) for s in range(2)]
     out = kload(h) + ["s_waitcnt lgkmcnt(8)"]
-    first = sm2_tile(cur, 0)
-    first[8] = ["s_nop 0"] + first[8]  # no MFMA between the last exponential and the pack that reads it
-    for grp in first:
-        out += grp
-    for m in range(MRT):
-        nxt = sm2_tile(cur, m + 1) if m + 1 < MRT else [[] for _ in range(9)]
-        out.append(f"{MFMA} {L(m)}, {ONES}, {PW(m)}, {L(m)}")
-        out += nxt[0]
-        for c in range(CB):
-            out.append(f"{MFMA} {O(m, c)}, {VRAW(c)}, {PW(m)}, {O(m, c)}")
-            out += nxt[c + 1]
+    rg, s = groups[0]
+    out += sm2_exp(cur, rg, s, 0) + sm2_exp(cur, rg, s, 1) + sm2_pack(cur, rg, s, 0) + sm2_exp(cur, rg, s, 2) + sm2_pack(cur, rg, s, 1)
+    out += rowsum(rg, s, 0) + sm2_exp(cur, rg, s, 3) + sm2_pack(cur, rg, s, 2) + rowsum(rg, s, 1) + sm2_pack(cur, rg, s, 3)
+    out += rowsum(rg, s, 2) + rowsum(rg, s, 3)
+    for gi, (rg, s) in enumerate(groups):
+        nx = groups[gi + 1] if gi + 1 < len(groups) else None
+        for blk in range(NBLK):
+            out.append(f"{MFMA} {O(rg, blk)}, {VRAW(s, blk)}, {PW(rg, s)}, {O(rg, blk)}")
+            if nx is None:
+                continue
+            out += sm2_exp(cur, nx[0], nx[1], blk)
+            if blk == 1:
+                out += sm2_pack(cur, *nx, 0)
+            if blk == 2:
+                out += sm2_pack(cur, *nx, 1) + rowsum(*nx, 0)
+            if blk == 3:
+                out += sm2_pack(cur, *nx, 2) + rowsum(*nx, 1) + sm2_pack(cur, *nx, 3) + rowsum(*nx, 2) + rowsum(*nx, 3)
     return out
 
 
@@ -196,33 +206,31 @@ def rescale(h: int, tag: str) -> list[str]:
     reference point up by the row maximum: shift the exp2 arguments, scale row sum and outputs by exp2(-shift)."""
     cur = 0 if h == 0 else 32
     # (a row without a reference point has threshold -inf: the difference is +inf, or NaN when it has no key yet either,
-    # which the maxima drop)
-    out = [f"v_sub_f32 {tmp}, {TMAX(m)}, {MTHR(m)}" for m, tmp in enumerate((T1, T2, T3, T4))]
-    out += [f"v_max3_f32 {T1}, {T1}, {T2}, {T3}", f"v_max_f32 {T1}, {T1}, {T4}", f"v_cmp_lt_f32 vcc, 0, {T1}"]
-    out.append(f"s_cbranch_vccz .Lpp_noresc_{tag}_%=")
-    for m in range(MRT):
-        x = TMAX(m)
-        # maximum over the four lanes that hold one row (lanes l, l ^ 16, l ^ 32, l ^ 48)
-        out += [f"v_mov_b32 {T1}, {x}", f"v_mov_b32 {T2}, {x}", "s_nop 1", f"v_permlane16_swap_b32 {T1}, {T2}", "s_nop 1",
-                f"v_max_f32 {T3}, {T1}, {T2}", f"v_mov_b32 {T1}, {T3}", f"v_mov_b32 {T2}, {T3}", "s_nop 1",
-                f"v_permlane32_swap_b32 {T1}, {T2}", "s_nop 1", f"v_max_f32 {T3}, {T1}, {T2}"]
-        out += [f"v_cmp_gt_f32 vcc, {T3}, {MTHR(m)}", f"s_cbranch_vccz .Lpp_skip{m}_{tag}_%="]
+    # which the maximum drops)
+    out = [f"v_sub_f32 {T1}, {TMAX(0)}, {MTHR(0)}", f"v_sub_f32 {T2}, {TMAX(1)}, {MTHR(1)}", f"v_max_f32 {T1}, {T1}, {T2}",
+           f"v_cmp_lt_f32 vcc, 0, {T1}", f"s_cbranch_vccz .Lpp_noresc_{tag}_%="]
+    for rg in range(NRG):
+        x = TMAX(rg)
+        # maximum over the two lanes that hold one row (lanes l, l ^ 32)
+        out += [f"v_mov_b32 {T1}, {x}", f"v_mov_b32 {T2}, {x}", "s_nop 1", f"v_permlane32_swap_b32 {T1}, {T2}", "s_nop 1",
+                f"v_max_f32 {T3}, {T1}, {T2}"]
+        out += [f"v_cmp_gt_f32 vcc, {T3}, {MTHR(rg)}", f"s_cbranch_vccz .Lpp_skip{rg}_{tag}_%="]
         out += [f"v_cndmask_b32 {T4}, 0, {T3}, vcc",                       # shift: the row maximum where the row moves
                 f"v_exp_f32_e64 {T5}, -{T3}",
-                f"v_cmp_neq_f32 {S_P}, {MTHR(m)}, {NINF}",
+                f"v_cmp_neq_f32 {S_P}, {MTHR(rg)}, {NINF}",
                 f"v_cndmask_b32_e64 {T5}, 0, {T5}, {S_P}",                 # a row without a reference point: outputs are zero
                 f"v_cndmask_b32 {T5}, 1.0, {T5}, vcc",                     # alpha
-                f"v_cndmask_b32 {MTHR(m)}, {MTHR(m)}, {THRC}, vcc"]
-        out += [f"v_sub_f32 {SE(cur, m, u, r)}, {SE(cur, m, u, r)}, {T4}" for u in range(2) for r in range(4)]
-        out.append(f"v_sub_f32 {MNEG(m)}, {MNEG(m)}, {T4}")
-        regs = [128 + 4 * m + k for k in range(4)] + [32 * m + k for k in range(32)]
+                f"v_cndmask_b32 {MTHR(rg)}, {MTHR(rg)}, {THRC}, vcc"]
+        out += [f"v_sub_f32 {SE(cur, rg, q, r)}, {SE(cur, rg, q, r)}, {T4}" for q in range(4) for r in range(4)]
+        out += [f"v_sub_f32 {MNEG(rg)}, {MNEG(rg)}, {T4}", f"v_mul_f32 {LSUM(rg)}, {LSUM(rg)}, {T5}"]
+        regs = [64 * rg + k for k in range(64)]
         for q in range(0, len(regs), 4):
             grp = regs[q:q + 4]
             tmp = [T1, T2, T3, T4]
             out += [f"v_accvgpr_read_b32 {t}, a{a}" for t, a in zip(tmp, grp)]
             out += [f"v_mul_f32 {t}, {t}, {T5}" for t in tmp]
             out += [f"v_accvgpr_write_b32 a{a}, {t}" for t, a in zip(tmp, grp)]
-        out.append(f".Lpp_skip{m}_{tag}_%=:")
+        out.append(f".Lpp_skip{rg}_{tag}_%=:")
     out.append(f".Lpp_noresc_{tag}_%=:")
     return out
 
@@ -338,10 +346,10 @@ def loop(rnd: bool) -> list[str]:
     if PROF:
         out += [f"s_mov_b32 s{76 + k}, 0" for k in range(8)] + ["s_memtime s[84:85]", "s_waitcnt lgkmcnt(0)", "s_mov_b32 s87, s84", "s_mov_b32 s88, s84"]
     # ---- set-up
-    out += [f"v_accvgpr_write_b32 a{k}, 0" for k in range(144)]
-    out += [f"v_mov_b32 {MNEG(m)}, 0" for m in range(MRT)] + [f"v_mov_b32 {NINF}, 0xff800000"]
-    out += [f"v_mov_b32 {MTHR(m)}, {NINF}" for m in range(MRT)]
-    out += [f"v_mov_b32 {THRC}, 0x{float_bits(LAZY_LOG2E):08x}"] + [f"v_mov_b32 v{144 + k}, 0x3f803f80" for k in range(4)]
+    out += [f"v_accvgpr_write_b32 a{k}, 0" for k in range(128)]
+    out += [f"v_mov_b32 {MNEG(rg)}, 0" for rg in range(NRG)] + [f"v_mov_b32 {LSUM(rg)}, 0" for rg in range(NRG)] + [f"v_mov_b32 {NINF}, 0xff800000"]
+    out += [f"v_mov_b32 {MTHR(rg)}, {NINF}" for rg in range(NRG)]
+    out += [f"v_mov_b32 {THRC}, 0x{float_bits(LAZY_LOG2E):08x}", f"v_mov_b32 {ONES2}, 0x3f803f80"]
     out += [f"s_mov_b32 {S_R2}, 0x7fffffff", f"s_mov_b32 {S_R3}, 0x00020000",
             f"s_lshl_b32 {S_PMASK}, 1, {S_PSHIFT}", f"s_add_i32 {S_PMASK}, {S_PMASK}, -1",
             f"s_mov_b32 {S_HH}, 0", f"s_mov_b32 {S_T}, 0", f"s_mov_b32 {S_A0}, {S_RLO}",
@@ -353,7 +361,7 @@ def loop(rnd: bool) -> list[str]:
     out += [f"s_mov_b32 {S_CUR}, {(NSTG - 1) * STAGE_B}", f"s_mov_b32 {S_NXT}, 0"]
     # logits of the first half, K operands of the second (both in tile 0, stage 0)
     out += [f"v_mov_b32 {KADDR(ks)}, {KBASE(ks)}" for ks in range(NKS)]
-    out += kload(0) + ["s_waitcnt lgkmcnt(0)"] + [qk(n, 0) for n in range(32)] + ["s_nop 7", "s_nop 7"] + kload(1)
+    out += kload(0) + ["s_waitcnt lgkmcnt(0)"] + [qk(n, 0) for n in range(16)] + ["s_nop 7", "s_nop 7"] + kload(1)
     out.append(".Lpp_tile_%=:")
     out += rotate_stages()
     h0, cold0 = half(0, rnd)
@@ -371,7 +379,7 @@ def loop(rnd: bool) -> list[str]:
     out += publish("tail", S_T) + site(-1, "st")
     out += [f"s_add_i32 {S_T}, {S_T}, 1",
             f"s_add_i32 {S_FBUF}, {S_FBUF}, {STAGE_B}", f"s_cmp_eq_u32 {S_FBUF}, {NSTG * STAGE_B}", f"s_cselect_b32 {S_FBUF}, 0, {S_FBUF}",
-            "s_branch .Lpp_tail_%=", ".Lpp_end_%=:", "s_waitcnt lgkmcnt(0)", "s_mov_b32 m0, s58", "s_nop 7", "s_nop 7"]
+            "s_branch .Lpp_tail_%=", ".Lpp_end_%=:", "s_waitcnt lgkmcnt(0)", "s_mov_b32 m0, s58", "s_nop 7", "s_nop 7", "s_nop 7"]
     if PROF:
         out += []
     return out

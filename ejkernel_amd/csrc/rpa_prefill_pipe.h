@@ -41,12 +41,12 @@ namespace rpa {
 
 struct PipeCfg {
   static constexpr int D = 128;
-  static constexpr int MRT = 4;                     // 16-row tiles per wavefront
-  static constexpr int NKS = D / 32;                // k-steps of the QK^T contraction
-  static constexpr int CB = D / 16;                 // MFMA column blocks of the output
+  static constexpr int NRG = 2;                     // groups of 32 rows per wavefront (one 32x32 MFMA tile each)
+  static constexpr int NKS = D / 16;                // k-steps of the QK^T contraction
+  static constexpr int NBLK = D / 32;               // blocks of 32 output elements
   static constexpr int TK = 64;                     // keys per tile (two halves of 32)
   static constexpr int ROWB = D * 2;                // LDS bytes per K row
-  static constexpr int WROWS = 16 * MRT;            // rows per wavefront
+  static constexpr int WROWS = 32 * NRG;            // rows per wavefront
   static constexpr int WGROWS = kWgWaves * WROWS;   // rows per workgroup: 256
   static constexpr int TILE_B = TK * ROWB;          // one K (or V) tile: 16 KiB
   static constexpr int NSTG = RPA_PP_NSTG;          // LDS stages
@@ -72,12 +72,13 @@ typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 // What the key loop takes and leaves, each member bound to the registers the instruction stream uses for it
 // (register map in gen_prefill_pipe_asm.py).
 struct PipeIo {
-  f32x32_t o0, o1, o2, o3;  // out: O^T accumulators of the four row tiles
-  f32x16_t l;               // out: row sums
-  f32x4_t mneg, mthr;       // out: exp2 offset and threshold per row tile
-  f32x32_t q0, q1;          // in: Q operands
-  i32x4_t mspan, rowlo;     // in: per-lane bounds of the visible keys
-  i32x4_t kbase, kpiece;    // in: LDS addresses of the K operand reads; fetch: piece offsets in a K row
+  f32x32_t o0, o1, o2, o3;  // out: O^T accumulators, row group 0 blocks 0-1, 2-3, row group 1 blocks 0-1, 2-3
+  f32x4_t lsum;             // out: row sums of the lane's keys per row group ([0], [1])
+  f32x4_t mneg, mthr;       // out: exp2 offset and threshold per row group ([0], [1])
+  f32x32_t q0, q1;          // in: Q operands of row group 0, 1
+  i32x4_t mspan, rowlo;     // in: per-lane bounds of the visible keys per row group ([0], [1])
+  i32x4_t kbase0, kbase1;   // in: LDS addresses of the K operand reads per k-step
+  i32x4_t kpiece;           // in: fetch: piece offsets in a K row
   i32x4_t misc;             // in: LDS address of the V^T reads, fetch: row in a K block, in a V block, V piece offset
   float cfac;               // in: factor of the exp2 argument
   i32x8_t s0, s1;           // in: scalars (see the register map)
@@ -95,31 +96,33 @@ struct PipeIo {
 #define RPA_PPA_PROF_CLOBBERS
 #endif
 
-#define RPA_PPA_CLOBBERS                                                                                                  \
-  "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17",    \
-  "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33", "v34", \
-  "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", \
-  "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v128", "v129", "v130", "v131",    \
-  "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143", "v144", "v145",        \
-  "v146", "v147", "v152", "v153", "v154", "v155", "v156", "v157", "v158", "v159", "v164", "v165", "v166", "v167",        \
-  "v168", "v170", "v171", "v176", "v195", "v196", "v197", "v198", "v199", "v200", "v201", "v202", "v203", "v204",        \
-  "v205", "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213", "v214", "v215", "a144", "a145", "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154",        \
-  "a155", "a156", "a157", "a158", "a159", "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168",        \
-  "a169", "a170", "a171", "a172", "a173", "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182",        \
-  "a183", "a184", "a185", "a186", "a187", "a188", "a189", "a190", "a191", "a192", "a193", "a194", "a195", "a196",        \
-  "a197", "a198", "a199", "a200", "a201", "a202", "a203", "a204", "a205", "a206", "a207", "s52", "s53", "s54", "s55",    \
-  "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63", "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", \
-  "s73", "s74", "s75", "s89", "s90", "s91", "s92", "vcc", "scc", "memory"
+#define RPA_PPA_CLOBBERS \
+  "v0", "v1", "v2", "v3", "v4", "v5", "v6", "v7", "v8", "v9", "v10", "v11", "v12", "v13", "v14", "v15", "v16", "v17",  \
+  "v18", "v19", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33",      \
+  "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49",      \
+  "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63", "v128", "v129",    \
+  "v130", "v131", "v132", "v133", "v134", "v135", "v136", "v137", "v138", "v139", "v140", "v141", "v142", "v143",      \
+  "v146", "v152", "v153", "v156", "v157", "v168", "v170", "v171", "v176", "v195", "v196", "v197", "v198", "v199",      \
+  "v200", "v201", "v202", "v203", "v204", "v205", "v206", "v207", "v208", "v209", "v210", "v211", "v212", "v213",      \
+  "v214", "v215", "v216", "v217", "v218", "v219", "v220", "v221", "v222", "v223", "a128", "a129", "a130", "a131",      \
+  "a132", "a133", "a134", "a135", "a136", "a137", "a138", "a139", "a140", "a141", "a142", "a143", "a144", "a145",      \
+  "a146", "a147", "a148", "a149", "a150", "a151", "a152", "a153", "a154", "a155", "a156", "a157", "a158", "a159",      \
+  "a160", "a161", "a162", "a163", "a164", "a165", "a166", "a167", "a168", "a169", "a170", "a171", "a172", "a173",      \
+  "a174", "a175", "a176", "a177", "a178", "a179", "a180", "a181", "a182", "a183", "a184", "a185", "a186", "a187",      \
+  "a188", "a189", "a190", "a191", "s52", "s53", "s54", "s55", "s56", "s57", "s58", "s59", "s60", "s61", "s62", "s63",  \
+  "s64", "s65", "s66", "s67", "s68", "s69", "s70", "s71", "s72", "s73", "s74", "s75", "s89", "s90", "s91", "s92",      \
+  "vcc", "scc", "memory"
 
 // The key loop of one tile for one wavefront.  LDS stages 0 and 1 hold the first two K/V tiles (or the only one) and
 // have been published by a barrier; the stream runs every later barrier and fetch of the tile itself.
 template <bool kRound>
 __device__ __forceinline__ void pipe_key_loop(PipeIo& R) {
 #define RPA_PPA_OPERANDS                                                                                                  \
-  : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={a[128:143]}"(R.l),          \
+  : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={v[144:147]}"(R.lsum),       \
     "={v[148:151]}"(R.mneg), "={v[172:175]}"(R.mthr) RPA_PPA_PROF_OUT                                                  \
-  : "{v[64:95]}"(R.q0), "{v[96:127]}"(R.q1), "{v[160:163]}"(R.mspan), "{v[178:181]}"(R.rowlo), "{v[182:185]}"(R.kbase), \
-    "{v[186:189]}"(R.misc), "{v[190:193]}"(R.kpiece), "{v169}"(R.cfac), "{s[36:43]}"(R.s0), "{s[44:51]}"(R.s1)         \
+  : "{v[64:95]}"(R.q0), "{v[96:127]}"(R.q1), "{v[160:163]}"(R.mspan), "{v[178:181]}"(R.rowlo), "{v[224:227]}"(R.kbase0), \
+    "{v[228:231]}"(R.kbase1), "{v[186:189]}"(R.misc), "{v[190:193]}"(R.kpiece), "{v169}"(R.cfac), "{s[36:43]}"(R.s0),   \
+    "{s[44:51]}"(R.s1)                                                                                                 \
   : RPA_PPA_CLOBBERS RPA_PPA_PROF_CLOBBERS
   if constexpr (kRound) asm volatile(RPA_PPA_LOOP_ROUND RPA_PPA_OPERANDS);
   else asm volatile(RPA_PPA_LOOP_PLAIN RPA_PPA_OPERANDS);
@@ -130,7 +133,7 @@ template <bool kMimic>
 __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
                                                   int qt) {
   using C = PipeCfg;
-  constexpr int MRT = C::MRT;
+  constexpr int NRG = C::NRG;
   const RpaParams& p = a.p;
 #ifdef RPA_PP_PROF2
   const uint64_t pt0 = __builtin_readcyclecounter();
@@ -138,14 +141,12 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
 #endif
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int i = lane & 15, g = lane >> 4;
+  const int i = lane & 31, g = lane >> 5;  // 32x32 MFMA tiles: lane (i, g) owns row i of a row group
   const int G = p.num_q_heads / p.num_kv_heads;
   const int W = p.sliding_window;
   const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
   const char* kvb = static_cast<const char*>(p.kv_pages);
-  const float cap = kMimic ? rbf(p.logits_soft_cap) : p.logits_soft_cap;
-  const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
   const int pos0 = si.kv_len - si.q_len;  // position of the sequence's first query token
   constexpr int hd = C::D;
 
@@ -156,68 +157,70 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
   const int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
   const int t_last = range_hi - 1;
 
-  // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
+  // ---- this wavefront's rows: row group rg holds rows w_row_lo + 32 rg + i
   const int w_row_lo = wg_row_lo + wave * C::WROWS;
-  int pos_n[MRT];
-  auto row_of = [&](int m, int opaque0, bool& valid, int& head, size_t& q_off) {
-    const int R = w_row_lo + 16 * m + i + opaque0;
+  int pos_n[NRG];
+  auto row_of = [&](int rg, int opaque0, bool& valid, int& head, size_t& q_off) {
+    const int R = w_row_lo + 32 * rg + i + opaque0;
     valid = R < si.rows;
     const int qi = valid ? R / G : 0;
     head = j * G + (valid ? R - qi * G : 0);
     q_off = (static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head) * hd;
     return qi;
   };
-  bf16x8_t qreg[MRT][C::NKS];
+  PipeIo R;
   const float scale = rbf(p.softmax_scale);
-  const float post_scale = logit_scale(p);
-  // Without a soft cap the fp32 logit scale of the unscaled-q arithmetic is folded into the exp2 argument.
-  const bool fold_scale = !kMimic && cap == 0.f;
-  const float sf = fold_scale ? post_scale : 1.f, sf_log2e = sf * kLog2e;
-  // One interval test per half: no row tile of this wavefront needs a per-key mask iff all_lo < a0 <= all_hi.
+  // The fp32 logit scale of the unscaled-q arithmetic is folded into the exp2 argument (the host sends a batch
+  // with a soft cap, or with a scale that is not positive, to the plain tile).
+  const float sf_log2e = (kMimic ? 1.f : logit_scale(p)) * kLog2e;
+  // One interval test per half: no row group of this wavefront needs a per-key mask iff all_lo < a0 <= all_hi.
   int all_lo = -0x7fffffff, all_hi = 0x7fffffff;
 #pragma unroll
-  for (int m = 0; m < MRT; ++m) {
+  for (int rg = 0; rg < NRG; ++rg) {
     bool valid;
     int head;
     size_t q_off;
-    const int qi = row_of(m, 0, valid, head, q_off);
-    pos_n[m] = valid ? pos0 + qi : -1;
-    const int tr_lo = w_row_lo + 16 * m, tr_hi = min(tr_lo + 16, si.rows);
+    const int qi = row_of(rg, 0, valid, head, q_off);
+    pos_n[rg] = valid ? pos0 + qi : -1;
+    const int tr_lo = w_row_lo + 32 * rg, tr_hi = min(tr_lo + 32, si.rows);
     const bool t_any = tr_hi > tr_lo;
     const int t_pos_lo = pos0 + tr_lo / G, t_pos_hi = pos0 + (max(tr_hi, tr_lo + 1) - 1) / G;
-    // the row tile sees all 32 keys from a0 on iff nomask_lo < a0 <= nomask_hi (a tile without rows never does)
+    // the row group sees all 32 keys from a0 on iff nomask_lo < a0 <= nomask_hi (a group without rows never does)
     const int nomask_hi = t_any ? min(t_pos_lo - 31, range_hi - 32) : -0x7fffffff;
     const int nomask_lo = max(W > 0 ? t_pos_hi - W : -0x7fffffff, si.start - 1);
     all_lo = max(all_lo, nomask_lo);
     all_hi = min(all_hi, nomask_hi);
+    // Q operands: lane (i, g) holds elements 16 ks + 8 g .. + 7 of its row, scaled as the arithmetic asks
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
-      u32x4_t sc;
+      if (valid) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 16 * ks + 8 * g);
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
-                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
-      qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
+      for (int e = 0; e < 4; ++e) {
+        const float f = __uint_as_float(pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
+                                                    q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale)));
+        if (rg == 0) R.q0[4 * ks + e] = f;
+        else R.q1[4 * ks + e] = f;
+      }
     }
   }
   const bool w_any = w_row_lo < si.rows;
   const int w_pos_hi = pos0 + (min(w_row_lo + C::WROWS, si.rows) - 1) / G;
   const int w_act_hi = min(range_hi - 1, w_pos_hi);  // last key this wavefront's rows can see
 
-  f32x4_t o_acc[MRT][C::CB];
-  f32x4_t l_acc[MRT];
-  // Softmax reference point m per row, kept as the exp2 offset -m log2(e) (0 while the row has seen no key) and as
-  // the threshold for exp2 arguments: kLazy log2(e) once there is a reference point, -inf before.
-  float m_thr[MRT], m_neg[MRT];
+  // Results of the key loop: O^T accumulators as the 32x32 MFMA leaves them, the lane's part of the row sums, and the
+  // softmax reference point m per row as the exp2 offset -m log2(e) and its threshold (-inf: the row saw no key).
+  float o_acc[NRG][C::NBLK][16];
+  float l_part[NRG], m_thr[NRG], m_neg[NRG];
 #pragma unroll
-  for (int m = 0; m < MRT; ++m) {
-    m_thr[m] = -INFINITY;
-    m_neg[m] = 0.f;
-    l_acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int rg = 0; rg < NRG; ++rg) {
+    m_thr[rg] = -INFINITY;
+    m_neg[rg] = 0.f;
+    l_part[rg] = 0.f;
 #pragma unroll
-    for (int c = 0; c < C::CB; ++c) o_acc[m][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int blk = 0; blk < C::NBLK; ++blk)
+#pragma unroll
+      for (int k = 0; k < 16; ++k) o_acc[rg][blk][k] = 0.f;
   }
 
   // ---- cooperative fetch (as in rpa_prefill.h): one wave-wide direct-to-LDS load moves 4 rows; wavefront w moves
@@ -288,39 +291,36 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     const int hb = __builtin_amdgcn_readfirstlane(
         w_any && w_act_hi >= range_lo ? min(2 * n_tiles, ((w_act_hi - range_lo) >> 5) + 1) : 0);
 
-    PipeIo R;
     const int lds_base = static_cast<int>(reinterpret_cast<uintptr_t>(lds));  // LDS pointers are 32-bit offsets
-    // LDS addresses of the operand reads in stage 0: K per k-step; V^T, with the transposing read: in each group of 16
-    // lanes, lanes 4e..4e+3 point at 16 consecutive elements of key e of a 4-key block (see rpa_prefill.h)
+    // LDS addresses of the operand reads in stage 0.  K, per k-step: lane (i, g) reads the 16-byte piece 2 ks + g of
+    // key row i (pieces swizzled by the row, see rpa_prefill.h).  V^T, with the transposing read: in each group of 16
+    // lanes, lanes 4e..4e+3 point at 16 consecutive elements (one column unit) of key e of a 4-key block; the groups
+    // of a half-wave take the two column units of a block of 32 elements, the half-waves the key blocks g.
 #pragma unroll
-    for (int ks = 0; ks < C::NKS; ++ks) R.kbase[ks] = lds_base + i * C::ROWB + 16 * ((4 * ks + g) ^ C::swz(i));
-    const int v_key = 4 * g + (i >> 2);
-    R.misc[0] = lds_base + C::TILE_B + (v_key / C::RB) * 1024 + (v_key % C::RB) * 32 + 8 * (i & 3);
+    for (int ks = 0; ks < C::NKS; ++ks) {
+      const int addr = lds_base + i * C::ROWB + 16 * ((2 * ks + g) ^ C::swz(i));
+      if (ks < 4) R.kbase0[ks] = addr;
+      else R.kbase1[ks - 4] = addr;
+    }
+    const int x16 = lane & 15;
+    R.misc[0] = lds_base + C::TILE_B + g * 1024 + ((lane >> 4) & 1) * 128 + (x16 >> 2) * 32 + 8 * (x16 & 3);
     // fetch: the lane's row in a 4-row block and its 16-byte piece, K (swizzled by the row in the tile) and V
     R.misc[1] = l_row;
     R.misc[2] = v_row;
     R.misc[3] = static_cast<int>(v_src) + hd * 2;
 #pragma unroll
     for (int n = 0; n < C::HB; ++n) R.kpiece[n] = 16 * (l_slot ^ C::swz(C::RB * n + l_row));
-    // Per-lane bounds of the keys row tile m may see (none for a row past the end: an unreachable first key)
+    // Per-lane bounds of the keys a row group may see (none for a row past the end: an unreachable first key)
+    R.rowlo = i32x4_t{0, 0, 0, 0};
+    R.mspan = i32x4_t{0, 0, 0, 0};
 #pragma unroll
-    for (int m = 0; m < MRT; ++m) {
-      const int hi = min(pos_n[m], range_hi - 1);
-      const int lo = max(W > 0 ? pos_n[m] - W + 1 : -0x40000000, si.start);
-      R.rowlo[m] = (hi < lo ? 0x40000000 : lo) - 4 * g;
-      R.mspan[m] = max(hi - lo, 0);
+    for (int rg = 0; rg < NRG; ++rg) {
+      const int hi = min(pos_n[rg], range_hi - 1);
+      const int lo = max(W > 0 ? pos_n[rg] - W + 1 : -0x40000000, si.start);
+      R.rowlo[rg] = (hi < lo ? 0x40000000 : lo) - 4 * g;
+      R.mspan[rg] = max(hi - lo, 0);
     }
     R.cfac = sf_log2e;
-#pragma unroll
-    for (int m = 0; m < MRT; ++m)
-#pragma unroll
-      for (int ks = 0; ks < C::NKS; ++ks)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float f = __uint_as_float(__builtin_bit_cast(u32x4_t, qreg[m][ks])[e]);
-          if (m < 2) R.q0[4 * (4 * m + ks) + e] = f;
-          else R.q1[4 * (4 * (m - 2) + ks) + e] = f;
-        }
     const uint64_t bt_addr = reinterpret_cast<uint64_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq);
     const uint64_t kv_addr = reinterpret_cast<uint64_t>(kvb) + static_cast<uint64_t>(2 * j * hd * 2);
     auto sgpr = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
@@ -350,30 +350,32 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     }
 #endif
 #pragma unroll
-    for (int m = 0; m < MRT; ++m) {
-      l_acc[m][0] = R.l[4 * m];
-      m_neg[m] = R.mneg[m];
-      m_thr[m] = R.mthr[m];
+    for (int rg = 0; rg < NRG; ++rg) {
+      l_part[rg] = R.lsum[rg];
+      m_neg[rg] = R.mneg[rg];
+      m_thr[rg] = R.mthr[rg];
 #pragma unroll
-      for (int c = 0; c < C::CB; ++c)
+      for (int blk = 0; blk < C::NBLK; ++blk)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          o_acc[m][c][r] = (m == 0 ? R.o0 : m == 1 ? R.o1 : m == 2 ? R.o2 : R.o3)[4 * c + r];
+        for (int k = 0; k < 16; ++k) {
+          const int idx = 16 * (blk & 1) + k;
+          o_acc[rg][blk][k] = rg == 0 ? (blk < 2 ? R.o0[idx] : R.o1[idx]) : (blk < 2 ? R.o2[idx] : R.o3[idx]);
+        }
     }
   }
 
   // ---- normalise (with optional sinks) and store
 #pragma unroll
-  for (int m = 0; m < MRT; ++m) {
+  for (int rg = 0; rg < NRG; ++rg) {
     bool valid;
     int head;
     size_t q_off;
     int opaque0 = 0;
     asm volatile("" : "+v"(opaque0));
-    row_of(m, opaque0, valid, head, q_off);
+    row_of(rg, opaque0, valid, head, q_off);
+    const float l_run = l_part[rg] + __shfl_xor(l_part[rg], 32, kWave);  // the two lanes of a row hold half its keys each
     if (!valid) continue;
-    const float l_run = l_acc[m][0];
-    const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+    const float m_row = m_thr[rg] == -INFINITY ? -INFINITY : -m_neg[rg] * (1.f / kLog2e);
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
@@ -387,14 +389,16 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     }
     const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
     bf16_t* orow = out + q_off;
-    // MFMA c holds head_dim elements 16 c + 4 g + r of this lane's row
+    // register 4 q + r of block blk holds head_dim element 32 blk + 8 q + 4 g + r of this lane's row
 #pragma unroll
-    for (int c = 0; c < C::CB; ++c) {
-      u32x2_t w;
-      w[0] = pack_bf16x2(o_acc[m][c][0] * inv, o_acc[m][c][1] * inv);
-      w[1] = pack_bf16x2(o_acc[m][c][2] * inv, o_acc[m][c][3] * inv);
-      *reinterpret_cast<u32x2_t*>(orow + 16 * c + 4 * g) = w;
-    }
+    for (int blk = 0; blk < C::NBLK; ++blk)
+#pragma unroll
+      for (int qq = 0; qq < 4; ++qq) {
+        u32x2_t w;
+        w[0] = pack_bf16x2(o_acc[rg][blk][4 * qq] * inv, o_acc[rg][blk][4 * qq + 1] * inv);
+        w[1] = pack_bf16x2(o_acc[rg][blk][4 * qq + 2] * inv, o_acc[rg][blk][4 * qq + 3] * inv);
+        *reinterpret_cast<u32x2_t*>(orow + 32 * blk + 8 * qq + 4 * g) = w;
+      }
   }
 #ifdef RPA_PP_PROF2
   if ((threadIdx.x & (kWave - 1)) == 0) {
