@@ -1,11 +1,13 @@
-"""JAX entry point: the op as an XLA FFI custom call (``jax.ffi``) over ``librpa_mi355x.so``.
+"""JAX entry points: the ops as XLA FFI custom calls (``jax.ffi``) over ``librpa_mi355x.so``.
 
 Importing this module needs JAX with a ROCm backend.  It compiles ``csrc/rpa_xla_ffi.cc``
-against the FFI headers inside jaxlib (``jax.ffi.include_dir()``), registers the handler
+against the FFI headers inside jaxlib (``jax.ffi.include_dir()``), registers the handlers
 for platform ``"ROCM"`` and exposes ``ragged_page_attention`` with the reference's
-signature (ejkernel/modules/operations/ragged_page_attention.py:540-562), traceable under
-``jax.jit``.  Like the reference's native call (ejkernel/callib/_triton_call.py:760-799)
-it is forward-only: no JVP and no batching rule.
+signature (ejkernel/modules/operations/ragged_page_attention.py:540-562), plus
+``ragged_page_attention_v3`` (cache donated and returned, as the reference's jitted program does,
+ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:110-126), ``page_attention`` and
+``ragged_decode_attention``, all traceable under ``jax.jit``.  Like the reference's native call
+(ejkernel/callib/_triton_call.py:760-799) they are forward-only: no JVP and no batching rule.
 
 This image has no JAX, so this module has not been built or run here; the torch-tensor
 entry point in ``ejkernel_amd.modules`` is the tested one.  Both go through the same C ABI.
@@ -27,6 +29,8 @@ from .modules.operations.configs import RaggedPageAttentionConfig
 
 _FFI_LIB = LIB_DIR / "librpa_mi355x_xla_ffi.so"
 _TARGET = "mi355x_rpa_fwd"
+_TARGETS = {_TARGET: "RpaFwd", "mi355x_rpa_v3": "RpaV3", "mi355x_page_attention": "RpaPageAttn",
+            "mi355x_ragged_decode_attention": "RpaRaggedDecode"}
 _registered = False
 
 
@@ -46,7 +50,8 @@ def _register():
     if not _FFI_LIB.exists():
         build_ffi()
     lib = ctypes.CDLL(str(_FFI_LIB))
-    jax.ffi.register_ffi_target(_TARGET, jax.ffi.pycapsule(lib.RpaFwd), platform="ROCM")
+    for target, symbol in _TARGETS.items():
+        jax.ffi.register_ffi_target(target, jax.ffi.pycapsule(getattr(lib, symbol)), platform="ROCM")
     _registered = True
 
 
@@ -63,11 +68,6 @@ def ragged_page_attention(queries, kv_pages, context_lens, block_tables, query_s
     total_tokens, num_q_heads, head_dim = queries.shape
     num_pages, page_size, combined, _ = kv_pages.shape
     max_num_seqs, pages_per_seq = block_tables.shape
-    dims = _native.RpaParams()
-    dims.total_tokens, dims.num_q_heads, dims.num_kv_heads, dims.head_dim = total_tokens, num_q_heads, combined // 2, head_dim
-    dims.page_size, dims.num_pages, dims.max_num_seqs, dims.pages_per_seq = page_size, num_pages, max_num_seqs, pages_per_seq
-    dims.softmax_scale = 1.0
-    ws_bytes = int(_native.load().rpa_workspace_bytes(ctypes.byref(dims)))
     if not isinstance(num_seqs, jax.Array):
         num_seqs = jnp.asarray([num_seqs], dtype=jnp.int32)
     operands = [queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs]
@@ -78,11 +78,8 @@ def ragged_page_attention(queries, kv_pages, context_lens, block_tables, query_s
         elif aux.shape[0] != num_q_heads:
             aux = jnp.repeat(aux, num_q_heads // aux.shape[0], axis=0)
         operands.append(aux)
-    call = jax.ffi.ffi_call(
-        _TARGET,
-        (jax.ShapeDtypeStruct(queries.shape, queries.dtype), jax.ShapeDtypeStruct((ws_bytes,), jnp.uint8)),
-    )
-    out, _ = call(
+    call = jax.ffi.ffi_call(_TARGET, jax.ShapeDtypeStruct(queries.shape, queries.dtype))
+    out = call(
         *operands,
         softmax_scale=np.float32(head_dim**-0.5 if softmax_scale is None else softmax_scale),
         logits_soft_cap=np.float32(0.0 if logits_soft_cap is None else logits_soft_cap),
@@ -94,3 +91,45 @@ def ragged_page_attention(queries, kv_pages, context_lens, block_tables, query_s
         num_stages=np.int32(cfg.num_stages or 0),
     )
     return out
+
+
+def ragged_page_attention_v3(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution, /, *,
+                             softmax_scale=None, sliding_window=None, logits_soft_cap=None, q_scale=None, k_scale=None,
+                             v_scale=None):
+    """Cache update + attention; returns ``(out, kv_cache)`` with the cache updated in place (operand 3 is aliased to
+    the second result, so jit the caller with the cache donated as the reference does)."""
+    _register()
+    call = jax.ffi.ffi_call(
+        "mi355x_rpa_v3",
+        (jax.ShapeDtypeStruct(queries.shape, queries.dtype), jax.ShapeDtypeStruct(kv_cache.shape, kv_cache.dtype)),
+        input_output_aliases={3: 1},
+    )
+    f32 = lambda x: np.float32(0.0 if x is None else x)  # noqa: E731
+    return call(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution,
+                softmax_scale=np.float32(queries.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale),
+                logits_soft_cap=f32(logits_soft_cap), q_scale=f32(q_scale), k_scale=f32(k_scale), v_scale=f32(v_scale),
+                sliding_window=np.int32(0 if sliding_window is None else sliding_window))
+
+
+def page_attention(query, key_cache, value_cache, context_lens, block_tables, /, *, attn_scale=None):
+    """One query token per sequence over separate paged K and V caches ``[blocks, kv heads, block, head_dim]``."""
+    _register()
+    call = jax.ffi.ffi_call("mi355x_page_attention", jax.ShapeDtypeStruct(query.shape, query.dtype))
+    return call(query, key_cache, value_cache, context_lens, block_tables,
+                attn_scale=np.float32(query.shape[-1] ** -0.5 if attn_scale is None else attn_scale))
+
+
+def ragged_decode_attention(query, key, value, sequence_start, sequence_end, softmax_aux=None, /, *, softmax_scale=None,
+                            logits_soft_cap=None, sliding_window=None):
+    """One query token per sequence over contiguous K and V ``[batch, seq_len, kv heads, head_dim]``; ``sliding_window``
+    is ``(left, right)`` as in the reference, of which the left part applies to a decode step."""
+    _register()
+    operands = [query, key, value, sequence_start, sequence_end]
+    if softmax_aux is not None:
+        aux = jnp.asarray(softmax_aux, jnp.float32)
+        operands.append(aux[None] if aux.ndim == 1 else aux)
+    call = jax.ffi.ffi_call("mi355x_ragged_decode_attention", jax.ShapeDtypeStruct(query.shape, query.dtype))
+    return call(*operands,
+                softmax_scale=np.float32(query.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale),
+                logits_soft_cap=np.float32(0.0 if logits_soft_cap is None else logits_soft_cap),
+                window_left=np.int32(-1 if sliding_window is None else int(sliding_window[0])))
