@@ -221,3 +221,4 @@ def test_hbm_traffic_file_is_well_formed():
         assert name in WORKLOADS
         want = (e["fetch_size_kib"] * e["fetch_scale"] + e["write_size_kib"] * e["write_scale"]) * 1024.0
         assert abs(e["bytes"] - want) <= 1e-6 * want
+

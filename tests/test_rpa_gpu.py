@@ -472,6 +472,23 @@ def test_concurrent_streams_do_not_share_a_workspace():
             assert torch.equal(o, alone[k])
 
 
+def test_workspace_cache_is_bounded_over_many_streams():
+    """Every (device, stream) gets its own workspace; past the bound the least recently used one is dropped, and a call on
+    a stream whose workspace was dropped allocates (and clears) a new one."""
+    import importlib
+
+    m = importlib.import_module("ejkernel_amd.modules.operations.ragged_page_attention")
+    b = small([1, 3, 1], [300, 90, 17])
+    want = to_np(run_hip(b))
+    streams = [torch.cuda.Stream() for _ in range(m._MAX_WORKSPACES + 4)]
+    for st in streams + streams[:2]:
+        with torch.cuda.stream(st):
+            out = RaggedPageAttention().run(*b.args(), softmax_scale=b.softmax_scale, cfg=RaggedPageAttentionConfig())
+        st.synchronize()
+        assert np.array_equal(to_np(out), want)
+        assert len(m._workspaces) <= m._MAX_WORKSPACES
+
+
 def test_launch_recorded_in_a_hip_graph_replays_correctly():
     """The launch only enqueues (no allocation, no synchronisation, tickets and queue counters left at zero), so it can
     be captured; every replay on new input values must equal the eager result bit for bit."""
