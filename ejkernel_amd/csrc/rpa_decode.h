@@ -367,27 +367,33 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
     // Who writes, who reads: this wavefront writes its slot; the wavefront that draws the last ticket of the
     // (sequence, kv head) -- any workgroup, usually on another XCD with another L2 -- reads every slot.  Partials are
-    // written and read with agent-scope relaxed atomics, i.e. write-through stores and cache-bypassing loads that
-    // meet in memory-side storage, so no L2 write-back or invalidate is needed around the ticket.  What the hand-off
-    // needs is order: every store of this wavefront must have completed before its ticket increment can be seen.
-    // The explicit s_waitcnt vmcnt(0) below provides that (on gfx9 stores count in vmcnt, and a store leaves the
-    // counter when it has been acknowledged by the level its scope bits write through to); the fences beside it only
-    // keep the compiler from moving memory operations across.  The reader orders itself by data dependence: its
-    // loads are issued after the ticket value has come back and been compared.
-    const size_t slot = static_cast<size_t>(part.slot);
+    // written and read at agent scope (sc1): write-through stores and loads that do not hit in a non-coherent L2 meet
+    // in memory-side storage, so no L2 write-back or invalidate is needed around the ticket.  The row statistics and
+    // the ticket are relaxed atomics; the accumulators are 16-byte buffer accesses that carry the same scope bit
+    // (atomics end at eight bytes, and eight-byte accesses cost a memory burst each: with 8 rows at head_dim 256 they
+    // took a tenth of the kernel).  What the hand-off needs beyond that is order: every store of this wavefront must
+    // have completed before its ticket increment can be seen.  The explicit s_waitcnt vmcnt(0) below provides that (on
+    // gfx9 stores count in vmcnt, and a store leaves the counter when it has been acknowledged by the level its scope
+    // bits write through to); the fences beside it only keep the compiler from moving memory operations across.  The
+    // reader orders itself by data dependence: its loads are issued after the ticket value has come back and been
+    // compared.
+    //
+    // The accumulators travel as they sit in registers: piece n (= 8 * slice + MFMA number) of row i, lane group g, is
+    // the 16 bytes at ((n * 16 + i) * 4 + g) * 16 of the slot, so one store covers 64 contiguous bytes per valid row.
+    const size_t slot = static_cast<size_t>(__builtin_amdgcn_readfirstlane(part.slot));
+    constexpr int kAgentScope = 16;  // auxiliary bit 4 of a buffer access: sc1, coherent across the device's L2s
+    const __amdgpu_buffer_rsrc_t slots_rsrc = __builtin_amdgcn_make_buffer_rsrc(a.partial_o, 0, 0x7fffffff, 0x00020000);
+    auto slot_piece = [&](uint32_t sl, int n, int row) -> int {
+      return static_cast<int>(sl * static_cast<uint32_t>(16 * D * 4) + static_cast<uint32_t>(((n * 16 + row) * 4 + g) * 16));
+    };
     if (row_valid) {
-      uint64_t* po = reinterpret_cast<uint64_t*>(a.partial_o + (slot * 16 + i) * D);
       if constexpr (kPass != 1)
 #pragma unroll
-      for (int sN = 0; sN < C::NS; ++sN)
+        for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const uint64_t v = static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e][r])) |
-                               (static_cast<uint64_t>(__float_as_uint(o_acc[sN][2 * e + 1][r])) << 32);
-            __hip_atomic_store(po + (128 * sN + 32 * g + 8 * r) / 2 + e, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          }
+          for (int c = 0; c < 8; ++c)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, o_acc[sN][c]), slots_rsrc,
+                                                   slot_piece(static_cast<uint32_t>(slot), sN * 8 + c, i), 0, kAgentScope);
       if (g == 0) {
         const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_run)) | (static_cast<uint64_t>(__float_as_uint(l_run)) << 32);
         __hip_atomic_store(reinterpret_cast<uint64_t*>(a.partial_ml) + slot * 16 + i, v, __ATOMIC_RELAXED,
@@ -439,21 +445,18 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       if (rv) {
         for (int k0 = part.first_w; k0 <= part.last_w; k0 += kChunk * pp) {
           uint64_t mlv[kChunk];
-          uint64_t ov[kChunk][C::NS][4][4];
+          u32x4_t ov[kChunk][C::NS][8];
 #pragma unroll
           for (int c = 0; c < kChunk; ++c) {
             const size_t sl = part_slot(min(k0 + c * pp + sub, part.last_w), part.stream_a, part.sh);
             mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + rrow) * D);
             if constexpr (kPass != 1)
 #pragma unroll
             for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                  ov[c][sN][r][e] = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
-                                                      __HIP_MEMORY_SCOPE_AGENT);
+              for (int cc = 0; cc < 8; ++cc)
+                ov[c][sN][cc] = __builtin_amdgcn_raw_buffer_load_b128(slots_rsrc, slot_piece(static_cast<uint32_t>(sl), sN * 8 + cc, rrow),
+                                                                      0, kAgentScope);
           }
 #pragma unroll
           for (int c = 0; c < kChunk; ++c) {
@@ -466,12 +469,9 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
             for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)
+              for (int cc = 0; cc < 8; ++cc)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                  o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e]));
-                  o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e] >> 32));
-                }
+                for (int r = 0; r < 4; ++r) o_acc[sN][cc][r] += w * __uint_as_float(ov[c][sN][cc][r]);
           }
         }
       }
@@ -513,21 +513,18 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     if (row_valid) {
       for (int k0 = part.first_w; k0 <= part.last_w; k0 += kMergeChunk) {
         uint64_t mlv[kMergeChunk];
-        uint64_t ov[kMergeChunk][C::NS][4][4];
+        u32x4_t ov[kMergeChunk][C::NS][8];
 #pragma unroll
         for (int c = 0; c < kMergeChunk; ++c) {
           const size_t sl = part_slot(min(k0 + c, part.last_w), part.stream_a, part.sh);
           mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const uint64_t* src = reinterpret_cast<const uint64_t*>(a.partial_o + (sl * 16 + i) * D);
           if constexpr (kPass != 1)
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
-#pragma unroll
-              for (int e = 0; e < 4; ++e)
-                ov[c][sN][r][e] = __hip_atomic_load(src + (128 * sN + 32 * g + 8 * r) / 2 + e, __ATOMIC_RELAXED,
-                                                    __HIP_MEMORY_SCOPE_AGENT);
+            for (int cc = 0; cc < 8; ++cc)
+              ov[c][sN][cc] = __builtin_amdgcn_raw_buffer_load_b128(slots_rsrc, slot_piece(static_cast<uint32_t>(sl), sN * 8 + cc, i), 0,
+                                                                    kAgentScope);
         }
 #pragma unroll
         for (int c = 0; c < kMergeChunk; ++c) {
@@ -540,12 +537,9 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-            for (int r = 0; r < 4; ++r)
+            for (int cc = 0; cc < 8; ++cc)
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                o_acc[sN][2 * e][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e]));
-                o_acc[sN][2 * e + 1][r] += w * __uint_as_float(static_cast<uint32_t>(ov[c][sN][r][e] >> 32));
-              }
+              for (int r = 0; r < 4; ++r) o_acc[sN][cc][r] += w * __uint_as_float(ov[c][sN][cc][r]);
         }
       }
     }

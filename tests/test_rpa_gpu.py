@@ -478,7 +478,7 @@ def test_workspace_cache_is_bounded_over_many_streams():
     import importlib
 
     m = importlib.import_module("ejkernel_amd.modules.operations.ragged_page_attention")
-    b = small([1, 3, 1], [300, 90, 17])
+    b = small([1, 3, 1], [100, 90, 17])
     want = to_np(run_hip(b))
     streams = [torch.cuda.Stream() for _ in range(m._MAX_WORKSPACES + 4)]
     for st in streams + streams[:2]:
