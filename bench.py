@@ -65,6 +65,12 @@ def parse():
     ap.add_argument("--copy-probe", type=int, default=0, metavar="MIB",
                     help="instead of the benchmark, run a plain device copy of MIB MiB --steps times (a kernel of "
                          "known traffic, used to scale the FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--sustain", type=float, default=0.0, metavar="SECONDS",
+                    help="instead of the benchmark, launch the workload (or the --gemm-probe product) back to back for "
+                         "SECONDS and print the time per launch with the board's power sensor and power cap (hwmon)")
+    ap.add_argument("--gemm-probe", type=int, default=0, metavar="N",
+                    help="instead of the benchmark, time the vendor library's bf16 N x N x N matrix product (what the "
+                         "matrix cores of this box sustain under its power limit; context for the MFMA-bound figures)")
     return ap.parse_args()
 
 
@@ -341,6 +347,73 @@ def roofline_of(counts, ev_ms):
     return roof
 
 
+def library_gemm_tflops(n=8192, reps=10):
+    """bf16 n x n x n product of the vendor library (hipBLASLt through torch), best and median of `reps` timed calls.
+    Not a baseline of this op: it shows how far below the published matrix peak a plain GEMM runs on the same box, in
+    the same process, minutes apart -- long MFMA-bound kernels are held by the power limit, and boxes differ."""
+    import torch
+
+    a = torch.randn(n, n, device="cuda:0", dtype=torch.bfloat16)
+    b = torch.randn(n, n, device="cuda:0", dtype=torch.bfloat16)
+    for _ in range(3):
+        a @ b
+    torch.cuda.synchronize()
+    ts = []
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        a @ b
+        e1.record()
+        torch.cuda.synchronize()
+        ts.append(e0.elapsed_time(e1))
+    ts.sort()
+    flops = 2.0 * n ** 3
+    return {"n": n, "median": flops / ts[len(ts) // 2] / 1e9, "best": flops / ts[0] / 1e9}
+
+
+def board_power_watts():
+    """(power drawn now, power cap) of the first GPU from the driver's hwmon files, in watts; None where unreadable."""
+    import glob
+
+    def read(pattern):
+        for f in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/" + pattern)):
+            try:
+                return int(open(f).read()) / 1e6
+            except (OSError, ValueError):
+                pass
+        return None
+
+    now = read("power1_input")
+    return (now if now is not None else read("power1_average")), read("power1_cap")
+
+
+def sustain(fn, seconds, what, flops=None, nbytes=None):
+    """Back-to-back launches of `fn` for `seconds`; the power sensor is read between batches of 50 launches."""
+    import torch
+
+    idle = board_power_watts()[0]
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n, watts = 0, []
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(50):
+            fn()
+        torch.cuda.synchronize()
+        n += 50
+        watts.append(board_power_watts()[0])
+    ms = (time.perf_counter() - t0) / n * 1e3
+    watts = sorted(w for w in watts if w is not None)
+    res = {"sustain": what, "seconds": seconds, "launches": n, "ms_per_launch": ms, "power_idle_w": idle,
+           "power_w_median": watts[len(watts) // 2] if watts else None, "power_cap_w": board_power_watts()[1]}
+    if flops:
+        res["tflops"] = flops / ms / 1e9
+    if nbytes:
+        res["gbps"] = nbytes / ms / 1e6
+    print(json.dumps(res))
+
+
 def measure_config(name, steps, warmup, want_parity):
     """One entry of "configs": the named workload at full size, timed like the headline one and checked against the
     CPU restatement on a small sample of its sequences."""
@@ -361,6 +434,8 @@ def measure_config(name, steps, warmup, want_parity):
     ms_per_step, ev_ms, out = time_steps(step, steps, warmup)
     roof = roofline_of(counts, ev_ms)
     roof["traffic"] = measured_traffic_bytes(name)
+    if roof["bound"] == "mfma":
+        roof["library_gemm_tflops"] = library_gemm_tflops()
     entry = {"workload": name, "ms_per_step": ms_per_step, "kernel_ms_avg": roof["kernel_ms_avg"],
              "tokens_per_s": counts["tokens"] / (ms_per_step * 1e-3), "roofline": roof,
              "host_overhead_ms": ms_per_step - roof["kernel_ms_avg"]}
@@ -407,6 +482,14 @@ def main():
     dev = "cuda:0"
     if args.op in ("page_attention", "ragged_decode"):
         return page_attention_main(args)
+    if args.gemm_probe and args.sustain > 0:
+        n = args.gemm_probe
+        ga = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+        gb = torch.randn(n, n, device=dev, dtype=torch.bfloat16)
+        return sustain(lambda: ga @ gb, args.sustain, f"library bf16 GEMM {n}^3", flops=2.0 * n ** 3)
+    if args.gemm_probe:
+        print(json.dumps({"gemm_probe": library_gemm_tflops(args.gemm_probe, max(args.steps, 3)), "unit": "TFLOP/s", "dtype": "bf16"}))
+        return
     if args.copy_probe:
         n = args.copy_probe << 20
         src = torch.full((n,), 7, dtype=torch.uint8, device=dev)
@@ -445,11 +528,15 @@ def main():
             return ragged_page_attention_v3(*v3.args(), **v3.kwargs())[0]
         return ragged_page_attention(*batch.args(), **batch.kwargs())
 
+    if args.sustain > 0:
+        return sustain(step, args.sustain, args.workload, flops=counts["flops"], nbytes=counts["bytes"])
     ms_per_step, ev_ms, out = time_steps(step, args.steps, args.warmup)
     kernel_ms = sum(ev_ms) / len(ev_ms)
     tokens = counts["tokens"]
     roof = roofline_of(counts, ev_ms)
     roof["traffic"] = measured_traffic_bytes(args.workload) if args.scale == 1.0 and v3 is None else None
+    if roof["bound"] == "mfma" and args.scale == 1.0:
+        roof["library_gemm_tflops"] = library_gemm_tflops()
     gbps, tflops = roof["gbps"], roof["tflops"]
 
     line = {
