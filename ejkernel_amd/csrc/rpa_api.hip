@@ -312,6 +312,16 @@ int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stre
   if (p.workspace == nullptr || p.workspace_bytes < w.total)
     return rpa::fail(RPA_ERR_WORKSPACE, "workspace of %llu bytes is too small, rpa_ragged_decode_workspace_bytes() asks for %llu",
                      (unsigned long long)p.workspace_bytes, (unsigned long long)w.total);
+  if (tiled) {
+    // the attention kernel walks the sink keys itself, in the wavefront that finishes each (sequence, kv head)
+    rpa::PreState sinks;
+    sinks.sink_aux = params->softmax_aux;
+    sinks.sink_n = params->num_sinks;
+    sinks.sink_rows = params->aux_rows;
+    sinks.sink_limit = params->seq_len;
+    return rpa::dispatch(p, kv, true, stream, sinks);
+  }
+  // the scalar kernel: a pre-pass accumulates the sink keys into an attention state that it merges into every row
   char* ws = static_cast<char*>(p.workspace);
   rpa::SinkKeyArgs sk;
   sk.aux = params->softmax_aux;

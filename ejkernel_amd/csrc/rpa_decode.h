@@ -15,6 +15,8 @@ struct Cfg {
   static constexpr int NSLOT = 4 * NT;      // tokens each lane fetches per iteration
   static constexpr int ROWB = D * 2 + 16;   // LDS bytes per K row (16 B pad: conflict-free b128 reads)
   static constexpr int LDS_PER_WAVE = TT * ROWB;
+  static constexpr int SINK_KEYS = 8;                   // sink keys of ragged_decode_attention staged in LDS per wavefront
+  static constexpr int SINK_LDS = SINK_KEYS * 2 * D * 2 + 16 * SINK_KEYS * 4;  // their K rows, their V rows, 16 rows of biases
 };
 
 // Cache element types (kKv): 0 = the query dtype (bf16); 8-bit floats of the OCP formats: 1 = e4m3 (finite, no
@@ -351,6 +353,48 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       }
   };
 
+  // Sink keys of ragged_decode_attention: the part that starts a (sequence, kv head) also takes the keys
+  // [first, first + sink_n) below sink_limit, which are visible whatever the window and the end of the sequence say and
+  // carry the row's bias on positions below sink_n (si.start lies behind them, so the stream leaves them out).  Their K
+  // and V rows -- the first SINK_KEYS of them -- go straight to this wavefront's LDS now, without registers, and are
+  // used after the stream, when they have long arrived: the online softmax simply goes on over them.
+  bool sink_part = false;
+  int sink_first = 0, sink_keys = 0;
+  char* lds_sink = lds_k + (kWgWaves - static_cast<int>(threadIdx.x) / kWave) * C::LDS_PER_WAVE +
+                   (static_cast<int>(threadIdx.x) / kWave) * C::SINK_LDS;
+  auto sink_row = [&](int t) -> const char* {
+    int page = a.kv.contiguous ? s : bt[t >> a.page_shift];
+    page = min(max(page, 0), p.num_pages - 1);
+    return kvb + static_cast<uint64_t>(page) * page_b + static_cast<uint64_t>(t & (p.page_size - 1)) * stride_b + head_off;
+  };
+  if constexpr (kWaveOnly && kPass == 0 && kKv == 0) {
+    if (a.pre.sink_aux != nullptr && (!part.partial || range_lo == si.lo_al)) {
+      sink_first = kv_start_of(p, s);
+      sink_keys = max(0, min(a.pre.sink_n, a.pre.sink_limit - sink_first));
+      sink_part = sink_keys > 0;
+      if (sink_part) {
+        // one wave-wide load of 16 bytes per lane covers 64 / (hd / 8) whole rows, laid out row after row
+        const int pieces = hd >> 3, rows_per = kWave / pieces;
+        const int staged = min(sink_keys, C::SINK_KEYS);
+        for (int r0 = 0; r0 < staged; r0 += rows_per) {
+          const char* src = sink_row(sink_first + min(r0 + lane / pieces, staged - 1)) + 16 * (lane % pieces);
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(src),
+                                           (__attribute__((address_space(3))) void*)(lds_sink + r0 * hd * 2), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(src + v_delta),
+                                           (__attribute__((address_space(3))) void*)(lds_sink + (C::SINK_KEYS + r0) * hd * 2), 16, 0, 0);
+        }
+        // the biases of those positions, [bias row][key]: 4 bytes per lane, 8 rows per load
+#pragma unroll
+        for (int rr = 0; rr < 2; ++rr) {
+          const int brow = min(8 * rr + (lane >> 3), a.pre.sink_rows - 1);
+          const int bt_ = min(sink_first + (lane & 7), a.pre.sink_n - 1);
+          __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(a.pre.sink_aux + static_cast<size_t>(brow) * a.pre.sink_n + bt_),
+                                           (__attribute__((address_space(3))) void*)(lds_sink + C::SINK_KEYS * 2 * D * 2 + rr * 256), 4, 0, 0);
+        }
+      }
+    }
+  }
+
   if (range_hi > range_lo) {
     issue_loads(range_lo, kreg, vbuf0);
     for (int tile = range_lo; tile < range_hi; tile += 2 * C::TT) {
@@ -362,6 +406,84 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 
   // ---- row sum across the four lane groups
   if constexpr (kPass != 2) l_run = row_groups_sum(l_run);
+
+  if constexpr (kWaveOnly && kPass == 0 && kKv == 0) {
+    if (sink_part) {
+      // Lane (row i, group g) holds q[32 ks + 8 g ..] and the outputs d = 128 sN + 32 g + 8 r + c: it takes those pieces
+      // of a sink key's K and V rows, and the four groups of a row add up their parts of the dot product.
+      const int bias_row = a.pre.sink_rows == 1 ? 0 : hg;
+      const float* __restrict__ bias = a.pre.sink_aux + static_cast<size_t>(bias_row) * a.pre.sink_n;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // the rows staged in LDS have arrived
+      for (int k = 0; k < sink_keys; ++k) {
+        const int t = sink_first + k;
+        u32x4_t kk[C::NKS], vv[C::NS][4];
+#pragma unroll
+        for (int ks = 0; ks < C::NKS; ++ks) kk[ks] = u32x4_t{0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) vv[sN][r] = u32x4_t{0u, 0u, 0u, 0u};
+        if (k < C::SINK_KEYS) {
+          const char* krow = lds_sink + k * hd * 2;
+          const char* vrow = krow + C::SINK_KEYS * hd * 2;
+#pragma unroll
+          for (int ks = 0; ks < C::NKS; ++ks)
+            if (32 * ks < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (128 * sN + 32 * g + 8 * r < hd) vv[sN][r] = *reinterpret_cast<const u32x4_t*>(vrow + 2 * (128 * sN + 32 * g + 8 * r));
+        } else {
+          // more sinks than the staged ones: from memory, one key at a time
+          const char* krow = sink_row(t);
+          const char* vrow = krow + v_delta;
+#pragma unroll
+          for (int ks = 0; ks < C::NKS; ++ks)
+            if (32 * ks < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+              if (128 * sN + 32 * g + 8 * r < hd) vv[sN][r] = *reinterpret_cast<const u32x4_t*>(vrow + 2 * (128 * sN + 32 * g + 8 * r));
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < C::NKS; ++ks) {
+          const u32x4_t qq = __builtin_bit_cast(u32x4_t, qreg[ks]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            dot = fmaf(__uint_as_float(qq[e] << 16), __uint_as_float(kk[ks][e] << 16), dot);
+            dot = fmaf(__uint_as_float(qq[e] & 0xffff0000u), __uint_as_float(kk[ks][e] & 0xffff0000u), dot);
+          }
+        }
+        dot += __shfl_xor(dot, 16, kWave);
+        dot += __shfl_xor(dot, 32, kWave);
+        float sc = kMimic ? rbf(dot) : dot * post_scale;
+        if (cap != 0.f) sc = soft_cap<kMimic>(sc, cap, inv_cap);
+        if (t < a.pre.sink_n)
+          sc += k < C::SINK_KEYS ? *reinterpret_cast<const float*>(lds_sink + C::SINK_KEYS * 2 * D * 2 + (C::SINK_KEYS * bias_row + k) * 4)
+                                 : bias[t];
+        const float m_new = fmaxf(m_run, sc);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a bias of -inf takes its key out
+        const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
+        float d = sc - m_use;
+        if (kMimic) d = rbf(d);
+        const float e = rbf(__builtin_amdgcn_exp2f(d * kLog2e));
+        l_run = l_run * alpha + e;
+        m_run = m_new;
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              o_acc[sN][2 * c][r] = fmaf(e, __uint_as_float(vv[sN][r][c] << 16), o_acc[sN][2 * c][r] * alpha);
+              o_acc[sN][2 * c + 1][r] = fmaf(e, __uint_as_float(vv[sN][r][c] & 0xffff0000u), o_acc[sN][2 * c + 1][r] * alpha);
+            }
+      }
+    }
+  }
 
   if (part.partial) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.

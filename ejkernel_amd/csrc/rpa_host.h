@@ -42,6 +42,12 @@ inline KvLayout interleaved_layout(const RpaParams& p) {
 struct PreState {
   const float* o = nullptr;   // [tokens, num_q_heads, head_dim]
   const float* ml = nullptr;  // [tokens, num_q_heads, 2]: maximum (-inf if no key), sum
+  // Or, instead of a state from an earlier kernel (tiled kernel only): the sink keys of ragged_decode_attention
+  // themselves.  The attention kernel then starts `sink_n` keys after kv_start[s] and the wavefront that finishes a
+  // (sequence, kv head) walks the keys [kv_start[s], kv_start[s] + sink_n) below `sink_limit` itself, with
+  // sink_aux[row][t] added to the logit of absolute position t < sink_n (_xla_impl_fwd.py:71-75, :98-134).
+  const float* sink_aux = nullptr;  // [sink_rows, sink_n]
+  int32_t sink_n = 0, sink_rows = 1, sink_limit = 0;
 };
 
 // Sink keys of ragged_decode_attention (_xla_impl_fwd.py:71-75, :98-134): accumulates, per (sequence, query head),

@@ -471,7 +471,7 @@ template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv =
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<(D < 128 ? 128 : D), NT, kMimic>;
   using PC = PCfg<D, MRT>;
-  const size_t data = max(static_cast<size_t>(kWgWaves) * C::LDS_PER_WAVE,
+  const size_t data = max(static_cast<size_t>(kWgWaves) * (C::LDS_PER_WAVE + (a.pre.sink_aux != nullptr ? C::SINK_LDS : 0)),
                           static_cast<size_t>(kPipeTile<D, MRT> ? PipeCfg::LDS : PC::LDS));
   const size_t lds = sched_bytes((a.p.max_num_seqs + (1 << a.sched_shift) - 1) >> a.sched_shift) + data;
   // More than 64 KiB of dynamic LDS has to be allowed once per kernel (and device); the call is idempotent.
@@ -546,7 +546,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   const KvLayout canon = interleaved_layout(p);
   const bool canonical = kv.k_base == canon.k_base && kv.v_base == canon.v_base && kv.stride_b == canon.stride_b &&
                          kv.head_b == canon.head_b && kv.page_b == canon.page_b && kv.contiguous == 0;
-  const bool wave_only = pre.ml != nullptr || !canonical || (small_batch && tune().no_wave_only == 0);
+  const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !canonical || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);

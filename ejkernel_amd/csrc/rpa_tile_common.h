@@ -112,7 +112,7 @@ __device__ __forceinline__ SeqInfo seq_info(const TileArgs& a, int s, int G) {
   si.rows = si.q_len * G;
   si.n_rt = (si.rows + 15) >> 4;
   const int pos_min = si.kv_len - si.q_len;
-  si.start = kv_start_of(p, s);
+  si.start = kv_start_of(p, s) + a.pre.sink_n;  // sink keys, if any, are walked apart from the stream
   int lo = p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0;
   lo = max(lo, si.start);
   si.lo_al = lo & ~(TT - 1);

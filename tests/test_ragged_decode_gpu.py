@@ -168,6 +168,21 @@ def test_bf16_sinks_against_the_reference_program_on_one_block(kw, flags):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("ns,kw", [(9, dict()), (24, dict(head_dim=64)), (64, dict(head_dim=256, num_q_heads=16, num_kv_heads=8)),
+                                   (33, dict(num_q_heads=32, num_kv_heads=2))], ids=["9", "24-d64", "64-d256", "33-g16"])
+def test_bf16_many_sinks_against_float64(flags, ns, kw):
+    """More sink keys than the attention kernel stages per wavefront (8): the rest is read key by key; per-head biases,
+    a sink range cut by seq_len (sequence 9) and by nothing else (sequences 2 and 8 are empty but for their sinks)."""
+    b = sink_batch(**kw)
+    G = b.query.shape[1] // b.key.shape[2]
+    aux = torch.randn(G, ns, generator=torch.Generator().manual_seed(ns)) * 2.0
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=(50, 0), softmax_aux=aux.numpy())
+    out = to_np(ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, sliding_window=(50, 0),
+                                        _flags=flags))
+    assert_bf16_parity(out, ref, len(SINK_ENDS), f"{ns} sinks {kw}")
+
+
+@pytest.mark.parametrize("flags", PATHS)
 def test_float32_sinks_against_float64(flags):
     b = sink_batch(dtype=torch.float32)
     aux = torch.tensor([[0.5, -1.0, 2.0]])
