@@ -83,7 +83,9 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const RpaParams& p = a.p;
   const int lane = threadIdx.x & (kWave - 1);
   const int i = lane & 15, g = lane >> 4;
-  const int G = p.num_q_heads / p.num_kv_heads;
+  const bool pair = kWaveOnly && kKv == 0 && kPass == 0 && a.pair != 0;  // two kv heads of head_dim 64 per item
+  const int G_head = p.num_q_heads / p.num_kv_heads;
+  const int G = pair ? 2 * G_head : G_head;  // query heads of the item: j counts head pairs then
   const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
   const int W = p.sliding_window;
@@ -99,6 +101,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const int hg = row_valid ? R - qi * G : 0;
   const int pos_n = row_valid ? si.kv_len - si.q_len + qi : -1;
   const int head = j * G + hg;
+  const int hp = pair && hg >= G_head ? 1 : 0;  // which head of the pair this row belongs to
   // head_dim 64 runs on the 128-wide instantiation: q is padded with zeros, the upper eight 16-byte pieces of a K / V
   // row repeat the lower eight (K: multiplied by zero; V: output elements that are not stored).
   const int hd = p.head_dim;
@@ -111,7 +114,12 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (row_valid && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
+      if (pair) {
+        // contraction index 64 hp .. 64 hp + 63 carries this row's query; the other head's half stays zero
+        if (row_valid && (ks >> 1) == hp) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * (ks & 1) + 8 * g);
+      } else if (row_valid && 32 * ks < hd) {
+        raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
+      }
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -174,9 +182,11 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const int64_t v_delta = a.kv.v_base - a.kv.k_base;  // the V row of a (token, head) relative to its K row
   const uint32_t stride_b = a.kv.stride_b;            // bytes between tokens
   const uint64_t page_b = a.kv.page_b;
-  const uint32_t head_off = static_cast<uint32_t>(j) * a.kv.head_b;
+  const uint32_t head_off = static_cast<uint32_t>(pair ? 2 * j : j) * a.kv.head_b;
   const int piece = i & (hd / 8 - 1);  // i itself from head_dim 128 up
-  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + head_off + PIECE_B * static_cast<uint32_t>(piece);
+  // this lane's piece inside a token's record; with a head pair, pieces 8..15 are those of the second head
+  const uint32_t piece_off = head_off + PIECE_B * static_cast<uint32_t>(piece) + (pair && i >= 8 ? a.kv.head_b : 0u);
+  const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + piece_off;
   auto issue_loads = [&](int tile, raw_t (&kr)[C::NSLOT][C::NS], raw_t (&vr)[C::NSLOT][C::NS]) {
     if (a.uniform_page && tile + C::TT <= range_hi) {
 #pragma unroll
@@ -206,7 +216,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       int page = a.kv.contiguous ? s : bt[t4c >> a.page_shift];
       page = min(max(page, 0), p.num_pages - 1);
       const char* base = kvb + static_cast<uint64_t>(page) * page_b +
-                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + (head_off + PIECE_B * piece);
+                         static_cast<uint64_t>(t4c & (p.page_size - 1)) * stride_b + piece_off;
 #pragma unroll
       for (int r = 0; r < 4; ++r) {
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
@@ -726,7 +736,12 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       u32x4_t w;
 #pragma unroll
       for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[sN][2 * e][r] * inv, o_acc[sN][2 * e + 1][r] * inv);
-      if (128 * sN + 32 * g + 8 * r < hd) *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+      const int d0 = 128 * sN + 32 * g + 8 * r;
+      if (pair) {
+        if ((d0 >> 6) == hp) *reinterpret_cast<u32x4_t*>(orow + (d0 & 63)) = w;  // the half that is this row's head
+      } else if (d0 < hd) {
+        *reinterpret_cast<u32x4_t*>(orow + d0) = w;
+      }
     }
 }
 

@@ -75,7 +75,10 @@ void rpa_tile_kernel(TileArgs a) {
   extern __shared__ __align__(16) char smem[];
   const RpaParams& p = a.p;
   const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / kWave);
-  const int G = p.num_q_heads / p.num_kv_heads;
+  // items of the wave-level loop: one per kv head, or one per pair of kv heads (TileArgs::pair) with both heads' rows
+  const bool pair = kWaveOnly && kKv == 0 && kPass == 0 && a.pair != 0;
+  const int G = (pair ? 2 : 1) * (p.num_q_heads / p.num_kv_heads);
+  const int item_heads = pair ? p.num_kv_heads / 2 : p.num_kv_heads;
   // Schedule arrays: exclusive prefix sums over the sequences, kept for every K-th sequence (K = 1 for batches of up
   // to kTiledMaxSeqs sequences); the sequences in between are walked when an entry is looked up.
   const int shift = a.sched_shift, K = 1 << shift;
@@ -94,9 +97,9 @@ void rpa_tile_kernel(TileArgs a) {
   // (more than kWaveItemMaxRowTiles row tiles), or wave-level items (everything else).
   auto classify = [&](const SeqInfo& si, int& tiles, int& items, int& wg_items) {
     tiles = items = wg_items = 0;
-    if (si.eligible) tiles = p.num_kv_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
+    if (si.eligible) tiles = item_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
     else if (!kWaveOnly && si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
-    else items = p.num_kv_heads * si.n_rt;
+    else items = item_heads * si.n_rt;
   };
   const int per = (((nseq + kWgThreads - 1) / kWgThreads + K - 1) >> shift) << shift;  // a multiple of K per thread
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
@@ -339,7 +342,7 @@ void rpa_tile_kernel(TileArgs a) {
         const int s = find(item_start, 0, w, s_base);
         const SeqInfo si = seq_info<C::TT>(a, s, G);
         const int local = w - s_base;
-        const int j = local % p.num_kv_heads, rt = local / p.num_kv_heads;
+        const int j = local % item_heads, rt = local / item_heads;
         const int row_hi = min(rt * 16 + 16, si.rows);
         const int pos_min = si.kv_len - si.q_len + (rt * 16) / G, pos_max = si.kv_len - si.q_len + (row_hi - 1) / G;
         const int range_hi = min(si.kv_len, pos_max + 1);
@@ -361,7 +364,7 @@ void rpa_tile_kernel(TileArgs a) {
           // parts, a few at a time: the sum is smallest near P = 3 sqrt(T), i.e. sqrt(T) / 3 tiles per part.
           int min_share = a.min_share_tiles;
           if constexpr (kWaveOnly) {
-            const float avg = static_cast<float>(total_tiles) / static_cast<float>(max(1, nseq * p.num_kv_heads));
+            const float avg = static_cast<float>(total_tiles) / static_cast<float>(max(1, nseq * item_heads));
             min_share = max(min_share, min(kMaxMinShareTiles, static_cast<int>(__builtin_sqrtf(avg) * (1.f / 3.f))));
           }
           if (q >= min_share) {
@@ -412,6 +415,7 @@ struct Tune {
   int no_mimic;            // RPA_TUNE_NO_MIMIC
   int no_wave_only;        // RPA_TUNE_NO_WAVE_ONLY
   int wave_only_rows;      // RPA_TUNE_WAVE_ONLY_ROWS
+  int no_pair64;           // RPA_TUNE_NO_PAIR64: head_dim 64 decodes one kv head per item (experiments)
   int pipe;                // RPA_TUNE_PIPE: 0 = never use the software-pipelined prefill tile (head_dim 128)
   int pipe_stream_wgs;     // RPA_TUNE_PIPE_STREAM_WGS: workgroups (of one per compute unit) that take the decode stream first
   int pipe_min_tokens_per_seq;  // RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ: average query tokens per sequence from which it is used
@@ -431,6 +435,7 @@ static const Tune& tune() {
     x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
     x.no_wave_only = env_int("RPA_TUNE_NO_WAVE_ONLY", 0);
     x.wave_only_rows = env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows);
+    x.no_pair64 = env_int("RPA_TUNE_NO_PAIR64", 0);
     x.pipe = env_int("RPA_TUNE_PIPE", 1);
     x.pipe_min_tokens_per_seq = max(1, env_int("RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ", 128));
     x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
@@ -503,6 +508,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = tune().phase_mode;
+  a.pair = 0;
   a.even_xcd_permille = tune().even_xcd_permille;
   // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
   // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes
@@ -548,6 +554,10 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
                          kv.head_b == canon.head_b && kv.page_b == canon.page_b && kv.contiguous == 0;
   const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !canonical || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
+    // head_dim 64: two kv heads per item where that keeps a decode token's rows in one 16-row tile
+    a.pair = p.head_dim == 64 && p.num_kv_heads % 2 == 0 && 2 * (p.num_q_heads / p.num_kv_heads) <= 16 && pre.ml == nullptr &&
+             pre.sink_aux == nullptr && tune().no_pair64 == 0;
+    if (a.pair) a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 1);
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);
     return mimic ? launch_cfg<256, 1, 1, true, true>(a, grid, stream) : launch_cfg<256, 1, 1, false, true>(a, grid, stream);

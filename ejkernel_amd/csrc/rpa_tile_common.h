@@ -34,6 +34,12 @@ struct TileArgs {
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
   float* stats;       // row maximum and row sum per (token, query head) of a two-launch call (null otherwise)
   PreState pre;       // state accumulated by an earlier kernel, merged by the wave-level loop (null: none)
+  // head_dim 64, instantiation without prefill tiles: a wave-level item covers two kv heads (2 j, 2 j + 1) at once.
+  // The 128-wide loop then reads, per token, [K of head 2j | K of head 2j+1] as one K row and the two V rows as one V
+  // row -- in the interleaved cache 512 contiguous bytes per token instead of two visits of 256 -- with the query
+  // rows of the first head zero in the second half of the contraction and vice versa; every row keeps the half of the
+  // output that belongs to its head.
+  int pair;
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the

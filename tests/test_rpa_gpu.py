@@ -157,6 +157,27 @@ def test_bf16_head_dims(flags, D):
     assert_bf16_parity(to_np(run_hip(b, flags)), run_strict(b), b.total_valid_tokens, f"D {D}")
 
 
+@pytest.mark.parametrize("hq,hkv", [(8, 2), (4, 4), (32, 4), (64, 8), (6, 3), (32, 2), (16, 8)])
+@pytest.mark.parametrize("window,cap,sinks", [(None, None, False), (40, 20.0, True)])
+def test_bf16_head_dim_64_two_kv_heads_per_item(hq, hkv, window, cap, sinks):
+    """head_dim 64 in the wave-level loop: with an even number of kv heads and at most 8 query heads per kv head, an
+    item covers two kv heads (their rows share a 16-row tile: 2, 8 or 16 rows per decode token here; 3 kv heads and 16
+    query heads per kv head keep one kv head per item).  Decode tokens, short chunks whose row tiles straddle tokens and
+    heads, a sequence without keys before its own token, split (sequence, head pair)s; the exact kernel as cross-check."""
+    b = small([1, 3, 1, 7, 1, 2], [300, 90, 1, 7, 511, 40], num_q_heads=hq, num_kv_heads=hkv, head_dim=64, pages_per_seq=32,
+              sliding_window=window, logits_soft_cap=cap)
+    aux = (torch.randn(hq, 2, generator=torch.Generator().manual_seed(5)) * 2).numpy() if sinks else None
+    ref = run_strict(b, softmax_aux=aux)
+    out = run_hip(b, softmax_aux=aux)
+    assert_bf16_parity(to_np(out), ref, b.total_valid_tokens, f"{hq}/{hkv} W={window} cap={cap} sinks={sinks}")
+    assert torch.equal(run_hip(b, softmax_aux=aux), out)
+    assert_bf16_parity(to_np(run_hip(b, _native.RPA_FLAG_FORCE_GENERIC, softmax_aux=aux)), ref, b.total_valid_tokens, "generic")
+    # one long sequence: every head pair is cut into many parts and merged
+    if window is None:
+        b = small([1], [8000], num_q_heads=hq, num_kv_heads=hkv, head_dim=64, pages_per_seq=512)
+        assert_bf16_parity(to_np(run_hip(b)), run_strict(b), 1, f"long {hq}/{hkv}")
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128), (8, 2, 64), (4, 4, 64)])
 @pytest.mark.parametrize("window", [None, 48])
