@@ -245,3 +245,19 @@ def test_xla_ffi_handlers_type_check_against_the_api_stand_in():
     assert len(symbols) == 4
     for symbol in symbols:
         assert f"XLA_FFI_DEFINE_HANDLER_SYMBOL({symbol}," in text, symbol
+
+
+def test_bench_power_sensor_and_gpu_count_guard():
+    """bench.py's board power reader returns watts or None (no GPU here: None, or whatever hwmon file exists), never
+    raises; more than one GPU is refused with a message, as this build measures one GPU only."""
+    import subprocess
+    import sys
+
+    import bench
+
+    now, cap = bench.board_power_watts()
+    assert (now is None or now >= 0.0) and (cap is None or cap > 0.0)
+    assert bench.SETTLE_S > 0
+    root = Path(__file__).resolve().parents[1]
+    r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=str(root))
+    assert r.returncode == 2 and "one GPU" in r.stderr
