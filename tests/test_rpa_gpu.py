@@ -176,6 +176,12 @@ def test_bf16_head_dim_64_two_kv_heads_per_item(hq, hkv, window, cap, sinks):
     if window is None:
         b = small([1], [8000], num_q_heads=hq, num_kv_heads=hkv, head_dim=64, pages_per_seq=512)
         assert_bf16_parity(to_np(run_hip(b)), run_strict(b), 1, f"long {hq}/{hkv}")
+    # pages shorter than a 16-token sub-tile (per-lane page look-up) and longer ones
+    for page in (4, 64):
+        # (the reference yields NaN where one of its 64-page KV blocks lies left of the window: no window on 4-token pages)
+        b = small([1, 2, 1], [301, 77, 130], num_q_heads=hq, num_kv_heads=hkv, head_dim=64, page_size=page,
+                  pages_per_seq=max(2, 512 // page), sliding_window=window if page == 64 else None, logits_soft_cap=cap)
+        assert_bf16_parity(to_np(run_hip(b)), run_strict(b), b.total_valid_tokens, f"page {page} {hq}/{hkv}")
 
 
 @pytest.mark.parametrize("flags", PATHS)
