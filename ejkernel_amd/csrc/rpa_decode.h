@@ -393,10 +393,11 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(src + v_delta),
                                            (__attribute__((address_space(3))) void*)(lds_sink + (C::SINK_KEYS + r0) * hd * 2), 16, 0, 0);
         }
-        // the biases of those positions, [bias row][key]: 4 bytes per lane, 8 rows per load
+        // the biases of those positions for the 16 rows of this row tile, [row][key]: 4 bytes per lane, 8 rows per load
 #pragma unroll
         for (int rr = 0; rr < 2; ++rr) {
-          const int brow = min(8 * rr + (lane >> 3), a.pre.sink_rows - 1);
+          const int rrow = max(min(row_lo + 8 * rr + (lane >> 3), si.rows - 1), 0);  // a row of the item (the last one repeats)
+          const int brow = a.pre.sink_rows == 1 ? 0 : rrow % G;               // its query head within the kv head
           const int bt_ = min(sink_first + (lane & 7), a.pre.sink_n - 1);
           __builtin_amdgcn_global_load_lds(reinterpret_cast<const uint32_t*>(a.pre.sink_aux + static_cast<size_t>(brow) * a.pre.sink_n + bt_),
                                            (__attribute__((address_space(3))) void*)(lds_sink + C::SINK_KEYS * 2 * D * 2 + rr * 256), 4, 0, 0);
@@ -472,7 +473,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         float sc = kMimic ? rbf(dot) : dot * post_scale;
         if (cap != 0.f) sc = soft_cap<kMimic>(sc, cap, inv_cap);
         if (t < a.pre.sink_n)
-          sc += k < C::SINK_KEYS ? *reinterpret_cast<const float*>(lds_sink + C::SINK_KEYS * 2 * D * 2 + (C::SINK_KEYS * bias_row + k) * 4)
+          sc += k < C::SINK_KEYS ? *reinterpret_cast<const float*>(lds_sink + C::SINK_KEYS * 2 * D * 2 + (C::SINK_KEYS * i + k) * 4)
                                  : bias[t];
         const float m_new = fmaxf(m_run, sc);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a bias of -inf takes its key out

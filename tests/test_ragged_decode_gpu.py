@@ -183,6 +183,19 @@ def test_bf16_many_sinks_against_float64(flags, ns, kw):
 
 
 @pytest.mark.parametrize("flags", PATHS)
+@pytest.mark.parametrize("hq,hkv,ns", [(40, 1, 5), (24, 2, 3), (40, 1, 11), (64, 2, 2)])
+def test_bf16_per_head_sinks_with_more_than_16_query_heads_per_kv_head(flags, hq, hkv, ns):
+    """More than 16 query heads per kv head: a decode token's rows take several 16-row tiles, and each tile needs the
+    bias rows of its own query heads (rows 16 and up once read those of rows 0..15: found by a sweep of new seeds)."""
+    b = sink_batch(num_q_heads=hq, num_kv_heads=hkv)
+    aux = torch.randn(hq // hkv, ns, generator=torch.Generator().manual_seed(hq + ns)) * 2.0
+    ref = ragged_decode_exact(*np_args(b), softmax_scale=b.softmax_scale, sliding_window=(60, 0), softmax_aux=aux.numpy())
+    out = to_np(ragged_decode_attention(*b.args(), aux.to(DEV), softmax_scale=b.softmax_scale, sliding_window=(60, 0),
+                                        _flags=flags))
+    assert_bf16_parity(out, ref, len(SINK_ENDS), f"{hq}/{hkv} with {ns} sinks per head")
+
+
+@pytest.mark.parametrize("flags", PATHS)
 def test_float32_sinks_against_float64(flags):
     b = sink_batch(dtype=torch.float32)
     aux = torch.tensor([[0.5, -1.0, 2.0]])
