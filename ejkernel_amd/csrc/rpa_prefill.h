@@ -23,6 +23,10 @@
 
 #include "rpa_tile_common.h"
 
+#ifndef RPA_ROUND_MIN_D
+#define RPA_ROUND_MIN_D 128  // smallest head_dim whose prefill tiles round their logits to bf16 (see the key loop)
+#endif
+
 namespace rpa {
 
 template <int D, int MRT>
@@ -403,9 +407,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               for (int r = 0; r < 4; ++r)  // the cap's own bf16 roundings make it sensitive to its input: round that too
                 sv[u][r] = soft_cap<kMimic>(kMimic ? rbf(sv[u][r]) : sv[u][r], cap, inv_cap);
           }
-          else if (kMimic && D >= 128) {
+          else if (kMimic && D >= RPA_ROUND_MIN_D) {
             // the reference's logits are bf16 (_xla_impl_fwd.py:119-124): round them, two per conversion (head_dim 64
-            // keeps fp32 logits: its tiles are bound by vector instructions and the rounding costs them 16 %)
+            // keeps fp32 logits: its tiles are bound by vector instructions and the rounding costs them a fifth)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
