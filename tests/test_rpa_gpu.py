@@ -336,9 +336,8 @@ def test_bf16_random_batches(seed):
     """Seeded random shapes on the MFMA path and on the scalar path: the parity bound against the op-by-op restatement
     on every row where that is finite (rows it turns NaN -- its first-KV-block defect under a window -- are left to
     the second check), and a bound of 4e-2 / 2e-3 against the float64 evaluation on every row (bf16 logits alone put
-    up to 2.5e-2 between the restatement and float64 here).  An element further from the restatement than the bound
-    is accepted only where the device value is the one next to the float64 value (seeds 1039 and 1118 hold one such
-    element each on the prefill tiles: restatement 0.018-0.021 from float64, device 0.003-0.005)."""
+    up to 2.5e-2 between the restatement and float64 here).  Every path is held to the bound as it stands, the plain
+    and the pipelined prefill tiles included; no element is excused by its distance from float64."""
     b, what = random_rpa_batch(seed, DEV)
     rows = b.total_valid_tokens
     strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
