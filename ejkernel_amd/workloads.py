@@ -336,6 +336,8 @@ WORKLOADS = {
     "prefill_long": "2 prompts x 8192 tokens from scratch, 32q/8kv heads, D=128, page 32",
     # head_dim 64 with many query heads per kv head (the attention shape of gpt-oss), chunked prefill
     "prefill_head_dim_64": "32 chunks x 512 tokens after 2048, 64q/8kv heads, D=64, page 32",
+    # the decode batch of decode_llama3_8b with half the head_dim: K / V rows of 128 bytes
+    "decode_head_dim_64": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=64, page 16",
 }
 
 
@@ -390,6 +392,11 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         return make_batch(np.full(S, chunk), np.full(S, prior + chunk), num_q_heads=64, num_kv_heads=8, head_dim=64,
                           page_size=32, pages_per_seq=pages(prior + chunk, 32), seed=seed, device=device, dtype=dtype,
                           name=name)
+    if name == "decode_head_dim_64":
+        S = n(256)
+        kv = rng.integers(n(512), n(8192) + 1, size=S)
+        return make_batch(np.ones(S, int), kv, num_q_heads=32, num_kv_heads=8, head_dim=64, page_size=16,
+                          pages_per_seq=pages(n(8192), 16), seed=seed, device=device, dtype=dtype, name=name)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)

@@ -101,7 +101,8 @@ def test_bf16_decode_small_full_size(flags):
 
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("name,scale", [("decode_llama3_8b", 0.06), ("mixed_prefill_decode", 0.08),
-                                        ("decode_long_context", 0.04), ("prefill_long", 0.08), ("prefill_head_dim_64", 0.12)])
+                                        ("decode_long_context", 0.04), ("prefill_long", 0.08), ("prefill_head_dim_64", 0.12),
+                                        ("decode_head_dim_64", 0.06)])
 def test_bf16_scaled_workloads(flags, name, scale):
     b = make_workload(name, device=DEV, scale=scale)
     out = to_np(run_hip(b, flags))
