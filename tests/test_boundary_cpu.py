@@ -261,3 +261,38 @@ def test_bench_power_sensor_and_gpu_count_guard():
     root = Path(__file__).resolve().parents[1]
     r = subprocess.run([sys.executable, str(root / "bench.py"), "--gpus", "2"], capture_output=True, text=True, cwd=str(root))
     assert r.returncode == 2 and "one GPU" in r.stderr
+
+
+def test_ffi_attributes_named_alike_in_python_and_in_the_handlers():
+    """jax.ffi passes attributes by name: every keyword a wrapper in jax_ffi.py hands to its ffi_call must be an
+    Attr of the handler registered under that target, with nothing missing on either side, and the operand counts
+    must agree (optional trailing operands arrive through RemainingArgs).  Checked on the source text; neither file
+    can run here."""
+    import ast
+
+    root = Path(__file__).resolve().parents[1]
+    cc = (root / "ejkernel_amd" / "csrc" / "rpa_xla_ffi.cc").read_text()
+    py_src = (root / "ejkernel_amd" / "jax_ffi.py").read_text()
+    handlers = {}
+    for m in re.finditer(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((\w+),\s*\w+,(.*?)\);\n", cc, flags=re.S):
+        body = m.group(2)
+        handlers[m.group(1)] = (re.findall(r'\.Attr<\w+>\("(\w+)"\)', body), len(re.findall(r"\.Arg<", body)),
+                                ".RemainingArgs()" in body, len(re.findall(r"\.Ret<", body)))
+    targets = dict(re.findall(r'"(mi355x_\w+)":\s*"(Rpa\w+)"', py_src))
+    targets["mi355x_rpa_fwd" if "mi355x_rpa_fwd" in py_src else "_TARGET"] = "RpaFwd"
+    tree = ast.parse(py_src)
+    wrappers = {"ragged_page_attention": "RpaFwd", "ragged_page_attention_v3": "RpaV3", "page_attention": "RpaPageAttn",
+                "ragged_decode_attention": "RpaRaggedDecode"}
+    assert set(wrappers.values()) == set(handlers) and set(targets.values()) >= set(handlers)
+    for fn in [n for n in tree.body if isinstance(n, ast.FunctionDef) and n.name in wrappers]:
+        attrs, n_args, has_rest, n_rets = handlers[wrappers[fn.name]]
+        # the call whose callee is the `call` object made by jax.ffi.ffi_call: its keywords are the attributes
+        calls = [c for c in ast.walk(fn) if isinstance(c, ast.Call) and isinstance(c.func, ast.Name) and c.func.id == "call"]
+        assert len(calls) == 1, fn.name
+        kw = [k.arg for k in calls[0].keywords]
+        assert sorted(kw) == sorted(attrs), (fn.name, kw, attrs)
+        positional = calls[0].args
+        if any(isinstance(a, ast.Starred) for a in positional):
+            assert has_rest, fn.name          # a variable operand list needs RemainingArgs in the binding
+        else:
+            assert len(positional) == n_args and not has_rest, (fn.name, len(positional), n_args)
