@@ -97,7 +97,7 @@ void rpa_tile_kernel(TileArgs a) {
   // (more than kWaveItemMaxRowTiles row tiles), or wave-level items (everything else).
   auto classify = [&](const SeqInfo& si, int& tiles, int& items, int& wg_items) {
     tiles = items = wg_items = 0;
-    if (si.eligible) tiles = item_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT);
+    if (si.eligible) tiles = item_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT + a.item_pad_tiles);
     else if (!kWaveOnly && si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
     else items = item_heads * si.n_rt;
   };
@@ -397,10 +397,19 @@ void rpa_tile_kernel(TileArgs a) {
           int s_base;
           const int s = find(tile_start, 1, x, s_base);
           const SeqInfo si = seq_info<C::TT>(a, s, G);
+          // A (sequence, kv head) occupies its tiles plus item_pad_tiles empty positions in the stream: what a part
+          // costs beyond its tiles (its query rows, the first tile's latency, the hand-off of a partial result) is
+          // about that many iterations, and without them a wavefront whose share holds many short (sequence, kv
+          // head)s finishes tens of microseconds after the others.
           const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
+          const int per_item = per_head + a.item_pad_tiles;
           const int local = x - s_base;
-          const int j = local / per_head, t0 = local - j * per_head;
-          const int t1 = min(per_head, t0 + (x_end - x));
+          const int j = local / per_item, t0 = local - j * per_item;
+          const int t1 = min(per_item, t0 + (x_end - x));
+          if (t0 >= per_head) {  // only the padding of this (sequence, kv head) is left in the share
+            x += t1 - t0;
+            continue;
+          }
           Part part;
           part.stream_a = x - t0;
           part.sh = sh;
@@ -408,7 +417,7 @@ void rpa_tile_kernel(TileArgs a) {
           part.last_w = sh.owner(part.stream_a + per_head - 1);
           part.partial = part.first_w != part.last_w;
           part.slot = part_slot(worker, part.stream_a, sh);
-          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + t1 * C::TT), part);
+          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + min(t1, per_head) * C::TT), part);
           x += t1 - t0;
         }
       }
@@ -424,6 +433,7 @@ struct Tune {
   int wgs_per_cu;          // RPA_TUNE_WGS_PER_CU: workgroups of the persistent grid per compute unit (1..kTiledMaxWgsPerCu)
   int decode_wgs_per_cu;   // RPA_TUNE_DECODE_WGS_PER_CU: of these, how many stream a batch without prefill tiles (0 = rule)
   int min_share_tiles;     // RPA_TUNE_MIN_SHARE_TILES
+  int item_pad_tiles;      // RPA_TUNE_ITEM_PAD_TILES: empty stream positions per (sequence, kv head)
   int phase_mode;          // RPA_TUNE_PHASE_MODE
   int even_xcd_permille;   // RPA_TUNE_EVEN_XCD_PERMILLE
   int no_mimic;            // RPA_TUNE_NO_MIMIC
@@ -444,6 +454,7 @@ static const Tune& tune() {
     x.wgs_per_cu = min(kTiledMaxWgsPerCu, max(1, env_int("RPA_TUNE_WGS_PER_CU", 2)));
     x.decode_wgs_per_cu = max(0, env_int("RPA_TUNE_DECODE_WGS_PER_CU", 0));
     x.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
+    x.item_pad_tiles = min(64, env_int("RPA_TUNE_ITEM_PAD_TILES", -1));  // negative: 128 keys' worth of tiles
     x.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
     x.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
     x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
@@ -519,6 +530,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.stats = stats;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.min_share_tiles = tune().min_share_tiles;
+  // a part costs about as much as streaming 128 keys: 4 tiles of 32 keys, 8 of 16 (head_dim 256)
+  a.item_pad_tiles = tune().item_pad_tiles >= 0 ? tune().item_pad_tiles : (p.head_dim > 128 ? 8 : 4);
   a.page_shift = __builtin_ctz(p.page_size);
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = tune().phase_mode;

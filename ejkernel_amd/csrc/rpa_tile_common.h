@@ -26,6 +26,7 @@ struct TileArgs {
   int stream_grid;    // workgroups that take part when the batch has no prefill tiles
   int sched_shift;    // the schedule arrays hold every (1 << sched_shift)-th sequence's start (0: every sequence)
   int min_share_tiles; // small batches: tiles per streaming wavefront before more wavefronts are used
+  int item_pad_tiles;  // empty positions every (sequence, kv head) adds to the decode stream (the cost of a part in tiles)
   int even_xcd_permille;  // share of the decode stream given to the workgroups on even XCDs, in 1/1000
   int phase_mode;     // mixed batches: 4 = upper half of the grid streams, prefill tiles from queues; 0..3 = static
                       // split, streaming first on no / upper-half / odd / odd-octet workgroups
