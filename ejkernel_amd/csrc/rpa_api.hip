@@ -23,6 +23,15 @@ int fail(int code, const char* fmt, ...) {
   return code;
 }
 
+// The kernels fetch rows in 16-byte pieces wherever a row is a multiple of 16 bytes (every shape the MFMA path takes);
+// rows that are not go through the scalar kernel, element by element.
+static uint32_t data_alignment(const RpaParams& p) {
+  const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
+  return (static_cast<uint64_t>(p.head_dim) * esize) % 16 == 0 ? 16u : esize;
+}
+static bool aligned_to(const void* ptr, uint32_t bytes) { return (reinterpret_cast<uintptr_t>(ptr) & (bytes - 1)) == 0; }
+static bool data_aligned(const RpaParams& p, const void* ptr) { return aligned_to(ptr, data_alignment(p)); }
+
 static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_seq = false, bool contiguous = false) {
   if (p.total_tokens < 0 || p.num_q_heads <= 0 || p.num_kv_heads <= 0 || p.head_dim <= 0 || p.page_size <= 0 ||
       p.num_pages <= 0 || p.max_num_seqs <= 0 || p.pages_per_seq <= 0 || p.num_sinks < 0)
@@ -43,6 +52,11 @@ static int validate(const RpaParams& p, bool need_pointers, bool one_token_per_s
         (!one_token_per_seq && (!p.query_start_loc || !p.num_seqs)))
       return fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaParams");
     if (p.num_sinks > 0 && !p.sinks) return fail(RPA_ERR_INVALID_ARGUMENT, "num_sinks=%d but sinks is null", p.num_sinks);
+    if (!data_aligned(p, p.queries) || !data_aligned(p, p.kv_pages) || !data_aligned(p, p.out))
+      return fail(RPA_ERR_INVALID_ARGUMENT, "queries, the cache and out must be aligned to %u bytes", data_alignment(p));
+    if (!aligned_to(p.context_lens, 4) || !aligned_to(p.block_tables, 4) || !aligned_to(p.query_start_loc, 4) ||
+        !aligned_to(p.num_seqs, 4) || !aligned_to(p.sinks, 4))
+      return fail(RPA_ERR_INVALID_ARGUMENT, "int32 / fp32 arrays must be aligned to 4 bytes");
   }
   return RPA_OK;
 }
@@ -213,6 +227,7 @@ int rpa_page_attention_launch(const RpaPageAttnParams* params, void* hip_stream)
   int rc = rpa::validate(p, true, true);
   if (rc != RPA_OK) return rc;
   if (!params->value_cache) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaPageAttnParams");
+  if (!rpa::data_aligned(p, params->value_cache)) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "value_cache is not aligned like key_cache must be");
   const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
   rpa::KvLayout kv;
   kv.k_base = static_cast<const char*>(params->key_cache);
@@ -289,6 +304,8 @@ int rpa_ragged_decode_launch(const RpaRaggedDecodeParams* params, void* hip_stre
   if (rc != RPA_OK) return rc;
   if (!params->value || !params->sequence_start)
     return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null device pointer in RpaRaggedDecodeParams");
+  if (!rpa::data_aligned(p, params->value) || !rpa::aligned_to(params->sequence_start, 4) || !rpa::aligned_to(params->softmax_aux, 4))
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "value is not aligned like key must be, or an int32 / fp32 array is not aligned to 4 bytes");
   const uint32_t esize = p.dtype == RPA_DTYPE_BF16 ? 2u : 4u;
   rpa::KvLayout kv;
   kv.k_base = static_cast<const char*>(params->key);
@@ -375,6 +392,8 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   int rc = rpa::validate(v.attn, true);
   if (rc != RPA_OK) return rc;
   if (!v.new_keys || !v.new_values) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "null new_keys / new_values");
+  if (!rpa::aligned_to(v.new_keys, 16) || !rpa::aligned_to(v.new_values, 16) || !rpa::aligned_to(v.attn.kv_pages, 16))
+    return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "new_keys, new_values and the cache must be aligned to 16 bytes");
   if (v.attn.num_sinks != 0) return rpa::fail(RPA_ERR_INVALID_ARGUMENT, "ragged_page_attention_v3 has no sinks");
   const bool fp8 = v.cache_dtype == RPA_DTYPE_FP8_E4M3 || v.cache_dtype == RPA_DTYPE_FP8_E5M2;
   if (!fp8 && v.cache_dtype != v.attn.dtype)

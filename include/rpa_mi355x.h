@@ -59,7 +59,9 @@ extern "C" {
 #define RPA_FLAG_PLAIN_TILES 16u  /* never those: prefill tiles of 128 rows, two workgroups per compute unit          */
 
 typedef struct RpaParams {
-  /* ---- device buffers (argument names follow ragged_page_attention.py:540-547) ---- */
+  /* ---- device buffers (argument names follow ragged_page_attention.py:540-547).  queries, kv_pages and out are   */
+  /* aligned to 16 bytes (to the element where head_dim * sizeof(element) is not a multiple of 16), the int32 and   */
+  /* fp32 arrays to 4; a misaligned pointer is RPA_ERR_INVALID_ARGUMENT ---- */
   const void* queries;         /* [total_tokens, num_q_heads, head_dim]                      */
   const void* kv_pages;        /* [num_pages, page_size, 2*num_kv_heads, head_dim]; K of kv   */
                                /* head j at combined index 2j, V at 2j+1                      */

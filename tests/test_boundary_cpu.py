@@ -60,8 +60,8 @@ def test_ragged_decode_sink_arguments_are_checked_before_any_launch():
     p.num_sinks, p.aux_rows = 4, 1
     with_sinks = lib.rpa_ragged_decode_workspace_bytes(ctypes.byref(p))
     assert with_sinks >= plain + 4 * 8 * (128 + 2) * 4       # the sink keys' state per (sequence, query head)
-    buf = (ctypes.c_char * 64)()
-    addr = ctypes.addressof(buf)                              # never dereferenced: every call below fails first
+    buf = (ctypes.c_char * 192)()
+    addr = (ctypes.addressof(buf) + 63) & ~63                 # never dereferenced: every call below fails first
     for f in ("query", "key", "value", "sequence_start", "sequence_end", "out", "workspace"):
         setattr(p, f, addr)
     p.workspace_bytes = with_sinks
@@ -89,8 +89,8 @@ def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
     v.cache_dtype = _native.RPA_DTYPE_FP8_E4M3
     with_stats = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
     assert with_stats >= plain + 16 * 8 * 2 * 4              # row maximum and sum per (token, query head)
-    buf = (ctypes.c_char * 64)()
-    addr = ctypes.addressof(buf)                              # never dereferenced: every call below fails first
+    buf = (ctypes.c_char * 192)()
+    addr = (ctypes.addressof(buf) + 63) & ~63                 # never dereferenced: every call below fails first
     for f in ("queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs", "out", "workspace"):
         setattr(p, f, addr)
     v.new_keys = v.new_values = addr
@@ -116,6 +116,31 @@ def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
     assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_head_dim" in lib.rpa_last_error()
     v.cache_head_dim, v.cache_combined_heads = 128, 2         # fewer than 2 * num_kv_heads = 4
     assert lib.rpa_v3_launch(ctypes.byref(v), None) == -1 and b"cache_combined_heads" in lib.rpa_last_error()
+
+
+def test_misaligned_pointers_are_rejected_before_any_launch():
+    """Rows are fetched in 16-byte pieces wherever a row is a multiple of 16 bytes; rows that are not need the
+    element's own alignment (they run on the scalar kernel)."""
+    lib = _native.load()
+    p = _native.RpaParams()
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = 16, 8, 2, 128
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = 16, 64, 4, 16
+    p.softmax_scale = 0.1
+    p.dtype, p.compute = _native.RPA_DTYPE_BF16, _native.RPA_COMPUTE_BF16
+    buf = (ctypes.c_char * 192)()
+    addr = (ctypes.addressof(buf) + 63) & ~63                 # never dereferenced: every call below fails first
+    fields = ("queries", "kv_pages", "context_lens", "block_tables", "query_start_loc", "num_seqs", "out")
+    for bad, off, msg in (("queries", 8, b"16 bytes"), ("kv_pages", 2, b"16 bytes"), ("out", 4, b"16 bytes"),
+                          ("block_tables", 2, b"4 bytes"), ("context_lens", 1, b"4 bytes")):
+        for f in fields:
+            setattr(p, f, addr + (off if f == bad else 0))
+        assert lib.rpa_fwd_launch(ctypes.byref(p), None) == -1 and msg in lib.rpa_last_error(), bad
+    p.head_dim = 4                                            # rows of 8 bytes: the scalar kernel, element alignment
+    for f in fields:
+        setattr(p, f, addr)
+    p.queries = addr + 8
+    p.out = addr + 1
+    assert lib.rpa_fwd_launch(ctypes.byref(p), None) == -1 and b"2 bytes" in lib.rpa_last_error()
 
 
 def test_workspace_bytes_and_errors_without_gpu():
