@@ -18,6 +18,7 @@ grad, the same way the reference's native custom call refuses differentiation
 from __future__ import annotations
 
 import ctypes
+import threading
 from typing import Any, Literal
 
 import torch
@@ -29,6 +30,7 @@ __all__ = ["RaggedPageAttention", "ragged_page_attention"]
 
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
 _MAX_WORKSPACES = 16  # (device, stream) pairs kept; the least recently used one goes first (about 35 MB each)
+_workspaces_lock = threading.Lock()  # host threads launch on streams of their own at the same time
 
 
 def _compute_mode(compute_dtype: Any) -> int:
@@ -130,18 +132,19 @@ def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tens
     gets its own.
     """
     key = (device.index if device.index is not None else torch.cuda.current_device(), int(stream_ptr))
-    ws = _workspaces.pop(key, None)  # re-inserted below: the dict keeps its keys in order of last use
-    if ws is None or ws.numel() < nbytes:
-        # A stream that no longer exists leaves its workspace behind (torch has no hook for a stream's end), so the cache
-        # is bounded.  The evicted tensor's memory goes back to torch's caching allocator, which keeps it away from
-        # other streams until the work queued on this one has finished.
-        while len(_workspaces) >= _MAX_WORKSPACES:
-            _workspaces.pop(next(iter(_workspaces)))
-        ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
-        rc = _native.load().rpa_workspace_init(ctypes.c_void_p(ws.data_ptr()), ws.numel(), ctypes.c_void_p(stream_ptr))
-        if rc != 0:
-            raise RuntimeError(f"rpa_workspace_init failed ({rc}): {_native.last_error()}")
-    _workspaces[key] = ws
+    with _workspaces_lock:
+        ws = _workspaces.pop(key, None)  # re-inserted below: the dict keeps its keys in order of last use
+        if ws is None or ws.numel() < nbytes:
+            # A stream that no longer exists leaves its workspace behind (torch has no hook for a stream's end), so the
+            # cache is bounded.  The evicted tensor's memory goes back to torch's caching allocator, which keeps it away
+            # from other streams until the work queued on this one has finished.
+            while len(_workspaces) >= _MAX_WORKSPACES:
+                _workspaces.pop(next(iter(_workspaces)))
+            ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
+            rc = _native.load().rpa_workspace_init(ctypes.c_void_p(ws.data_ptr()), ws.numel(), ctypes.c_void_p(stream_ptr))
+            if rc != 0:
+                raise RuntimeError(f"rpa_workspace_init failed ({rc}): {_native.last_error()}")
+        _workspaces[key] = ws
     return ws
 
 

@@ -499,6 +499,49 @@ def test_concurrent_streams_do_not_share_a_workspace():
             assert torch.equal(o, alone[k])
 
 
+def test_host_threads_launch_at_the_same_time_on_streams_of_their_own():
+    """The C entry points are re-entrant (error text per thread, tuning knobs and kernel attributes set once under a
+    guard) and ctypes drops the interpreter lock around them, so two host threads really launch at once; every result
+    equals the one computed alone, bit for bit, and an error raised in one thread names that thread's mistake."""
+    import threading
+
+    batches = [make_workload("decode_long_context", device=DEV, scale=0.05), make_workload("mixed_prefill_decode", device=DEV, scale=0.1)]
+    alone = [run_hip(b) for b in batches]
+    torch.cuda.synchronize()
+    failures = []
+
+    def work(k):
+        try:
+            torch.cuda.set_device(0)
+            st = torch.cuda.Stream()
+            with torch.cuda.stream(st):
+                for rep in range(12):
+                    out = ragged_page_attention(*batches[k].args(), **batches[k].kwargs())
+                    if rep % 4 == 3:
+                        st.synchronize()
+                        if not torch.equal(out, alone[k]):
+                            failures.append((k, rep, "result differs"))
+                bad = batches[k]
+                try:  # a rejected call in this thread: the message is this thread's
+                    ragged_page_attention(bad.queries, bad.kv_pages, bad.context_lens, bad.block_tables, bad.query_start_loc,
+                                          bad.num_seqs, softmax_scale=float("nan") if k == 0 else 1.0,
+                                          logits_soft_cap=None if k == 0 else float("nan"))
+                    failures.append((k, "no error"))
+                except (ValueError, RuntimeError) as e:
+                    if ("softmax_scale is NaN" if k == 0 else "logits_soft_cap is NaN") not in str(e):
+                        failures.append((k, str(e)))
+            st.synchronize()
+        except Exception as e:  # noqa: BLE001
+            failures.append((k, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not failures, failures
+
+
 def test_workspace_cache_is_bounded_over_many_streams():
     """Every (device, stream) gets its own workspace; past the bound the least recently used one is dropped, and a call on
     a stream whose workspace was dropped allocates (and clears) a new one."""
