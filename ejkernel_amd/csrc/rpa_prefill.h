@@ -78,7 +78,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   const int W = p.sliding_window;
   const bf16_t* __restrict__ q = static_cast<const bf16_t*>(p.queries);
   bf16_t* __restrict__ out = static_cast<bf16_t*>(p.out);
-  const char* kvb = static_cast<const char*>(p.kv_pages);
+  const char* kvb = a.kv.k_base;
   // the reference's cap is a weakly typed scalar: it takes the logits' dtype (bf16) before it divides and multiplies
   const float cap = kMimic ? rbf(p.logits_soft_cap) : p.logits_soft_cap;
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
@@ -186,8 +186,12 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // lane order, so lane l fills piece slot l % PR of row l / PR and fetches the piece that the swizzle assigns
   // to that slot.  Block-table entries are scalar loads (the rows of a block share a page, except with pages
   // shorter than a block).
-  const uint32_t stride_b = static_cast<uint32_t>(2 * p.num_kv_heads * hd) * 2u;
-  const uint64_t page_b = static_cast<uint64_t>(p.page_size) * stride_b;
+  // The cache is [page][slot][combined head][row]: K of kv head j, then its V row, a.kv.head_b bytes per pair; rows
+  // may be longer than head_dim and a token may hold more rows than 2 * num_kv_heads (both padded by the caller).
+  const uint32_t stride_b = a.kv.stride_b;
+  const uint64_t page_b = a.kv.page_b;
+  const uint32_t head_off = static_cast<uint32_t>(j) * a.kv.head_b;                   // K row of this kv head inside a token
+  const uint32_t v_delta = static_cast<uint32_t>(a.kv.v_base - a.kv.k_base);          // its V row, from the K row
   const const_i32_ptr bt_c = reinterpret_cast<const_i32_ptr>(
       reinterpret_cast<uintptr_t>(p.block_tables + static_cast<size_t>(s) * p.pages_per_seq));
   const int l_row = lane / C::PR, l_slot = lane % C::PR;
@@ -204,9 +208,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     const int t_local = GROUP * wave + C::RB * n + l_row;
     pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
   }
-  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + hd * 2;  // V block 0; block n adds RB rows
+  const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + v_delta;  // V block 0; block n adds RB rows
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
-    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + hd * 2;
+    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + v_delta;
   };
   const bool group_in_page = p.page_size >= GROUP;
   auto fetch_tile = [&](int tile, int buf) {
@@ -216,7 +220,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       // the whole group lies in one page and inside the range: one block-table entry, one base address
       const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+                          static_cast<uint64_t>(t_first & (p.page_size - 1)) * stride_b + head_off;
       // Buffer addressing (scalar base in a resource descriptor, 32-bit per-lane offset): a wavefront is held for
       // about 50 cycles per direct-to-LDS load it issues this way, against about 100 with 64-bit per-lane addresses.
       const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(sbase), 0, 0x7fffffff, 0x00020000);
@@ -238,19 +242,19 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         const int t_local = GROUP * wave + C::RB * n + l_row;
         auto row_base = [&](int tok) {
           const int pg = min(max(p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + (tok >> a.page_shift)], 0), p.num_pages - 1);
-          return kvb + static_cast<uint64_t>(pg) * page_b + static_cast<uint64_t>(tok & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+          return kvb + static_cast<uint64_t>(pg) * page_b + static_cast<uint64_t>(tok & (p.page_size - 1)) * stride_b + head_off;
         };
         __builtin_amdgcn_global_load_lds(
             reinterpret_cast<const u32x4_t*>(row_base(min(t_c + l_row, t_last)) + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask)),
             (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
         const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(row_base(min(t_c + v_row, t_last)) + v_piece + hd * 2),
+        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(row_base(min(t_c + v_row, t_last)) + v_piece + v_delta),
                                          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
         continue;
       }
       const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
-                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + 2 * j * hd * 2;
+                          static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + head_off;
       const int tok = min(t_c + l_row, t_last);
       const int t_local = GROUP * wave + C::RB * n + l_row;
       const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
@@ -259,7 +263,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const int v_tok = min(t_c + v_row, t_last);
       const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
       __builtin_amdgcn_global_load_lds(
-          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + hd * 2),
+          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + v_delta),
           (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
     }
   };

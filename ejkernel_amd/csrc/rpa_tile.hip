@@ -574,12 +574,18 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
   const bool small_batch = p.query_start_loc == nullptr || ((p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) == 0 &&
                                                             rows <= tune().wave_only_rows);
-  // Prefill tiles address the cache as [page][slot][2 * kv heads][head_dim]; any other layout (two caches, one
-  // contiguous cache per sequence, rows padded beyond head_dim) runs through the wave-level loop alone.
+  // Prefill tiles address one paged cache with a token's K and V rows side by side, [page][slot][combined head][row]
+  // (rows may be padded beyond head_dim and tokens beyond 2 * kv heads: the plain tile takes the pitches from the
+  // layout; the pipelined tile's instruction stream has the unpadded ones built in); any other layout (two caches, one
+  // contiguous cache per sequence) runs through the wave-level loop alone.
   const KvLayout canon = interleaved_layout(p);
   const bool canonical = kv.k_base == canon.k_base && kv.v_base == canon.v_base && kv.stride_b == canon.stride_b &&
                          kv.head_b == canon.head_b && kv.page_b == canon.page_b && kv.contiguous == 0;
-  const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !canonical || (small_batch && tune().no_wave_only == 0);
+  const bool side_by_side = kv.contiguous == 0 && kv.k_base == canon.k_base && kv.v_base > kv.k_base &&
+                            static_cast<uint64_t>(kv.v_base - kv.k_base) * 2 == kv.head_b && kv.head_b % 32 == 0 &&
+                            kv.stride_b % 16 == 0 && kv.stride_b >= static_cast<uint64_t>(p.num_kv_heads) * kv.head_b &&
+                            kv.page_b == static_cast<uint64_t>(p.page_size) * kv.stride_b;
+  const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
     // head_dim 64: two kv heads per item where that keeps a decode token's rows in one 16-row tile
     a.pair = p.head_dim == 64 && p.num_kv_heads % 2 == 0 && 2 * (p.num_q_heads / p.num_kv_heads) <= 16 && pre.ml == nullptr &&
@@ -602,7 +608,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     const bool pipe_wanted = (p.flags & RPA_FLAG_PLAIN_TILES) == 0 &&
                              ((p.flags & RPA_FLAG_PIPE_TILES) != 0 ||
                               (tune().pipe != 0 && static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs));
-    if (pipe_wanted && pipe_ok) {
+    if (pipe_wanted && pipe_ok && canonical) {
       // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
       // number on every XCD) take the decode stream first and join the prefill queues when it is done
       const int g1 = device_cu_count();

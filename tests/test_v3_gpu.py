@@ -143,9 +143,10 @@ def test_validation_errors_follow_the_reference():
         ragged_page_attention_v3(*a, mesh=object())
 
 
-@pytest.mark.parametrize("name,n_sample", [("decode_llama3_8b", 10), ("mixed_prefill_decode", 12)])
+@pytest.mark.parametrize("name,n_sample", [("decode_llama3_8b", 10), ("mixed_prefill_decode", 12), ("prefill_head_dim_64", 3)])
 def test_full_size_workload(name, n_sample):
-    """Sampled parity against the oracle plus size-independent properties of the cache update."""
+    """Sampled parity against the oracle plus size-independent properties of the cache update (head_dim 64: cache rows
+    padded to 128 elements, the chunks on the prefill tiles)."""
     b = make_workload(name, device=DEV)
     v = to_v3(b, seed=5)
     rng = np.random.default_rng(1)
@@ -172,8 +173,9 @@ def test_full_size_workload(name, n_sample):
     t = torch.arange(total, device=DEV)
     pos = b.context_lens.long()[seq_of_tok] - torch.as_tensor(b.q_lens, device=DEV)[seq_of_tok] + (t - qsl[seq_of_tok])
     pg = b.block_tables.long()[seq_of_tok, pos // page]
-    assert torch.equal(rows_after[pg, pos % page, 0::2], v.keys[:total])
-    assert torch.equal(rows_after[pg, pos % page, 1::2], v.values[:total])
+    hx2, Dk = 2 * v.keys.shape[1], v.keys.shape[2]
+    assert torch.equal(rows_after[pg, pos % page, 0:hx2:2, :Dk], v.keys[:total])
+    assert torch.equal(rows_after[pg, pos % page, 1:hx2:2, :Dk], v.values[:total])
     checksum_after = cache.view(torch.int16).sum(dtype=torch.int64).item()
     assert checksum_after != checksum_before
 
@@ -194,14 +196,15 @@ def test_bf16_random_batches(seed):
             assert_bf16_parity_stepwise(to_np(out)[:rows], ref_out[:rows], f"{what} flags={flags}")
 
 
-@pytest.mark.parametrize("flags", [0, _native.RPA_FLAG_FORCE_GENERIC])
+@pytest.mark.parametrize("flags", [0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_FORCE_GENERIC])
 @pytest.mark.parametrize("D", [64, 192])
 @pytest.mark.parametrize("window", [None, 48])
 def test_cache_rows_padded_to_a_multiple_of_128(D, flags, window):
     """head_dim 64 lives in cache rows of 128 elements, 192 in rows of 256 (merge_kv pads them with zeros): the update
     writes whole token records, padding zeroed as the reference's scatter does (_kernel.py:44-57, :207-218), and leaves
     other tokens' padding alone; the attention never reads it (it holds random data).
-    head_dim 64 runs on the MFMA kernel's wave-level loop, 192 on the scalar kernel."""
+    head_dim 64 runs on the MFMA kernel -- its wave-level loop and, for longer chunks or on request, its prefill tiles,
+    which take the row and token pitches from the cache's layout -- and 192 on the scalar kernel."""
     v = small([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], head_dim=D, pages_per_seq=32, sliding_window=window)
     dalign = -(-D // 128) * 128
     assert v.kv_cache.shape[-1] == dalign and v.keys.shape[-1] == D
@@ -238,7 +241,7 @@ def test_bf16_random_batches_head_dim_64(seed):
     """Seeded random shapes at head_dim 64 (cache rows padded to 128): the cache bit for bit, outputs within the bound."""
     b, what = random_rpa_batch(seed, DEV, head_dims=(64,))
     rows = b.total_valid_tokens
-    for flags in (0, _native.RPA_FLAG_FORCE_GENERIC):
+    for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_FORCE_GENERIC):
         v = to_v3(random_rpa_batch(seed, DEV, head_dims=(64,))[0], seed=seed)
         ref_out, ref_cache = oracle(v)
         out, cache = run_hip(v, flags)
