@@ -66,10 +66,19 @@ struct PCfg {
 
 constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point by this much before O is rescaled
 
-template <int D, int MRT, bool kMimic>
+// kKv / kPass as in the wave-level loop (rpa_decode.h): with an 8-bit cache (kKv 1 = e4m3, 2 = e5m2) the K / V pieces
+// of a tile go through registers -- 8 bytes per lane and block, fetched one step ahead like the direct-to-LDS loads of
+// the 16-bit cache -- and are widened to bf16 (exactly) on their way into the same LDS layout, so everything after the
+// fetch is the 16-bit tile; kPass 1 walks K alone and leaves each row's softmax reference point and its sum of
+// exp(logit - point) in TileArgs::stats, kPass 2 forms P = round(exp(logit - point) / sum) in the cache dtype from
+// them and accumulates P V with no rescaling.
+template <int D, int MRT, bool kMimic, int kKv = 0, int kPass = 0>
 __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
                                              int qt) {
   using C = PCfg<D, MRT>;
+  static_assert(kKv == 0 || C::NSTG == 2, "the register stage of an 8-bit cache stands in for one LDS stage ahead");
+  static_assert((kKv == 0) == (kPass == 0), "an 8-bit cache runs as two passes, a 16-bit cache as one");
+  constexpr uint32_t PB = kKv != 0 ? 8u : 16u;  // bytes of a row piece (eight elements) in the cache
   const RpaParams& p = a.p;
   const int tid = threadIdx.x;
   const int lane = tid & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(tid / kWave);
@@ -134,9 +143,19 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       if (valid && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
       u32x4_t sc;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        sc[e] = pack_bf16x2(q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale),
-                            q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale));
+      for (int e = 0; e < 4; ++e) {
+        float q0 = q_operand<kMimic>(__uint_as_float(raw[e] << 16), p, scale);
+        float q1 = q_operand<kMimic>(__uint_as_float(raw[e] & 0xffff0000u), p, scale);
+        if constexpr (kKv != 0) {
+          if (p.q_scale > 0.f) {
+            // q / q_scale in the query dtype, clipped to the cache dtype's range and cast to it (_kernel.py:249-254)
+            q0 = fminf(fmaxf(rbf(q0), -fp8_max<kKv>()), fp8_max<kKv>());
+            q1 = fminf(fmaxf(rbf(q1), -fp8_max<kKv>()), fp8_max<kKv>());
+            round_fp8x2<kKv>(q0, q1);
+          }
+        }
+        sc[e] = pack_bf16x2(q0, q1);
+      }
       qreg[m][ks] = __builtin_bit_cast(bf16x8_t, sc);
     }
   }
@@ -171,10 +190,26 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // Softmax reference point m per row, kept as the exp2 offset -m log2(e) (0 while the row has seen no key) and
   // as the vote threshold for exp2 arguments: kLazy log2(e) once there is a reference point, -inf before.
   float m_thr[MRT], m_neg[MRT];
+  float l32[MRT];    // kPass 1: this lane's part of the row sum, in fp32
+  float inv_l[MRT];  // kPass 2: 1 / row sum from the statistics launch
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
     m_thr[m] = -INFINITY;
     m_neg[m] = 0.f;
+    l32[m] = 0.f;
+    inv_l[m] = 0.f;
+    if constexpr (kPass == 2) {
+      bool valid;
+      int head;
+      size_t q_off;
+      const int qi = row_of(m, 0, valid, head, q_off);
+      if (valid) {
+        const size_t idx = static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head;
+        const float ms = a.stats[2 * idx], ls = a.stats[2 * idx + 1];
+        m_neg[m] = ms == -INFINITY ? 0.f : -ms * kLog2e;
+        inv_l[m] = ls > 0.f ? 1.f / ls : 0.f;
+      }
+    }
     l_acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int sN = 0; sN < C::NS; ++sN)
@@ -199,23 +234,39 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
   // (Without the transposing read the V tile is laid out like the K tile.)
   const int v_row = C::TRV ? (lane >> 1) % C::RB : l_row;
-  const uint32_t v_src = 16u * (static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)) & pmask);  // byte offset in the row
+  const uint32_t v_src = PB * (static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)) & pmask);  // byte offset in the row
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
   uint32_t pre_off[HB];  // per-lane byte offset of K block n inside the group: row part + swizzled piece
 #pragma unroll
   for (int n = 0; n < HB; ++n) {
     const int t_local = GROUP * wave + C::RB * n + l_row;
-    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + PB * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
   }
   const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + v_delta;  // V block 0; block n adds RB rows
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
     return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + v_delta;
   };
   const bool group_in_page = p.page_size >= GROUP;
+  // 8-bit cache: this lane's K and V pieces of the tile being fetched, and where they go once widened
+  u32x2_t st_k[HB], st_v[HB];
+  char* st_dst = lds;
+  // One block of a tile: the lane's K piece and V piece, by address or by resource and offset.  16-bit cache: straight
+  // into LDS; 8-bit cache: into the register stage.
+  auto take = [&](int n, char* dst, const char* k_addr, const char* v_addr) {
+    if constexpr (kKv == 0) {
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(k_addr), (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
+      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(v_addr),
+                                       (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+    } else {
+      st_k[n] = *reinterpret_cast<const u32x2_t*>(k_addr);
+      if constexpr (kPass != 1) st_v[n] = *reinterpret_cast<const u32x2_t*>(v_addr);
+    }
+  };
   auto fetch_tile = [&](int tile, int buf) {
     const int t_first = tile + GROUP * wave;
     char* dst = lds + 2 * buf * C::TILE_B + HB * wave * 1024;
+    if constexpr (kKv != 0) st_dst = dst;
     if (group_in_page && t_first + GROUP - 1 <= t_last) {
       // the whole group lies in one page and inside the range: one block-table entry, one base address
       const int page = min(max(bt_c[t_first >> a.page_shift], 0), p.num_pages - 1);
@@ -226,10 +277,15 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(sbase), 0, 0x7fffffff, 0x00020000);
 #pragma unroll
       for (int n = 0; n < HB; ++n) {
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + n * 1024), 16,
-                                                 pre_off[n], 0, 0, 0);
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024),
-                                                 16, v_src_off(n), 0, 0, 0);
+        if constexpr (kKv == 0) {
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + n * 1024), 16,
+                                                   pre_off[n], 0, 0, 0);
+          __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024),
+                                                   16, v_src_off(n), 0, 0, 0);
+        } else {
+          st_k[n] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, pre_off[n], 0, 0);
+          if constexpr (kPass != 1) st_v[n] = __builtin_amdgcn_raw_buffer_load_b64(rsrc, v_src_off(n), 0, 0);
+        }
       }
       return;
     }
@@ -237,40 +293,43 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int n = 0; n < HB; ++n) {
       const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
+      const int t_local = GROUP * wave + C::RB * n + l_row;
+      const uint32_t k_piece = PB * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
+      const uint32_t v_piece = C::TRV ? v_src : k_piece;
       if (C::RB > 4 && p.page_size < C::RB) {
         // pages shorter than a block (pages of 4 tokens under 128-byte rows): every lane looks its own row's page up
-        const int t_local = GROUP * wave + C::RB * n + l_row;
         auto row_base = [&](int tok) {
           const int pg = min(max(p.block_tables[static_cast<size_t>(s) * p.pages_per_seq + (tok >> a.page_shift)], 0), p.num_pages - 1);
           return kvb + static_cast<uint64_t>(pg) * page_b + static_cast<uint64_t>(tok & (p.page_size - 1)) * stride_b + head_off;
         };
-        __builtin_amdgcn_global_load_lds(
-            reinterpret_cast<const u32x4_t*>(row_base(min(t_c + l_row, t_last)) + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask)),
-            (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
-        const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
-        __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(row_base(min(t_c + v_row, t_last)) + v_piece + v_delta),
-                                         (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+        take(n, dst, row_base(min(t_c + l_row, t_last)) + k_piece, row_base(min(t_c + v_row, t_last)) + v_piece + v_delta);
         continue;
       }
       const int page = min(max(bt_c[t_c >> a.page_shift], 0), p.num_pages - 1);
       const char* sbase = kvb + static_cast<uint64_t>(page) * page_b +
                           static_cast<uint64_t>(t_c & (p.page_size - 1)) * stride_b + head_off;
       const int tok = min(t_c + l_row, t_last);
-      const int t_local = GROUP * wave + C::RB * n + l_row;
-      const uint32_t off = static_cast<uint32_t>(tok - t_c) * stride_b + 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
-      __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(sbase + off),
-                                       (__attribute__((address_space(3))) void*)(dst + n * 1024), 16, 0, 0);
       const int v_tok = min(t_c + v_row, t_last);
-      const uint32_t v_piece = C::TRV ? v_src : 16u * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
-      __builtin_amdgcn_global_load_lds(
-          reinterpret_cast<const u32x4_t*>(sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + v_delta),
-          (__attribute__((address_space(3))) void*)(dst + C::TILE_B + n * 1024), 16, 0, 0);
+      take(n, dst, sbase + static_cast<uint32_t>(tok - t_c) * stride_b + k_piece,
+           sbase + static_cast<uint32_t>(v_tok - t_c) * stride_b + v_piece + v_delta);
     }
   };
   // Wait until at most `ahead` later tiles of this wave's direct-to-LDS loads are outstanding (they complete in
   // order); the barrier that follows publishes the oldest tile.  s_waitcnt takes an immediate: vmcnt is bits
   // [3:0] and [15:14]; 0x0F70 leaves the other counters unconstrained.
+  // 8-bit cache: the staged pieces (the compiler waits for them) are widened and written where the direct-to-LDS
+  // loads would have put them: bytes [16 lane, 16 lane + 16) of each 1 KiB block.  The stage they go to held the tile
+  // before the current one, which every wavefront left at the last barrier.
   auto wait_fetch = [&](int ahead) {
+    if constexpr (kKv != 0) {
+#pragma unroll
+      for (int n = 0; n < HB; ++n) {
+        *reinterpret_cast<u32x4_t*>(st_dst + n * 1024 + lane * 16) = fp8x8_to_bf16x8<kKv>(st_k[n]);
+        if constexpr (kPass != 1)
+          *reinterpret_cast<u32x4_t*>(st_dst + C::TILE_B + n * 1024 + lane * 16) = fp8x8_to_bf16x8<kKv>(st_v[n]);
+      }
+      return;
+    }
     static_assert(C::BPW * (C::NSTG - 2) <= 24, "extend the immediates below");
     switch (ahead * C::BPW) {
       case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
@@ -377,8 +436,8 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               s_acc[m][u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, kop[u][ks]), qreg[m][ks],
                                                                     s_acc[m][u], 0, 0, 0);
         }
-        load_v(0);
-        {
+        if constexpr (kPass != 1) {
+          load_v(0);
           // the V reads issue between the QK MFMAs, in the shadow of the matrix pipe, not after them
           constexpr int N_MFMA = 2 * C::NKS * MRT, PER_READ = N_MFMA / V_READS;
           static_assert(PER_READ >= 1 && PER_READ * V_READS == N_MFMA, "MFMAs per V read");
@@ -451,6 +510,20 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           // exceeds it by more than kLazy; probabilities then stay below e^kLazy, far inside bf16 / fp32 range.
           // The common case needs no cross-lane step at all: a wave-wide vote on the lane-local maxima, and the t
           // are the exp2 arguments as they stand.  When the point moves up by the row maximum, so do the t.
+          if constexpr (kPass == 2) {
+            // the reference point and the row sum are fixed: normalised probabilities, rounded to the cache dtype
+            // (exactly representable in bf16, which is how they enter P V)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+              float e0 = __builtin_amdgcn_exp2f(t[u][0]) * inv_l[m], e1 = __builtin_amdgcn_exp2f(t[u][1]) * inv_l[m];
+              float e2 = __builtin_amdgcn_exp2f(t[u][2]) * inv_l[m], e3 = __builtin_amdgcn_exp2f(t[u][3]) * inv_l[m];
+              round_fp8x2<kKv>(e0, e1);
+              round_fp8x2<kKv>(e2, e3);
+              pw[m][2 * u] = pack_bf16x2(e0, e1);
+              pw[m][2 * u + 1] = pack_bf16x2(e2, e3);
+            }
+            continue;
+          }
           if (__builtin_expect(__any(tmax > m_thr[m]), 0)) {
             tmax = row_groups_max(tmax);
             const bool bump = tmax > m_thr[m];  // then tmax is finite
@@ -462,11 +535,23 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               for (int r = 0; r < 4; ++r) t[u][r] -= shift;
             m_neg[m] -= shift;
             m_thr[m] = bump ? kLazy * kLog2e : m_thr[m];
-            l_acc[m] *= alpha;
+            if constexpr (kPass == 1) {
+              l32[m] *= alpha;
+            } else {
+              l_acc[m] *= alpha;
 #pragma unroll
-            for (int sN = 0; sN < C::NS; ++sN)
+              for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int c = 0; c < C::CB; ++c) o_acc[m][sN][c] *= alpha;
+                for (int c = 0; c < C::CB; ++c) o_acc[m][sN][c] *= alpha;
+            }
+          }
+          if constexpr (kPass == 1) {
+            // statistics only: the sum of the unrounded exponentials, in fp32
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) l32[m] += __builtin_amdgcn_exp2f(t[u][r]);
+            continue;
           }
 #pragma unroll
           for (int u = 0; u < 2; ++u) {
@@ -499,7 +584,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
         if constexpr (C::NS == 1) next_k();
         __builtin_amdgcn_sched_barrier(0);
         // O^T += V^T P^T: one A operand per MFMA column block c, used by every row tile
-        if (active) {
+        if (kPass != 1 && active) {
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN) {
             if (sN > 0) load_v(sN);
@@ -544,9 +629,18 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     int opaque0 = 0;
     asm volatile("" : "+v"(opaque0));
     row_of(m, opaque0, valid, head, q_off);
+    const float l_row1 = kPass == 1 ? row_groups_sum(l32[m]) : 0.f;  // the four lanes of a row, every lane taking part
     if (!valid) continue;
-    const float l_run = l_acc[m][0];
     const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+    if constexpr (kPass == 1) {
+      if (g == 0) {
+        float* st = a.stats + 2 * (q_off / hd);  // q_off = ((q0 + qi) * num_q_heads + head) * head_dim
+        st[0] = m_row;
+        st[1] = l_row1;
+      }
+      continue;
+    }
+    const float l_run = l_acc[m][0];
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;
@@ -558,7 +652,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       num_scale = m_row == -INFINITY ? 0.f : expf(m_row - mt);
       denom = num_scale * l_run + ssum;
     }
-    const float inv = num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
+    const float inv = kPass == 2 ? out_scale(p) : num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
     bf16_t* orow = out + q_off;
     if constexpr (C::TRV) {
       // MFMA c of a slice holds head_dim elements 16 c + 4 g + r of this lane's row

@@ -60,10 +60,14 @@ constexpr bool kPipeTile = D == 128 && MRT == 4;
 template <int D, int MRT>
 constexpr int kWavesPerSimd = kPipeTile<D, MRT> ? 1 : 2;
 
-template <int D, int MRT, bool kMimic>
+template <int D, int MRT, bool kMimic, int kKv, int kPass>
 __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt) {
-  if constexpr (kPipeTile<D, MRT>) prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
-  else prefill_tile<D, MRT, kMimic>(a, lds, si, s, j, qt);
+  if constexpr (kPipeTile<D, MRT>) {
+    static_assert(kKv == 0, "the pipelined tile reads a 16-bit cache");
+    prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
+  } else {
+    prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds, si, s, j, qt);
+  }
 }
 
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
@@ -320,7 +324,7 @@ void rpa_tile_kernel(TileArgs a) {
             j = rem / sz;
             member = full * kQueueRun + (rem - j * sz);
           }
-          run_prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, n_qt - 1 - member);
+          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, n_qt - 1 - member);
         }
         if (tid == 0) {
           const uint32_t done = __hip_atomic_fetch_add(&qctr[8], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -342,7 +346,7 @@ void rpa_tile_kernel(TileArgs a) {
           const int j = local / n_qt, member = local - j * n_qt;
           const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
           const int qt = (member + 5 * round0) % n_qt;
-          run_prefill_tile<D, MRT, kMimic>(a, lds_data, si, s, j, qt);
+          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, qt);
         }
       }
       // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
@@ -547,25 +551,6 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.partial_o = reinterpret_cast<float*>(ws + wl.partial_o_off);
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
-  if (stats != nullptr) {
-    // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities; both launches run
-    // every sequence through the wave-level loop.  A wavefront has half the bytes in flight that it has with a
-    // 16-bit cache, so both workgroups of a compute unit stream (0.70 ms against 0.84 ms on 256 x 512..8192 keys).
-    a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
-    int rc;
-    if (kv_elem == 2) {
-      rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)
-                             : launch_cfg<256, 1, 1, false, true, 2, 1>(a, grid, stream);
-      if (rc != RPA_OK) return rc;
-      return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 2>(a, grid, stream)
-                               : launch_cfg<256, 1, 1, false, true, 2, 2>(a, grid, stream);
-    }
-    rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
-                           : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
-    if (rc != RPA_OK) return rc;
-    return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
-                             : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
-  }
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && tune().no_mimic == 0;
   // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
   // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
@@ -585,6 +570,35 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
                             static_cast<uint64_t>(kv.v_base - kv.k_base) * 2 == kv.head_b && kv.head_b % 32 == 0 &&
                             kv.stride_b % 16 == 0 && kv.stride_b >= static_cast<uint64_t>(p.num_kv_heads) * kv.head_b &&
                             kv.page_b == static_cast<uint64_t>(p.page_size) * kv.stride_b;
+  if (stats != nullptr) {
+    // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities.  Batches of decode
+    // steps and short chunks run every sequence through the wave-level loop in both launches; a wavefront has half
+    // the bytes in flight that it has with a 16-bit cache, so both workgroups of a compute unit stream (0.70 ms
+    // against 0.84 ms on 256 x 512..8192 keys).  Batches with long chunks at head_dim 128 take the instantiation with
+    // prefill tiles, as a 16-bit cache does.
+    int rc;
+    if (!small_batch && side_by_side && p.head_dim == 128) {
+      if (kv_elem == 2) {
+        rc = launch_cfg<128, 2, 2, false, false, 2, 1>(a, grid, stream);
+        return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 2, 2>(a, grid, stream);
+      }
+      rc = launch_cfg<128, 2, 2, false, false, 1, 1>(a, grid, stream);
+      return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 1, 2>(a, grid, stream);
+    }
+    a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
+    if (kv_elem == 2) {
+      rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)
+                             : launch_cfg<256, 1, 1, false, true, 2, 1>(a, grid, stream);
+      if (rc != RPA_OK) return rc;
+      return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 2>(a, grid, stream)
+                               : launch_cfg<256, 1, 1, false, true, 2, 2>(a, grid, stream);
+    }
+    rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
+                           : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
+    if (rc != RPA_OK) return rc;
+    return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
+                             : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
+  }
   const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
     // head_dim 64: two kv heads per item where that keeps a decode token's rows in one 16-row tile

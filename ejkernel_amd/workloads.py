@@ -338,6 +338,9 @@ WORKLOADS = {
     "prefill_head_dim_64": "32 chunks x 512 tokens after 2048, 64q/8kv heads, D=64, page 32",
     # the decode batch of decode_llama3_8b with half the head_dim: K / V rows of 128 bytes
     "decode_head_dim_64": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=64, page 16",
+    # chunked prefill at the attention shape of gemma2_local's global layers (head_dim 256, soft cap, no window): the
+    # plain prefill tile's head_dim-256 instantiation
+    "prefill_head_dim_256": "16 chunks x 1024 tokens (prior 0..8192), 16q/8kv heads, D=256, page 16, cap 50",
 }
 
 
@@ -397,6 +400,12 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         kv = rng.integers(n(512), n(8192) + 1, size=S)
         return make_batch(np.ones(S, int), kv, num_q_heads=32, num_kv_heads=8, head_dim=64, page_size=16,
                           pages_per_seq=pages(n(8192), 16), seed=seed, device=device, dtype=dtype, name=name)
+    if name == "prefill_head_dim_256":
+        S, chunk = n(16), n(1024)
+        prior = rng.integers(0, n(8192) + 1, size=S)
+        return make_batch(np.full(S, chunk), prior + chunk, num_q_heads=16, num_kv_heads=8, head_dim=256, page_size=16,
+                          pages_per_seq=pages(n(8192) + chunk, 16), seed=seed, device=device, dtype=dtype, name=name,
+                          logits_soft_cap=50.0)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)

@@ -296,15 +296,21 @@ E4M3_CASES = dict(CASES)
 E4M3_CASES["long_decode"] = ([1, 1, 1, 1], [4000, 2500, 4096, 777], dict(pages_per_seq=256))
 
 
+# an 8-bit cache on the wave-level loop alone (what small batches get) and with prefill tiles forced (head_dim 128:
+# chunks of more than 64 rows per kv head then run on the tiles, in both passes)
+F8_PATHS = [pytest.param(0, id="items"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles")]
+
+
+@pytest.mark.parametrize("flags", F8_PATHS)
 @pytest.mark.parametrize("f8", BOTH_F8)
 @pytest.mark.parametrize("scales", [{}, dict(q_scale=0.05, k_scale=0.5, v_scale=2.0)], ids=["plain", "scales"])
 @pytest.mark.parametrize("case", list(E4M3_CASES))
-def test_e4m3_cache_parity_and_cache_update(case, scales, f8):
+def test_e4m3_cache_parity_and_cache_update(case, scales, f8, flags):
     q_lens, kv_lens, kw = E4M3_CASES[case]
     v = small_e4m3(q_lens, kv_lens, f8=f8, **kw)
     assert v.kv_cache.dtype == f8 and v.keys.dtype == f8 and v.kv_cache.shape[3] == 4
     ref_out, ref_cache = oracle_e4m3(v, **scales)
-    out, cache = run_hip(v, **scales)
+    out, cache = run_hip(v, flags, **scales)
     assert out.dtype == torch.bfloat16
     assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
     rows = int(sum(q_lens))
@@ -354,16 +360,17 @@ def test_e4m3_random_batches(seed):
     v = to_v3(b, seed=seed, cache_dtype=F8 if seed % 2 == 0 else torch.float8_e5m2)
     slack = np.zeros((v.queries.shape[0], v.queries.shape[1]), np.float32)
     ref_out, ref_cache = oracle_e4m3(v, slack=slack)
-    out, cache = run_hip(v)
-    assert np.array_equal(to_np(cache), ref_cache), what
-    if rows:
-        got, ref = to_np(out)[:rows].astype(np.float64), np.asarray(ref_out[:rows], np.float64)
-        d = np.abs(got - ref)
-        step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 7)
-        bound = np.maximum(2e-2, 2 * step) + 1.01 * slack[:rows, :, None] + step * (slack[:rows, :, None] > 0)
-        assert np.isfinite(got).all() and (d <= bound).all(), f"{what}: max-abs {d.max():.4g}, over the bound {(d > bound).sum()}"
-        assert d[slack[:rows] == 0].mean() <= 2e-3 if (slack[:rows] == 0).any() else True
-        assert (slack[:rows] > 0).mean() <= 0.05, f"{what}: {(slack[:rows] > 0).mean():.3f} of the rows carry an allowance"
+    for flags in (0, _native.RPA_FLAG_PREFILL_TILES):
+        out, cache = run_hip(v, flags)
+        assert np.array_equal(to_np(cache), ref_cache), what
+        if rows:
+            got, ref = to_np(out)[:rows].astype(np.float64), np.asarray(ref_out[:rows], np.float64)
+            d = np.abs(got - ref)
+            step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 7)
+            bound = np.maximum(2e-2, 2 * step) + 1.01 * slack[:rows, :, None] + step * (slack[:rows, :, None] > 0)
+            assert np.isfinite(got).all() and (d <= bound).all(), f"{what}: max-abs {d.max():.4g}, over the bound {(d > bound).sum()}"
+            assert d[slack[:rows] == 0].mean() <= 2e-3 if (slack[:rows] == 0).any() else True
+            assert (slack[:rows] > 0).mean() <= 0.05, f"{what}: {(slack[:rows] > 0).mean():.3f} of the rows carry an allowance"
 
 
 @pytest.mark.parametrize("name,n_sample,f8", [("decode_llama3_8b", 10, torch.float8_e4m3fn),
