@@ -574,16 +574,32 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // 8-bit cache: row statistics, then the attention with normalised, rounded probabilities.  Batches of decode
     // steps and short chunks run every sequence through the wave-level loop in both launches; a wavefront has half
     // the bytes in flight that it has with a 16-bit cache, so both workgroups of a compute unit stream (0.70 ms
-    // against 0.84 ms on 256 x 512..8192 keys).  Batches with long chunks at head_dim 128 take the instantiation with
-    // prefill tiles, as a 16-bit cache does.
+    // against 0.84 ms on 256 x 512..8192 keys).  Batches with long chunks take the instantiation with prefill tiles,
+    // as a 16-bit cache does.
     int rc;
-    if (!small_batch && side_by_side && p.head_dim == 128) {
-      if (kv_elem == 2) {
-        rc = launch_cfg<128, 2, 2, false, false, 2, 1>(a, grid, stream);
-        return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 2, 2>(a, grid, stream);
+    if (!small_batch && side_by_side) {
+      if (p.head_dim == 64) {
+        if (kv_elem == 2) {
+          rc = launch_cfg<64, 2, 4, false, false, 2, 1>(a, grid, stream);
+          return rc != RPA_OK ? rc : launch_cfg<64, 2, 4, false, false, 2, 2>(a, grid, stream);
+        }
+        rc = launch_cfg<64, 2, 4, false, false, 1, 1>(a, grid, stream);
+        return rc != RPA_OK ? rc : launch_cfg<64, 2, 4, false, false, 1, 2>(a, grid, stream);
       }
-      rc = launch_cfg<128, 2, 2, false, false, 1, 1>(a, grid, stream);
-      return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 1, 2>(a, grid, stream);
+      if (p.head_dim == 128) {
+        if (kv_elem == 2) {
+          rc = launch_cfg<128, 2, 2, false, false, 2, 1>(a, grid, stream);
+          return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 2, 2>(a, grid, stream);
+        }
+        rc = launch_cfg<128, 2, 2, false, false, 1, 1>(a, grid, stream);
+        return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 1, 2>(a, grid, stream);
+      }
+      if (kv_elem == 2) {
+        rc = launch_cfg<256, 1, 1, false, false, 2, 1>(a, grid, stream);
+        return rc != RPA_OK ? rc : launch_cfg<256, 1, 1, false, false, 2, 2>(a, grid, stream);
+      }
+      rc = launch_cfg<256, 1, 1, false, false, 1, 1>(a, grid, stream);
+      return rc != RPA_OK ? rc : launch_cfg<256, 1, 1, false, false, 1, 2>(a, grid, stream);
     }
     a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
     if (kv_elem == 2) {

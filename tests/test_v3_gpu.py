@@ -219,15 +219,16 @@ def test_cache_rows_padded_to_a_multiple_of_128(D, flags, window):
     assert_bf16_parity(to_np(out), ref_out, 176, f"padded rows D={D}")
 
 
+@pytest.mark.parametrize("flags", [pytest.param(0, id="items"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles")])
 @pytest.mark.parametrize("f8", [pytest.param(torch.float8_e4m3fn, id="e4m3"), pytest.param(torch.float8_e5m2, id="e5m2")])
-def test_8bit_cache_rows_padded_to_a_multiple_of_128(f8):
+def test_8bit_cache_rows_padded_to_a_multiple_of_128(f8, flags):
     v = to_v3(make_batch([5, 1, 40, 130, 0], [300, 255, 40, 200, 17], num_q_heads=8, num_kv_heads=2, head_dim=64,
                          page_size=16, pages_per_seq=32, seed=3, device=DEV), seed=3, cache_dtype=f8)
     assert v.kv_cache.shape[-1] == 128 and v.kv_cache.dtype == f8
     before = v.kv_cache.clone()
     ref_out, ref_cache = rpa_v3(*[to_np(a) for a in v.args()], cache_dtype={torch.float8_e4m3fn: "float8_e4m3fn",
                                 torch.float8_e5m2: "float8_e5m2"}[f8], query_dtype="bfloat16", **v.kwargs())
-    out, cache = run_hip(v)
+    out, cache = run_hip(v, flags)
     assert np.array_equal(to_np(cache), ref_cache), "updated cache differs"
     c8, b8 = cache.view(torch.uint8), before.view(torch.uint8)
     written = (c8[..., :64] != b8[..., :64]).flatten(2).any(-1)
@@ -296,8 +297,8 @@ E4M3_CASES = dict(CASES)
 E4M3_CASES["long_decode"] = ([1, 1, 1, 1], [4000, 2500, 4096, 777], dict(pages_per_seq=256))
 
 
-# an 8-bit cache on the wave-level loop alone (what small batches get) and with prefill tiles forced (head_dim 128:
-# chunks of more than 64 rows per kv head then run on the tiles, in both passes)
+# an 8-bit cache on the wave-level loop alone (what small batches get) and with prefill tiles forced (chunks of more
+# than 64 rows per kv head then run on the tiles, in both passes)
 F8_PATHS = [pytest.param(0, id="items"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles")]
 
 
