@@ -414,7 +414,7 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
       return rpa::fail(RPA_ERR_UNSUPPORTED, "an 8-bit cache takes bf16 queries and RPA_COMPUTE_BF16");
     if (!rpa::tiled_supported(v.attn))
       return rpa::fail(RPA_ERR_UNSUPPORTED,
-                       "an 8-bit cache runs on the MFMA kernel only (head_dim 64 / 128 / 256, page_size a power of two >= 4, "
+                       "an 8-bit cache runs on the MFMA kernel only (head_dim a multiple of 16 in 64..256, page_size a power of two >= 4, "
                        "no RPA_FLAG_FORCE_GENERIC)");
     const uint64_t need = rpa_v3_workspace_bytes(&v);
     if (v.attn.workspace == nullptr || v.attn.workspace_bytes < need)

@@ -117,7 +117,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       if (pair) {
         // contraction index 64 hp .. 64 hp + 63 carries this row's query; the other head's half stays zero
         if (row_valid && (ks >> 1) == hp) raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * (ks & 1) + 8 * g);
-      } else if (row_valid && 32 * ks < hd) {
+      } else if (row_valid && 32 * ks + 8 * g < hd) {
         raw = *reinterpret_cast<const u32x4_t*>(q + q_row_off + 32 * ks + 8 * g);
       }
       u32x4_t sc;
@@ -166,7 +166,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const float inv_cap = cap != 0.f ? 1.f / cap : 0.f;
 
   using raw_t = typename std::conditional<kKv != 0, u32x2_t, u32x4_t>::type;  // one lane's piece: eight elements
-  constexpr uint32_t PIECE_B = kKv != 0 ? 8u : 16u, SLICE_B = 16u * PIECE_B;
+  constexpr uint32_t PIECE_B = kKv != 0 ? 8u : 16u;
   raw_t kreg[C::NSLOT][C::NS];
   raw_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
 
@@ -183,7 +183,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const uint32_t stride_b = a.kv.stride_b;            // bytes between tokens
   const uint64_t page_b = a.kv.page_b;
   const uint32_t head_off = static_cast<uint32_t>(pair ? 2 * j : j) * a.kv.head_b;
-  const int piece = i & (hd / 8 - 1);  // i itself from head_dim 128 up
+  // A head_dim below the instantiation's width: the lanes past the row's last piece fetch a piece that exists (a
+  // repeat of the lower half where the piece count is a power of two, which the head pairs count on; else the last
+  // one) -- in K it meets the zeros q is padded with, in V it feeds output elements that are not stored.
+  const int npieces = hd / 8;
+  const int piece = (npieces & (npieces - 1)) == 0 ? (i & (npieces - 1)) : min(i, npieces - 1);  // i itself from head_dim 128 up
+  uint32_t slice_off[C::NS];  // this lane's piece of 128-slice sN, from its piece of slice 0
+#pragma unroll
+  for (int sN = 0; sN < C::NS; ++sN)
+    slice_off[sN] = sN == 0 ? 0u : PIECE_B * static_cast<uint32_t>(min(i + 16 * sN, npieces - 1) - piece);
   // this lane's piece inside a token's record; with a head pair, pieces 8..15 are those of the second head
   const uint32_t piece_off = head_off + PIECE_B * static_cast<uint32_t>(piece) + (pair && i >= 8 ? a.kv.head_b : 0u);
   const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + piece_off;
@@ -202,8 +210,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const char* row_v = row + v_delta;
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN) {
-            kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + (lane_off + SLICE_B * sN));
-            if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row_v + (lane_off + SLICE_B * sN));
+            kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + (lane_off + slice_off[sN]));
+            if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row_v + (lane_off + slice_off[sN]));
           }
         }
       }
@@ -222,8 +230,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
-          kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + SLICE_B * sN);
-          if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + v_delta + SLICE_B * sN);
+          kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + slice_off[sN]);
+          if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + v_delta + slice_off[sN]);
         }
       }
     }
@@ -384,6 +392,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       sink_part = sink_keys > 0;
       if (sink_part) {
         // one wave-wide load of 16 bytes per lane covers 64 / (hd / 8) whole rows, laid out row after row
+        // (a load that covers no whole number of rows spills its tail past the last staged row: the K region and the V
+        // region are SINK_KEYS rows of the instantiation's width each, which holds that tail for every head_dim)
         const int pieces = hd >> 3, rows_per = kWave / pieces;
         const int staged = min(sink_keys, C::SINK_KEYS);
         for (int r0 = 0; r0 < staged; r0 += rows_per) {
@@ -391,7 +401,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(src),
                                            (__attribute__((address_space(3))) void*)(lds_sink + r0 * hd * 2), 16, 0, 0);
           __builtin_amdgcn_global_load_lds(reinterpret_cast<const u32x4_t*>(src + v_delta),
-                                           (__attribute__((address_space(3))) void*)(lds_sink + (C::SINK_KEYS + r0) * hd * 2), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void*)(lds_sink + C::SINK_KEYS * D * 2 + r0 * hd * 2), 16, 0, 0);
         }
         // the biases of those positions for the 16 rows of this row tile, [row][key]: 4 bytes per lane, 8 rows per load
 #pragma unroll
@@ -436,10 +446,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           for (int r = 0; r < 4; ++r) vv[sN][r] = u32x4_t{0u, 0u, 0u, 0u};
         if (k < C::SINK_KEYS) {
           const char* krow = lds_sink + k * hd * 2;
-          const char* vrow = krow + C::SINK_KEYS * hd * 2;
+          const char* vrow = lds_sink + C::SINK_KEYS * D * 2 + k * hd * 2;
 #pragma unroll
           for (int ks = 0; ks < C::NKS; ++ks)
-            if (32 * ks < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
+            if (32 * ks + 8 * g < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
@@ -451,7 +461,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const char* vrow = krow + v_delta;
 #pragma unroll
           for (int ks = 0; ks < C::NKS; ++ks)
-            if (32 * ks < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
+            if (32 * ks + 8 * g < hd) kk[ks] = *reinterpret_cast<const u32x4_t*>(krow + 2 * (32 * ks + 8 * g));
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll

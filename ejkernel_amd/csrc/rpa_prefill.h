@@ -95,7 +95,11 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // (A head_dim below the instantiation's runs too: q is padded with zeros and the upper part of every K / V row in
   // LDS repeats the lower part -- K: multiplied by zero; V: output elements that are not stored.)
   const int hd = p.head_dim;
-  const uint32_t pmask = static_cast<uint32_t>(hd / 8 - 1);  // 16-byte pieces of a row that exist in memory
+  // Pieces (eight elements) of a row that exist in memory: a slot past the last one takes a piece that does exist -- a
+  // repeat of the lower ones where their count is a power of two, else the last one.
+  const uint32_t npieces = static_cast<uint32_t>(hd / 8);
+  const bool pieces_pow2 = (npieces & (npieces - 1)) == 0;
+  auto piece_of = [&](uint32_t slot) { return pieces_pow2 ? (slot & (npieces - 1)) : min(slot, npieces - 1); };
 
   // ---- key range of the workgroup's rows
   const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
@@ -140,7 +144,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int ks = 0; ks < C::NKS; ++ks) {
       u32x4_t raw = {0u, 0u, 0u, 0u};
-      if (valid && 32 * ks < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
+      if (valid && 32 * ks + 8 * g < hd) raw = *reinterpret_cast<const u32x4_t*>(q + q_off + 32 * ks + 8 * g);
       u32x4_t sc;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -234,14 +238,14 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
   // (Without the transposing read the V tile is laid out like the K tile.)
   const int v_row = C::TRV ? (lane >> 1) % C::RB : l_row;
-  const uint32_t v_src = PB * (static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)) & pmask);  // byte offset in the row
+  const uint32_t v_src = PB * piece_of(static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)));  // byte offset in the row
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
   uint32_t pre_off[HB];  // per-lane byte offset of K block n inside the group: row part + swizzled piece
 #pragma unroll
   for (int n = 0; n < HB; ++n) {
     const int t_local = GROUP * wave + C::RB * n + l_row;
-    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + PB * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
+    pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + PB * piece_of(static_cast<uint32_t>(l_slot ^ C::swz(t_local)));
   }
   const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + v_delta;  // V block 0; block n adds RB rows
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
@@ -294,7 +298,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     for (int n = 0; n < HB; ++n) {
       const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
       const int t_local = GROUP * wave + C::RB * n + l_row;
-      const uint32_t k_piece = PB * (static_cast<uint32_t>(l_slot ^ C::swz(t_local)) & pmask);
+      const uint32_t k_piece = PB * piece_of(static_cast<uint32_t>(l_slot ^ C::swz(t_local)));
       const uint32_t v_piece = C::TRV ? v_src : k_piece;
       if (C::RB > 4 && p.page_size < C::RB) {
         // pages shorter than a block (pages of 4 tokens under 128-byte rows): every lane looks its own row's page up
@@ -674,7 +678,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
           u32x4_t w;
 #pragma unroll
           for (int e = 0; e < 4; ++e) w[e] = pack_bf16x2(o_acc[m][sN][2 * e][r] * inv, o_acc[m][sN][2 * e + 1][r] * inv);
-          *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
+          if (128 * sN + 32 * g + 8 * r < hd) *reinterpret_cast<u32x4_t*>(orow + 128 * sN + 32 * g + 8 * r) = w;
         }
     }
   }

@@ -481,7 +481,8 @@ static int tiled_grid() { return device_cu_count() * tune().wgs_per_cu; }
 bool tiled_supported(const RpaParams& p) {
   if (p.flags & RPA_FLAG_FORCE_GENERIC) return false;
   if (p.dtype != RPA_DTYPE_BF16 || p.compute != RPA_COMPUTE_BF16) return false;
-  if (p.head_dim != 64 && p.head_dim != 128 && p.head_dim != 256) return false;
+  // 64, 128 and 256 have instantiations of their own width; other multiples of 16 in between run on the next wider one
+  if (p.head_dim < 64 || p.head_dim > 256 || p.head_dim % 16 != 0) return false;
   if (p.page_size < 4 || (p.page_size & (p.page_size - 1)) != 0) return false;  // shift/mask page arithmetic
   if (p.max_num_seqs > (kTiledMaxSeqs << kTiledMaxSchedShift)) return false;
   if (static_cast<uint64_t>(p.max_num_seqs) * p.num_kv_heads * 4 > kQueueCounterIndex * 4ull) return false;
@@ -586,7 +587,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
         rc = launch_cfg<64, 2, 4, false, false, 1, 1>(a, grid, stream);
         return rc != RPA_OK ? rc : launch_cfg<64, 2, 4, false, false, 1, 2>(a, grid, stream);
       }
-      if (p.head_dim == 128) {
+      if (p.head_dim <= 128) {
         if (kv_elem == 2) {
           rc = launch_cfg<128, 2, 2, false, false, 2, 1>(a, grid, stream);
           return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 2, 2>(a, grid, stream);
@@ -633,7 +634,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // chunks with many decode sequences is bound by its decode stream, which needs a streaming workgroup on every
     // compute unit beside the prefill tiles (two workgroups per unit: the plain tile).  The host cannot see the lengths,
     // so it goes by the average number of query tokens per sequence.
-    const bool pipe_ok = p.page_size >= 16 && p.logits_soft_cap == 0.f &&
+    const bool pipe_ok = p.head_dim == 128 && p.page_size >= 16 && p.logits_soft_cap == 0.f &&
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
     const bool pipe_wanted = (p.flags & RPA_FLAG_PLAIN_TILES) == 0 &&
                              ((p.flags & RPA_FLAG_PIPE_TILES) != 0 ||

@@ -354,6 +354,27 @@ def test_bf16_random_batches(seed):
         assert not out[rows:].any()
 
 
+@pytest.mark.parametrize("seed", range(3000, 3040))
+def test_bf16_random_batches_head_dims_between_the_instantiated_ones(seed):
+    """head_dim 80, 96, 112 run on the 128-wide MFMA kernel and 144, 160, 192, 224 on the 256-wide one (q padded with
+    zeros, the lanes past a row's last 16-byte piece fetching a piece that exists, output elements past head_dim not
+    stored): same bounds as the other random batches, on the wave-level loop, the plain prefill tiles and the scalar
+    kernel, and nothing written outside the rows of `out`."""
+    b, what = random_rpa_batch(seed, DEV, head_dims=(80, 96, 112, 144, 160, 192, 224))
+    rows = b.total_valid_tokens
+    strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
+    finite = np.isfinite(strict).all(axis=(1, 2))
+    for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_PIPE_TILES,
+                  _native.RPA_FLAG_FORCE_GENERIC):
+        out = to_np(run_hip(b, flags))
+        assert np.isfinite(out[:rows]).all(), what
+        if finite.any():
+            assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}")
+        mx, mean = err_stats(out, exact, rows)
+        assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
+        assert not out[rows:].any()
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("D", [16, 128])
 def test_cap_that_bf16_does_not_hold_is_rounded_before_use(flags, D):

@@ -237,13 +237,15 @@ def test_8bit_cache_rows_padded_to_a_multiple_of_128(f8, flags):
     assert_bf16_parity(to_np(out), ref_out, 176, "8-bit padded rows")
 
 
-@pytest.mark.parametrize("seed", range(300, 316))
+@pytest.mark.parametrize("seed", range(300, 332))
 def test_bf16_random_batches_head_dim_64(seed):
-    """Seeded random shapes at head_dim 64 (cache rows padded to 128): the cache bit for bit, outputs within the bound."""
-    b, what = random_rpa_batch(seed, DEV, head_dims=(64,))
+    """Seeded random shapes at head_dim 64 (cache rows padded to 128) and, from seed 316 on, at head dims between the
+    instantiated ones (96, 80, 192, 160: rows padded to 128 or 256): the cache bit for bit, outputs within the bound."""
+    dims = (64,) if seed < 316 else (80, 96, 160, 192)
+    b, what = random_rpa_batch(seed, DEV, head_dims=dims)
     rows = b.total_valid_tokens
     for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, _native.RPA_FLAG_FORCE_GENERIC):
-        v = to_v3(random_rpa_batch(seed, DEV, head_dims=(64,))[0], seed=seed)
+        v = to_v3(random_rpa_batch(seed, DEV, head_dims=dims)[0], seed=seed)
         ref_out, ref_cache = oracle(v)
         out, cache = run_hip(v, flags)
         assert np.array_equal(to_np(cache), ref_cache), what
@@ -356,7 +358,8 @@ def test_e4m3_random_batches(seed):
     step of that probability times the value row: the restatement reports that allowance per row (zero nearly
     everywhere) and it is added to the bound.  Seeds 1123 and 1341 hold such a row (0.027 and 0.19 from the
     restatement in one (token, head) row each, every other row bit for bit)."""
-    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256))   # an odd number of kv heads pads the packed cache
+    # an odd number of kv heads pads the packed cache; head_dim 96 and 192 live in rows of 128 and 256 bytes
+    b, what = random_rpa_batch(seed, DEV, head_dims=(128, 256) if seed < 230 or seed > 1000 else (96, 192))
     rows = b.total_valid_tokens
     v = to_v3(b, seed=seed, cache_dtype=F8 if seed % 2 == 0 else torch.float8_e5m2)
     slack = np.zeros((v.queries.shape[0], v.queries.shape[1]), np.float32)
