@@ -276,8 +276,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
       for (int u = 0; u < NT; ++u)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-          sv[u][r] = soft_cap<kMimic>(sv[u][r], cap, inv_cap);
+        for (int r = 0; r < 4; r += 2) soft_cap2<kMimic>(sv[u][r], sv[u][r + 1], cap, inv_cap);
     }
     if (need_mask) {
 #pragma unroll

@@ -471,8 +471,10 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
-              for (int r = 0; r < 4; ++r)  // the cap's own bf16 roundings make it sensitive to its input: round that too
-                sv[u][r] = soft_cap<kMimic>(kMimic ? rbf(sv[u][r]) : sv[u][r], cap, inv_cap);
+              for (int r = 0; r < 4; r += 2) {  // the cap's own bf16 roundings make it sensitive to its input: round that too
+                if (kMimic) rbf2(sv[u][r], sv[u][r + 1]);
+                soft_cap2<kMimic>(sv[u][r], sv[u][r + 1], cap, inv_cap);
+              }
           }
           else if (kMimic && D >= RPA_ROUND_MIN_D) {
             // the reference's logits are bf16 (_xla_impl_fwd.py:119-124): round them, two per conversion (head_dim 64

@@ -171,11 +171,41 @@ __device__ __forceinline__ float tanh_fast(float x) {
   const float small = x * fmaf(x2, fmaf(x2, 2.f / 15.f, -1.f / 3.f), 1.f);
   return fabsf(x) < 0.0625f ? small : big;
 }
+// tanh of a bf16 value whose result the caller rounds to bf16.  Below 1/32 the result rounds back to the argument
+// (tanh(y) = y (1 - y^2/3 + ...) and y^2/3 < 3.3e-4 there, a sixth of the smallest relative half-step of bf16, 2^-9),
+// so the series of tanh_fast is not needed; from 1/32 up 1 - 2 / (1 + e^(2y)) is accurate to 5e-6 relative.
+__device__ __forceinline__ float tanh_of_bf16(float y) {
+  const float e = __builtin_amdgcn_exp2f(y * (2.f * kLog2e));
+  const float big = fmaf(-2.f, __builtin_amdgcn_rcpf(1.f + e), 1.f);
+  return fabsf(y) < 0.03125f ? y : big;
+}
+// Two values rounded to bf16 with one packed conversion.
+__device__ __forceinline__ void rbf2(float& a, float& b) {
+  const uint32_t pk = pack_bf16x2(a, b);
+  a = __uint_as_float(pk << 16);
+  b = __uint_as_float(pk & 0xffff0000u);
+}
 // cap * tanh(x / cap) with the reference's bf16 rounding after each op (kMimic) or in plain fp32.
 template <bool kMimic>
 __device__ __forceinline__ float soft_cap(float x, float cap, float inv_cap) {
-  if (kMimic) return rbf(rbf(tanh_fast(rbf(x * inv_cap))) * cap);
+  if (kMimic) return rbf(rbf(tanh_of_bf16(rbf(x * inv_cap))) * cap);
   return cap * tanh_fast(x * inv_cap);
+}
+// The same for two logits at once: the roundings share their conversions.
+template <bool kMimic>
+__device__ __forceinline__ void soft_cap2(float& a, float& b, float cap, float inv_cap) {
+  if (kMimic) {
+    float ya = a * inv_cap, yb = b * inv_cap;
+    rbf2(ya, yb);
+    float ta = tanh_of_bf16(ya), tb = tanh_of_bf16(yb);
+    rbf2(ta, tb);
+    a = ta * cap;
+    b = tb * cap;
+    rbf2(a, b);
+  } else {
+    a = cap * tanh_fast(a * inv_cap);
+    b = cap * tanh_fast(b * inv_cap);
+  }
 }
 
 // Reductions over the four lane groups that hold one query row (lanes l, l^16, l^32, l^48), with the gfx950
