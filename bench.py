@@ -453,7 +453,7 @@ def sustain(fn, seconds, what, flops=None, nbytes=None, quiet=False):
 
 # (vector elements, LDS operand reads) per block of 32 MFMAs that csrc/probe_mfma_mix.hip instantiates; an element is
 # 5.5 vector instructions, so 24 elements with 16 reads is about the mix of the pipelined prefill tile's key loop
-MFMA_MIXES = [(0, 0), (0, 16), (24, 0), (24, 16), (48, 0), (48, 16), (64, 16)]
+MFMA_MIXES = [(0, 0), (-16, 0), (0, 16), (24, 0), (24, 16), (48, 0), (48, 16), (64, 16)]  # -16: 64 MFMAs of 16x16x32 instead
 
 
 def mfma_mix_probe(seconds):

@@ -83,6 +83,39 @@ void mfma_mix_kernel(const uint4* __restrict__ src, float* __restrict__ dst, uns
   }
 }
 
+// The same matrix work as 64 v_mfma_f32_16x16x32_bf16 per block (the shape the plain prefill tile and the decode loop
+// use) and nothing else: what the smaller shape costs against the larger one.
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1)))
+void mfma_16x16_kernel(const uint4* __restrict__ src, float* __restrict__ dst, unsigned long long* __restrict__ clocks, int iters) {
+  typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+  const int tid = threadIdx.x;
+  const unsigned long long c0 = __builtin_readcyclecounter(), r0 = __builtin_amdgcn_s_memrealtime();
+  bf16x8_t a[4], b[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    a[k] = __builtin_bit_cast(bf16x8_t, src[kLdsPieces + tid * 8 + k]);
+    b[k] = __builtin_bit_cast(bf16x8_t, src[kLdsPieces + tid * 8 + 4 + k]);
+  }
+  f32x4_t acc[16];
+#pragma unroll
+  for (int k = 0; k < 16; ++k) acc[k] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int it = 0; it < iters; ++it) {
+#pragma unroll
+    for (int m = 0; m < 64; ++m)
+      acc[m & 15] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[m & 3], b[(m >> 2) & 3], acc[m & 15], 0, 0, 0);
+  }
+  float total = 0.f;
+#pragma unroll
+  for (int k = 0; k < 16; ++k)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) total += acc[k][r];
+  dst[blockIdx.x * 256 + tid] = total;
+  if (tid == 0) {
+    clocks[2 * blockIdx.x] = __builtin_readcyclecounter() - c0;
+    clocks[2 * blockIdx.x + 1] = __builtin_amdgcn_s_memrealtime() - r0;
+  }
+}
+
 template <int E, int L>
 int launch(int grid, const void* src, void* dst, void* clocks, int iters, hipStream_t stream) {
   hipLaunchKernelGGL((mfma_mix_kernel<E, L>), dim3(grid), dim3(256), 0, stream, static_cast<const uint4*>(src),
@@ -98,7 +131,7 @@ extern "C" {
 uint64_t mfma_mix_probe_src_bytes(void) { return static_cast<uint64_t>(kSrcPieces) * 16; }
 
 // One launch on `grid` workgroups (dst: grid * 256 floats; clocks: per workgroup the shader-clock cycles and the
-// 100 MHz ticks its loop took).  Returns the floating-point operations of the launch's MFMAs, or 0 for a mix that is
+// 100 MHz ticks its loop took).  vector_elements = -16 selects 64 MFMAs of the 16x16x32 shape per block, alone.  Returns the floating-point operations of the launch's MFMAs, or 0 for a mix that is
 // not instantiated.
 double mfma_mix_probe_launch(int vector_elements, int lds_reads, int grid, int iters, const void* src, void* dst, void* clocks,
                              void* stream) {
@@ -111,6 +144,11 @@ double mfma_mix_probe_launch(int vector_elements, int lds_reads, int grid, int i
   else if (vector_elements == 24 && lds_reads == 16) rc = launch<24, 16>(grid, src, dst, clocks, iters, s);
   else if (vector_elements == 48 && lds_reads == 16) rc = launch<48, 16>(grid, src, dst, clocks, iters, s);
   else if (vector_elements == 64 && lds_reads == 16) rc = launch<64, 16>(grid, src, dst, clocks, iters, s);
+  else if (vector_elements == -16 && lds_reads == 0) {  // the 16x16x32 shape, MFMAs alone
+    hipLaunchKernelGGL(mfma_16x16_kernel, dim3(grid), dim3(256), 0, s, static_cast<const uint4*>(src), static_cast<float*>(dst),
+                       static_cast<unsigned long long*>(clocks), iters);
+    rc = hipGetLastError() == hipSuccess ? 0 : -4;
+  }
   if (rc != 0) return 0.0;
   return static_cast<double>(grid) * 4.0 * iters * 32.0 * (2.0 * 32 * 32 * 16);
 }
