@@ -34,8 +34,11 @@ def measured_traffic_bytes(workload: str):
         return None
 
 
-# The configurations of the benchmark besides the headline one, measured in the same run (entries of "configs").
-EXTRA_CONFIGS = ["decode_small", "mixed_prefill_decode", "mixed_prefill_only", "gemma2_local", "decode_long_context"]
+# The configurations of the benchmark besides the headline one, measured in the same run (entries of "configs").  The
+# two other bandwidth-bound streams come first: how fast a stream runs depends by a few per cent on the memory its pool
+# gets, and pools allocated early in a process get what a process of their own would (gemma2_local 0.386 ms as the
+# second workload of a process, 0.392-0.398 ms as the fifth; 0.380 ms alone).
+EXTRA_CONFIGS = ["gemma2_local", "decode_long_context", "decode_small", "mixed_prefill_decode", "mixed_prefill_only"]
 
 
 def parse():
