@@ -341,6 +341,10 @@ WORKLOADS = {
     # chunked prefill at the attention shape of gemma2_local's global layers (head_dim 256, soft cap, no window): the
     # plain prefill tile's head_dim-256 instantiation
     "prefill_head_dim_256": "16 chunks x 1024 tokens (prior 0..8192), 16q/8kv heads, D=256, page 16, cap 50",
+    # a head_dim between the instantiated widths (rows of 192 bytes on the 128-wide kernel): the decode batch of
+    # decode_llama3_8b and a mixed batch, 16 chunks x 256 tokens beside 112 decode sequences
+    "decode_head_dim_96": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=96, page 16",
+    "mixed_head_dim_96": "16 chunks x 256 tokens (prior 0..2048) + 112 decode seqs (kv 256..4096), 32q/8kv heads, D=96, page 32",
 }
 
 
@@ -406,6 +410,20 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         return make_batch(np.full(S, chunk), prior + chunk, num_q_heads=16, num_kv_heads=8, head_dim=256, page_size=16,
                           pages_per_seq=pages(n(8192) + chunk, 16), seed=seed, device=device, dtype=dtype, name=name,
                           logits_soft_cap=50.0)
+    if name == "decode_head_dim_96":
+        S = n(256)
+        kv = rng.integers(n(512), n(8192) + 1, size=S)
+        return make_batch(np.ones(S, int), kv, num_q_heads=32, num_kv_heads=8, head_dim=96, page_size=16,
+                          pages_per_seq=pages(n(8192), 16), seed=seed, device=device, dtype=dtype, name=name)
+    if name == "mixed_head_dim_96":
+        n_pre, n_dec, chunk = n(16), n(112), n(256)
+        prior = rng.integers(0, n(2048) + 1, size=n_pre)
+        kv_dec = rng.integers(n(256), n(4096) + 1, size=n_dec)
+        q = np.concatenate([np.full(n_pre, chunk), np.ones(n_dec, int)])
+        kv = np.concatenate([prior + chunk, kv_dec])
+        order = rng.permutation(n_pre + n_dec)
+        return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=96, page_size=32,
+                          pages_per_seq=pages(max(n(4096), n(2048) + chunk), 32), seed=seed, device=device, dtype=dtype, name=name)
     if name == "gemma2_local":
         S = n(64)
         kv = rng.integers(n(2048), n(32768) + 1, size=S)

@@ -58,7 +58,9 @@ def permuted(b, seed=9):
 
 @pytest.mark.parametrize("name,n_sample,permute", [("decode_small", 8, True), ("decode_llama3_8b", 12, True),
                                                    ("mixed_prefill_decode", 14, True), ("mixed_prefill_only", 3, True),
-                                                   ("gemma2_local", 4, False), ("decode_long_context", 2, False)])
+                                                   ("gemma2_local", 4, False), ("decode_long_context", 2, False),
+                                                   ("decode_head_dim_96", 12, True), ("mixed_head_dim_96", 10, True),
+                                                   ("prefill_head_dim_256", 1, True), ("decode_head_dim_64", 12, True)])
 def test_full_size_workload(name, n_sample, permute):
     b = make_workload(name, device=DEV)
     out = run(b)
