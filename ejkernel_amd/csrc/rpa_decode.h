@@ -572,58 +572,78 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
       const bool rv = rrow < R;
       constexpr int kChunk = C::NS == 1 ? 2 : 1;
       const uint64_t* ml = reinterpret_cast<const uint64_t*>(a.partial_ml) + rrow;
-      if (rv)
-        for (int k0 = part.first_w; k0 <= part.last_w; k0 += 4 * pp) {
-          uint64_t v[4];
-#pragma unroll
-          for (int c = 0; c < 4; ++c) {
-            const int k = min(k0 + c * pp + sub, part.last_w);
-            v[c] = __hip_atomic_load(ml + static_cast<size_t>(part_slot(k, part.stream_a, part.sh)) * 16, __ATOMIC_RELAXED,
-                                     __HIP_MEMORY_SCOPE_AGENT);
-          }
-#pragma unroll
-          for (int c = 0; c < 4; ++c) M = fmaxf(M, __uint_as_float(static_cast<uint32_t>(v[c])));
-        }
-#pragma unroll
-      for (int d = 1; d < 16; d <<= 1)
-        if (d >= rp) M = fmaxf(M, __shfl_xor(M, d, kWave));
-      const float M_use = M == -INFINITY ? 0.f : M;
+      // One pass with a reference point of the lane's own that moves as parts come in (the parts' maxima are not read
+      // ahead of their sums: that was a memory round trip of its own per 16 parts), and the next chunk's loads are in
+      // flight while the current one is added: a merge of 128 parts waits for about three round trips instead of 24.
+      float Mi = -INFINITY;
 #pragma unroll
       for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
         for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
       if (rv) {
-        for (int k0 = part.first_w; k0 <= part.last_w; k0 += kChunk * pp) {
-          uint64_t mlv[kChunk];
-          u32x4_t ov[kChunk][C::NS][8];
+        const int step = kChunk * pp;
+        uint64_t ml_a[kChunk], ml_b[kChunk];
+        u32x4_t ov_a[kChunk][C::NS][8], ov_b[kChunk][C::NS][8];
+        auto fetch = [&](int k0, uint64_t (&mlv)[kChunk], u32x4_t (&ov)[kChunk][C::NS][8]) {
 #pragma unroll
           for (int c = 0; c < kChunk; ++c) {
             const size_t sl = part_slot(min(k0 + c * pp + sub, part.last_w), part.stream_a, part.sh);
             mlv[c] = __hip_atomic_load(ml + sl * 16, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             if constexpr (kPass != 1)
 #pragma unroll
-            for (int sN = 0; sN < C::NS; ++sN)
+              for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int cc = 0; cc < 8; ++cc)
-                ov[c][sN][cc] = __builtin_amdgcn_raw_buffer_load_b128(slots_rsrc, slot_piece(static_cast<uint32_t>(sl), sN * 8 + cc, rrow),
-                                                                      0, kAgentScope);
+                for (int cc = 0; cc < 8; ++cc)
+                  ov[c][sN][cc] = __builtin_amdgcn_raw_buffer_load_b128(slots_rsrc, slot_piece(static_cast<uint32_t>(sl), sN * 8 + cc, rrow),
+                                                                        0, kAgentScope);
           }
+        };
+        auto take = [&](int k0, const uint64_t (&mlv)[kChunk], const u32x4_t (&ov)[kChunk][C::NS][8]) {
 #pragma unroll
           for (int c = 0; c < kChunk; ++c) {
             if (k0 + c * pp + sub > part.last_w) continue;  // past the last part: the load repeated it, it is not added again
             const float mk = __uint_as_float(static_cast<uint32_t>(mlv[c]));
             const float lk = __uint_as_float(static_cast<uint32_t>(mlv[c] >> 32));
-            const float w = __builtin_amdgcn_exp2f((mk - M_use) * kLog2e);
-            L += w * lk;
+            const float m_new = fmaxf(Mi, mk);
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;
+            const float keep = __builtin_amdgcn_exp2f((Mi - m_use) * kLog2e);  // 1 while the point stays, 0 for the first part
+            const float w = __builtin_amdgcn_exp2f((mk - m_use) * kLog2e);
+            L = L * keep + w * lk;
+            Mi = m_new;
             if constexpr (kPass != 1)
 #pragma unroll
-            for (int sN = 0; sN < C::NS; ++sN)
+              for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
-              for (int cc = 0; cc < 8; ++cc)
+                for (int cc = 0; cc < 8; ++cc)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) o_acc[sN][cc][r] += w * __uint_as_float(ov[c][sN][cc][r]);
+                  for (int r = 0; r < 4; ++r) o_acc[sN][cc][r] = o_acc[sN][cc][r] * keep + w * __uint_as_float(ov[c][sN][cc][r]);
+          }
+        };
+        fetch(part.first_w, ml_a, ov_a);
+        for (int k0 = part.first_w; k0 <= part.last_w; k0 += 2 * step) {
+          const bool second = k0 + step <= part.last_w;
+          if (second) fetch(k0 + step, ml_b, ov_b);
+          take(k0, ml_a, ov_a);
+          if (second) {
+            if (k0 + 2 * step <= part.last_w) fetch(k0 + 2 * step, ml_a, ov_a);
+            take(k0 + step, ml_b, ov_b);
           }
         }
+      }
+      // the lanes of one row: a common reference point, then sums
+      M = Mi;
+#pragma unroll
+      for (int d = 1; d < 16; d <<= 1)
+        if (d >= rp) M = fmaxf(M, __shfl_xor(M, d, kWave));
+      {
+        const float M_use = M == -INFINITY ? 0.f : M;
+        const float to_row = __builtin_amdgcn_exp2f((Mi - M_use) * kLog2e);  // 0 for a lane that took no part
+        L *= to_row;
+        if constexpr (kPass != 1)
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int c = 0; c < 8; ++c) o_acc[sN][c] *= to_row;
       }
 #pragma unroll
       for (int d = 1; d < 16; d <<= 1)
