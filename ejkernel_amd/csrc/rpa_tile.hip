@@ -523,6 +523,18 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
+// 8-bit cache (kv_elem 1 = e4m3, 2 = e5m2): the statistics launch, then the attention launch.
+template <int D, int NT, int MRT, bool kWaveOnly>
+static int launch_two_pass(int kv_elem, const TileArgs& a, int grid, hipStream_t stream) {
+  int rc;
+  if (kv_elem == 2) {
+    rc = launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 1>(a, grid, stream);
+    return rc != RPA_OK ? rc : launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 2>(a, grid, stream);
+  }
+  rc = launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 1>(a, grid, stream);
+  return rc != RPA_OK ? rc : launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 2>(a, grid, stream);
+}
+
 static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre, float* stats,
                              int kv_elem = 0) {
   WorkspaceLayout wl;
@@ -577,44 +589,14 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // the bytes in flight that it has with a 16-bit cache, so both workgroups of a compute unit stream (0.70 ms
     // against 0.84 ms on 256 x 512..8192 keys).  Batches with long chunks take the instantiation with prefill tiles,
     // as a 16-bit cache does.
-    int rc;
     if (!small_batch && side_by_side) {
-      if (p.head_dim == 64) {
-        if (kv_elem == 2) {
-          rc = launch_cfg<64, 2, 4, false, false, 2, 1>(a, grid, stream);
-          return rc != RPA_OK ? rc : launch_cfg<64, 2, 4, false, false, 2, 2>(a, grid, stream);
-        }
-        rc = launch_cfg<64, 2, 4, false, false, 1, 1>(a, grid, stream);
-        return rc != RPA_OK ? rc : launch_cfg<64, 2, 4, false, false, 1, 2>(a, grid, stream);
-      }
-      if (p.head_dim <= 128) {
-        if (kv_elem == 2) {
-          rc = launch_cfg<128, 2, 2, false, false, 2, 1>(a, grid, stream);
-          return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 2, 2>(a, grid, stream);
-        }
-        rc = launch_cfg<128, 2, 2, false, false, 1, 1>(a, grid, stream);
-        return rc != RPA_OK ? rc : launch_cfg<128, 2, 2, false, false, 1, 2>(a, grid, stream);
-      }
-      if (kv_elem == 2) {
-        rc = launch_cfg<256, 1, 1, false, false, 2, 1>(a, grid, stream);
-        return rc != RPA_OK ? rc : launch_cfg<256, 1, 1, false, false, 2, 2>(a, grid, stream);
-      }
-      rc = launch_cfg<256, 1, 1, false, false, 1, 1>(a, grid, stream);
-      return rc != RPA_OK ? rc : launch_cfg<256, 1, 1, false, false, 1, 2>(a, grid, stream);
+      if (p.head_dim == 64) return launch_two_pass<64, 2, 4, false>(kv_elem, a, grid, stream);
+      if (p.head_dim <= 128) return launch_two_pass<128, 2, 2, false>(kv_elem, a, grid, stream);
+      return launch_two_pass<256, 1, 1, false>(kv_elem, a, grid, stream);
     }
     a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
-    if (kv_elem == 2) {
-      rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 1>(a, grid, stream)
-                             : launch_cfg<256, 1, 1, false, true, 2, 1>(a, grid, stream);
-      if (rc != RPA_OK) return rc;
-      return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 2, 2>(a, grid, stream)
-                               : launch_cfg<256, 1, 1, false, true, 2, 2>(a, grid, stream);
-    }
-    rc = p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 1>(a, grid, stream)
-                           : launch_cfg<256, 1, 1, false, true, 1, 1>(a, grid, stream);
-    if (rc != RPA_OK) return rc;
-    return p.head_dim <= 128 ? launch_cfg<128, 2, 2, false, true, 1, 2>(a, grid, stream)
-                             : launch_cfg<256, 1, 1, false, true, 1, 2>(a, grid, stream);
+    return p.head_dim <= 128 ? launch_two_pass<128, 2, 2, true>(kv_elem, a, grid, stream)
+                             : launch_two_pass<256, 1, 1, true>(kv_elem, a, grid, stream);
   }
   const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side || (small_batch && tune().no_wave_only == 0);
   if (wave_only) {
