@@ -374,7 +374,9 @@ def test_e4m3_random_batches(seed):
             bound = np.maximum(2e-2, 2 * step) + 1.01 * slack[:rows, :, None] + step * (slack[:rows, :, None] > 0)
             assert np.isfinite(got).all() and (d <= bound).all(), f"{what}: max-abs {d.max():.4g}, over the bound {(d > bound).sum()}"
             assert d[slack[:rows] == 0].mean() <= 2e-3 if (slack[:rows] == 0).any() else True
-            assert (slack[:rows] > 0).mean() <= 0.05, f"{what}: {(slack[:rows] > 0).mean():.3f} of the rows carry an allowance"
+            # one (token, head) row in twenty at most -- two rows in batches of a few dozen, where one row is already more
+            n_allowed = max(2, int(np.ceil(0.05 * slack[:rows].size)))
+            assert (slack[:rows] > 0).sum() <= n_allowed, f"{what}: {(slack[:rows] > 0).sum()} of {slack[:rows].size} rows carry an allowance"
 
 
 @pytest.mark.parametrize("name,n_sample,f8", [("decode_llama3_8b", 10, torch.float8_e4m3fn),
