@@ -38,7 +38,12 @@ def measured_traffic_bytes(workload: str):
 # two other bandwidth-bound streams come first: how fast a stream runs depends by a few per cent on the memory its pool
 # gets, and pools allocated early in a process get what a process of their own would (gemma2_local 0.386 ms as the
 # second workload of a process, 0.392-0.398 ms as the fifth; 0.380 ms alone).
-EXTRA_CONFIGS = ["gemma2_local", "decode_long_context", "decode_small", "mixed_prefill_decode", "mixed_prefill_only"]
+EXTRA_CONFIGS = ["gemma2_local", "decode_long_context", "decode_small", "mixed_prefill_decode", "mixed_prefill_only",
+                 "prefill_single_16k"]
+# Prompts too long for the CPU restatement: checked on a prefix against it and on sampled rows against float64
+# (long_prompt_parity).  prefill_single_16k is not one of the five benchmark configurations: it shows the prefill tile
+# where a tile walks up to 16384 keys and what a tile costs besides its key loop no longer counts.
+LONG_PROMPT_CONFIGS = ("prefill_single_16k", "prefill_long")
 
 
 def parse():
@@ -155,6 +160,79 @@ def cpu_sample_and_parity(batch, out, want_baseline, want_parity, n_seqs, budget
                       f"bf16 rounding points), OpenMP over {threads} threads",
         }
     return res
+
+
+def long_prompt_parity(batch, out, prefix_tokens=768, sampled_tokens=48):
+    """Parity for a workload of few, very long prompts, which the CPU restatement cannot walk in seconds.  Causal
+    attention makes the first `prefix_tokens` rows of a prompt the attention of that prefix alone: those rows are checked
+    against the restatement of the reference program on the prefix as a prompt of its own (the parity bound, widened to
+    two bf16 steps of the value where that is larger).  Rows deep
+    in the prompt are checked, `sampled_tokens` positions per prompt, against a float64 evaluation on the device (plain
+    torch: gather the prompt's K / V rows, scores, softmax, product) with the bound the tests use against float64."""
+    import numpy as np
+    import torch
+
+    from ejkernel_amd.workloads import Batch
+    from oracle import rpa_oracle_c
+    from tests.helpers import err_stats, oracle_args, to_np
+
+    m = batch.meta
+    G = m["num_q_heads"] // m["num_kv_heads"]
+    page = m["page_size"]
+    cu = batch.query_start_loc.cpu().numpy()
+    worst = {"prefix_max_abs": 0.0, "prefix_mean_abs": 0.0, "deep_max_abs": 0.0, "deep_mean_abs": 0.0}
+    rows_prefix = rows_deep = over_bound = 0
+    rng = np.random.default_rng(0)
+    for s in range(len(batch.q_lens)):
+        L, q0 = int(batch.kv_lens[s]), int(cu[s])
+        if int(batch.q_lens[s]) != L:
+            raise ValueError("long_prompt_parity takes prompts from scratch")
+        n0 = min(prefix_tokens, L)
+        n_pg = -(-n0 // page)
+        phys = batch.block_tables[s, :n_pg].long()
+        t_alloc = ((n0 + 7) // 8) * 8 + 8
+        q = torch.zeros((t_alloc,) + tuple(batch.queries.shape[1:]), dtype=batch.queries.dtype)
+        q[:n0] = batch.queries[q0:q0 + n0].cpu()
+        sub = Batch(queries=q, kv_pages=batch.kv_pages[phys].cpu(), context_lens=torch.tensor([n0], dtype=torch.int32),
+                    block_tables=torch.arange(n_pg, dtype=torch.int32)[None], query_start_loc=torch.tensor([0, n0], dtype=torch.int32),
+                    num_seqs=torch.tensor([1], dtype=torch.int32), softmax_scale=batch.softmax_scale,
+                    sliding_window=batch.sliding_window, logits_soft_cap=batch.logits_soft_cap, q_lens=np.array([n0]),
+                    kv_lens=np.array([n0]), name=batch.name + "/prefix", meta=dict(m))
+        ref = rpa_oracle_c.rpa_strict_c(*oracle_args(sub), softmax_scale=sub.softmax_scale, logits_soft_cap=sub.logits_soft_cap,
+                                        sliding_window=sub.sliding_window, io_dtype="bfloat16", threads=rpa_oracle_c.max_threads())
+        got = to_np(out[q0:q0 + n0])
+        mx, mean = err_stats(got, ref, n0)
+        worst["prefix_max_abs"], worst["prefix_mean_abs"] = max(worst["prefix_max_abs"], mx), max(worst["prefix_mean_abs"], mean)
+        # The first rows of a prompt see one or two keys and return values of magnitude 2..8, whose bf16 step is
+        # 0.016..0.031: the bound is the parity bound or two bf16 steps of the value, whichever is larger (the bound of
+        # tests.helpers.assert_bf16_parity_stepwise, which the prefill tiles are held to in the tests).
+        ref64 = np.asarray(ref[:n0], np.float64)
+        step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref64), 1e-30))) - 7)
+        over_bound += int((np.abs(np.asarray(got[:n0], np.float64) - ref64) > np.maximum(2e-2, 2 * step)).sum())
+        rows_prefix += n0
+        # rows deep in the prompt, in float64 on the device
+        pages = batch.kv_pages[batch.block_tables[s, : -(-L // page)].long()]          # [pages, page, 2 Hkv, D]
+        kv = pages.reshape(-1, 2 * m["num_kv_heads"], m["head_dim"])[:L].double()
+        k, v = kv[:, 0::2], kv[:, 1::2]                                                 # [L, Hkv, D]
+        pos = np.unique(np.concatenate([rng.integers(n0, L, size=sampled_tokens - 1), [L - 1]])) if L > n0 else np.array([L - 1])
+        for t in pos:
+            qt = batch.queries[q0 + int(t)].double().reshape(m["num_kv_heads"], G, m["head_dim"])
+            sc = torch.einsum("hgd,khd->hgk", qt, k[: int(t) + 1]) * batch.softmax_scale
+            if batch.logits_soft_cap:
+                sc = batch.logits_soft_cap * torch.tanh(sc / batch.logits_soft_cap)
+            if batch.sliding_window:
+                sc[..., : max(0, int(t) + 1 - batch.sliding_window)] = -float("inf")
+            ref_t = torch.einsum("hgk,khd->hgd", torch.softmax(sc, dim=-1), v[: int(t) + 1]).reshape(m["num_q_heads"], m["head_dim"])
+            d = (out[q0 + int(t)].double() - ref_t).abs()
+            worst["deep_max_abs"] = max(worst["deep_max_abs"], float(d.max()))
+            worst["deep_mean_abs"] += float(d.mean())
+            rows_deep += 1
+        del pages, kv, k, v
+    worst["deep_mean_abs"] /= max(rows_deep, 1)
+    worst.update({"rows_prefix": rows_prefix, "rows_deep": rows_deep, "prefix_elements_over_bound": over_bound,
+                  "ok": bool(over_bound == 0 and worst["prefix_mean_abs"] <= 2e-3 and
+                             worst["deep_max_abs"] <= 4e-2 and worst["deep_mean_abs"] <= 2e-3)})
+    return worst
 
 
 def cpu_sample_and_parity_v3(batch, v3, out, want_baseline, want_parity, n_seqs, budget_s=12.0):
@@ -537,7 +615,10 @@ def measure_config(name, steps, warmup, want_parity):
         torch.cuda.synchronize()
         entry["graph_replay_ms"] = (time.perf_counter() - t0) * 1e3 / reps
     if want_parity:
-        entry["parity"] = cpu_sample_and_parity(batch, out, False, True, 0, budget_s=2.0)["parity"]
+        if name in LONG_PROMPT_CONFIGS:
+            entry["parity"] = long_prompt_parity(batch, out)
+        else:
+            entry["parity"] = cpu_sample_and_parity(batch, out, False, True, 0, budget_s=2.0)["parity"]
     del batch, out
     torch.cuda.empty_cache()
     return entry
@@ -629,7 +710,10 @@ def main():
         "roofline": roof,
     }
     if not (args.no_cpu_baseline and args.no_parity):
-        if v3 is None:
+        if v3 is None and args.workload in LONG_PROMPT_CONFIGS and args.scale == 1.0:
+            if not args.no_parity:
+                line["parity"] = long_prompt_parity(batch, out)
+        elif v3 is None:
             line.update(cpu_sample_and_parity(batch, out, not args.no_cpu_baseline, not args.no_parity, args.cpu_seqs))
         else:
             # Repeating the call rewrites the same rows with the same values, so the cache after the timed steps is the

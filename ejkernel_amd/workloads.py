@@ -345,6 +345,8 @@ WORKLOADS = {
     # decode_llama3_8b and a mixed batch, 16 chunks x 256 tokens beside 112 decode sequences
     "decode_head_dim_96": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=96, page 16",
     "mixed_head_dim_96": "16 chunks x 256 tokens (prior 0..2048) + 112 decode seqs (kv 256..4096), 32q/8kv heads, D=96, page 32",
+    # one long prompt: 512 prefill tiles of 256 rows that walk up to 16384 keys each (per-tile costs vanish)
+    "prefill_single_16k": "1 prompt x 16384 tokens from scratch, 32q/8kv heads, D=128, page 32",
 }
 
 
@@ -393,6 +395,10 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
     if name == "prefill_long":
         L = n(8192)
         return make_batch(np.full(2, L), np.full(2, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
+                          pages_per_seq=pages(L, 32), seed=seed, device=device, dtype=dtype, name=name)
+    if name == "prefill_single_16k":
+        L = n(16384)
+        return make_batch(np.full(1, L), np.full(1, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
                           pages_per_seq=pages(L, 32), seed=seed, device=device, dtype=dtype, name=name)
     if name == "prefill_head_dim_64":
         S, chunk, prior = n(32), n(512), n(2048)

@@ -8,6 +8,7 @@ import inspect
 import re
 from pathlib import Path
 
+import numpy as np
 import pytest
 import torch
 
@@ -281,6 +282,25 @@ def test_mfma_mix_probe_library_is_built_and_exports_its_entry_points():
     assert lib.mfma_mix_probe_src_bytes() == (2048 + 2048) * 16
     assert hasattr(lib, "mfma_mix_probe_launch")
     assert not hasattr(_native.load(), "mfma_mix_probe_launch")
+
+
+def test_bench_long_prompt_parity_leg_detects_damage():
+    """bench.py checks prompts too long for the restatement on a prefix (against it) and on sampled deep rows (float64):
+    the float64 result passes, a damaged prefix row and a damaged sampled row (the last one is always sampled) fail."""
+    import bench
+    from ejkernel_amd.workloads import make_workload
+    from tests.helpers import run_exact
+
+    b = make_workload("prefill_single_16k", device="cpu", scale=0.03)
+    L = int(b.q_lens[0])
+    out = torch.from_numpy(np.asarray(run_exact(b), np.float32)).to(torch.bfloat16)
+    r = bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)
+    assert r["ok"] and r["rows_prefix"] == 100 and 1 <= r["rows_deep"] <= 6
+    out[L - 1] += 0.25
+    assert not bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)["ok"]
+    out[L - 1] -= 0.25
+    out[7] += 0.5
+    assert not bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)["ok"]
 
 
 def test_bench_power_sensor_and_gpu_count_guard():
