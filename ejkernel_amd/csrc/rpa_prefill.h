@@ -14,7 +14,7 @@
 // tile, so the online softmax is lane-local as in the decode loop.  The row sums come from one
 // extra MFMA against a vector of ones (they add exactly the bf16 probabilities that enter P V).
 // Logits are rounded to bf16 where the reference rounds them (kMimic; _xla_impl_fwd.py:119-124), as in the decode
-// loop -- except at head_dim 64, see below; the arithmetic of ragged_page_attention_v3 keeps them in fp32.  The K operands of a half are requested one
+// loop; the arithmetic of ragged_page_attention_v3 keeps them in fp32.  The K operands of a half are requested one
 // half ahead and the barrier that publishes the next tile sits before the last P V of a tile, so
 // LDS latency and barrier skew hide behind matrix work.  Halves of a step that lie entirely in a
 // wavefront's causal future, left of its window or before the sequence's first visible key are
@@ -24,7 +24,7 @@
 #include "rpa_tile_common.h"
 
 #ifndef RPA_ROUND_MIN_D
-#define RPA_ROUND_MIN_D 128  // smallest head_dim whose prefill tiles round their logits to bf16 (see the key loop)
+#define RPA_ROUND_MIN_D 64  // smallest head_dim whose prefill tiles round their logits to bf16: all of them (see the key loop)
 #endif
 
 namespace rpa {
@@ -477,8 +477,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
               }
           }
           else if (kMimic && D >= RPA_ROUND_MIN_D) {
-            // the reference's logits are bf16 (_xla_impl_fwd.py:119-124): round them, two per conversion (head_dim 64
-            // keeps fp32 logits: its tiles are bound by vector instructions and the rounding costs them a fifth)
+            // the reference's logits are bf16 (_xla_impl_fwd.py:119-124): round them, two per conversion (at head_dim 64,
+            // whose tiles are bound by vector instructions, that is 13 % of the time; a build with -DRPA_ROUND_MIN_D=128
+            // keeps fp32 logits there and lands up to three bf16 steps from the reference on rows of a few keys)
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll

@@ -217,7 +217,7 @@ def test_bf16_head_dim_64_prefill_tiles(page, hq, hkv, window, sinks):
     strict, exact = run_strict(b, softmax_aux=aux_np)[:rows], run_exact(b, softmax_aux=aux_np)[:rows]
     finite = np.isfinite(strict).all(axis=(1, 2))  # short pages: the restatement's first KV block under a window is NaN
     assert finite.mean() > 0.5
-    assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], what, exact=exact[finite])
+    assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], what)
     mx, mean = err_stats(out, exact, rows)
     assert mx <= 4e-2 and mean <= 2e-3, f"{what}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
 
@@ -354,21 +354,18 @@ def test_bf16_random_batches(seed):
         assert not out[rows:].any()
 
 
-@pytest.mark.parametrize("seed", [8038, 5162])
-def test_head_dim_64_prefill_tiles_on_seeds_where_fp32_logits_show(seed):
-    """Seeds found by sweeping new ones: at head_dim 64 the forced prefill tiles (fp32 logits) land up to three bf16 steps
-    from the restatement on a row that sees a handful of keys (seed 8038: 0.0234) -- and on the bf16 value next to the
-    float64 one, nearer to it than the restatement is.  That is the one allowance in these tests, and it holds here;
-    the library's own choice for such small batches (the wave-level loop, which rounds as the reference does) stays
-    inside the plain bound."""
+@pytest.mark.parametrize("seed", [8028, 8038, 9067])
+def test_head_dim_64_prefill_tiles_on_seeds_that_once_showed_fp32_logits(seed):
+    """Seeds found by sweeping new ones while the head_dim-64 prefill tiles kept fp32 logits: a row that sees a handful of
+    keys then landed three bf16 steps from the restatement (0.0234).  The tiles round their logits where the reference
+    does now, and the plain bound holds on the forced tiles as on the library's own choice."""
     b, what = random_rpa_batch(seed, DEV, head_dims=(64,))
     rows = b.total_valid_tokens
-    strict, exact = run_strict(b)[:rows], run_exact(b)[:rows]
+    strict = run_strict(b)[:rows]
     finite = np.isfinite(strict).all(axis=(1, 2))
-    out = to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES))
-    assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} tiles", exact=exact[finite])
-    out = to_np(run_hip(b, 0))
-    assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} default path")
+    for flags in (_native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES, 0):
+        out = to_np(run_hip(b, flags))
+        assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], f"{what} flags={flags}")
 
 
 @pytest.mark.parametrize("seed", range(3000, 3040))
