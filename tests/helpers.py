@@ -65,17 +65,25 @@ def assert_bf16_parity(out, ref, rows, what=""):
     return mx, mean
 
 
-def assert_bf16_parity_stepwise(out, ref, what=""):
+def assert_bf16_parity_stepwise(out, ref, what="", exact=None):
     """The parity bound, widened to two bf16 steps of the value where that is larger: rows that see one or two keys
     return values of magnitude 2..8, whose step is 0.016..0.031, and the reference's chain of bf16 roundings puts its
     restatement up to 1.5 steps from the float64 value there.  Every path rounds where the reference does and is held to
-    this bound as it stands."""
+    this bound as it stands.
+
+    `exact` (the float64 evaluation) is given only for a reference program that normalises the probabilities before
+    the product with V (`ragged_decode_attention`: e / l, the product, l times it and the division are four bf16
+    roundings after the exponential, where a one-pass kernel divides once in fp32): there an element may sit three steps
+    from the restatement if it is at least as close to the float64 value as the restatement is."""
     ref = np.asarray(ref, np.float64)
     out64 = np.asarray(out, np.float64)
     d = np.abs(out64 - ref)
     step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref), 1e-30))) - 7)
     assert np.isfinite(np.asarray(out)).all(), f"{what}: non-finite output"
     over = d > np.maximum(BF16_MAX_ABS, 2 * step)
+    if exact is not None and over.any():
+        ex = np.asarray(exact, np.float64)
+        over &= ~((d <= np.maximum(BF16_MAX_ABS, 3 * step) + 1e-12) & (np.abs(out64 - ex) <= np.abs(ref - ex)))
     assert not over.any() and d.mean() <= BF16_MEAN_ABS, f"{what}: max-abs {d.max():.4g} mean-abs {d.mean():.4g}"
 
 

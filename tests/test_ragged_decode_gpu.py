@@ -257,7 +257,7 @@ def test_full_size_workload(name, n_sample):
     assert_bf16_parity(to_np(out[ids.to(DEV)]), ref, len(ids), name)
 
 
-@pytest.mark.parametrize("seed", range(300, 340))
+@pytest.mark.parametrize("seed", [*range(300, 340), 11103, 11155, 20206, 20234])
 def test_bf16_random_batches(seed):
     """Seeded random shapes, starts, ends, windows, caps and sinks on both paths: within the parity bound of the
     reference program's restatement with one KV block per sequence on the rows it keeps finite, and within 4e-2 / 2e-3 of
@@ -293,6 +293,6 @@ def test_bf16_random_batches(seed):
                                             **kw))
         assert np.isfinite(out).all(), what
         if finite.any():
-            assert_bf16_parity_stepwise(out[finite], strict[finite], f"{what} flags={flags}")
+            assert_bf16_parity_stepwise(out[finite], strict[finite], f"{what} flags={flags}", exact=exact[finite])
         mx, mean = err_stats(out, exact, n)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
