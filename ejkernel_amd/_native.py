@@ -21,6 +21,7 @@ RPA_FLAG_FP32_LOGITS = 2
 RPA_FLAG_PREFILL_TILES = 4
 RPA_FLAG_PIPE_TILES = 8
 RPA_FLAG_PLAIN_TILES = 16
+RPA_FLAG_NO_LOGIT_STASH = 32
 
 EXPORTED_SYMBOLS = (
     "rpa_abi_version",

@@ -382,7 +382,8 @@ uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims) {
   const uint64_t base = rpa_workspace_bytes(&dims->attn);
   if (base == 0 || (dims->cache_dtype != RPA_DTYPE_FP8_E4M3 && dims->cache_dtype != RPA_DTYPE_FP8_E5M2)) return base;
   const uint64_t rows = static_cast<uint64_t>(dims->attn.total_tokens > 0 ? dims->attn.total_tokens : 0) * dims->attn.num_q_heads;
-  return ((base + 255) & ~255ull) + ((rows * 8 + 255) & ~255ull);
+  // behind the kernels' part: the row statistics, then the logits kept between the two launches (if any)
+  return ((base + 255) & ~255ull) + ((rows * 8 + 255) & ~255ull) + ((rpa::logit_stash_bytes(dims->attn) + 255) & ~255ull);
 }
 
 int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
@@ -450,9 +451,11 @@ int rpa_v3_launch(const RpaV3Params* params, void* hip_stream) {
   if (!fp8) return rpa::dispatch(p, kv, rpa::tiled_supported(p), stream);
   const uint64_t base = (rpa_workspace_bytes(&p) + 255) & ~255ull;
   float* stats = reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base);
+  const uint64_t stats_bytes = (static_cast<uint64_t>(p.total_tokens > 0 ? p.total_tokens : 0) * p.num_q_heads * 8 + 255) & ~255ull;
+  float* logits = rpa::logit_stash_bytes(p) != 0 ? reinterpret_cast<float*>(static_cast<char*>(p.workspace) + base + stats_bytes) : nullptr;
   RpaParams q = p;
   q.workspace_bytes = base;
-  rc = rpa::launch_tiled_fp8(q, kv, v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 2 : 1, stats, stream);
+  rc = rpa::launch_tiled_fp8(q, kv, v.cache_dtype == RPA_DTYPE_FP8_E5M2 ? 2 : 1, stats, logits, stream);
   if (rc != RPA_OK) return rpa::fail(rc, "kernel launch failed: %s", hipGetErrorString(hipGetLastError()));
   return RPA_OK;
 }

@@ -76,6 +76,10 @@ constexpr float fp8_max() { return kKv == 2 ? 57344.f : 448.f; }
 // probabilities to the cache dtype (ragged_page_attention_v3, _kernel.py:279), which needs the row maximum and sum
 // before the first P V product, so it runs as two launches: 1 = row statistics only (maximum and sum of exp over
 // the visible keys, written to TileArgs::stats), 2 = P = round(exp(s - m) / l) with m, l from there, O = P V.
+// Where TileArgs::logits is given, launch 1 also leaves every logit it computed there (capped and masked, fp32, one
+// row of logit_pitch keys per (token, query head)) and the second launch is 3 instead of 2: the same arithmetic on the
+// stored logits, with no K rows read, no Q and no first product -- for a decode step that is 8 bytes of logits written
+// and read per key and query head against a K row of head_dim bytes per key and kv head.
 template <int D, int NT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
                                              int j, int rt, int range_lo, int range_hi, const Part& part) {
@@ -147,7 +151,16 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     for (int c = 0; c < 8; ++c) o_acc[sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   float m_run = -INFINITY, l_run = 0.f;
   float m_fix = 0.f, inv_l = 0.f;  // kPass == 2: the row's maximum and 1 / sum from the statistics launch
-  if constexpr (kPass == 2) {
+  constexpr bool kNorm = kPass >= 2;    // probabilities normalised with the statistics of an earlier launch
+  constexpr bool kStored = kPass == 3;  // ... and the logits of that launch instead of K
+  // This lane's stored logits (an absent row repeats the item's first one: read, never written).  A (token, kv head)
+  // owns logit_pitch * G floats, laid out [key / 4][query head of the kv head][key % 4]: the 32 keys of a tile and
+  // the G rows of a decode token are one contiguous run of 128 G bytes.
+  float* lrow = nullptr;
+  if constexpr (kPass == 1 || kStored)
+    if (a.logits != nullptr)
+      lrow = a.logits + (static_cast<size_t>(si.q0 + qi) * p.num_kv_heads + j) * static_cast<size_t>(a.logit_pitch) * G + 4 * hg;
+  if constexpr (kNorm) {
     const size_t idx = static_cast<size_t>(si.q0 + qi) * p.num_q_heads + head;
     const float ms = a.stats[2 * idx], ls = a.stats[2 * idx + 1];
     m_fix = ms == -INFINITY ? 0.f : ms;
@@ -169,6 +182,10 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   constexpr uint32_t PIECE_B = kKv != 0 ? 8u : 16u;
   raw_t kreg[C::NSLOT][C::NS];
   raw_t vbuf0[C::NSLOT][C::NS], vbuf1[C::NSLOT][C::NS];
+  f32x4_t sreg[NT];  // kStored: this lane's four logits per sub-tile, requested with the V rows
+  // tiles never reach past the pitch (a multiple of 64 that covers every position a block-table row can hold); the
+  // clamp only keeps a lane in its row should the metadata be malformed
+  auto logit_off = [&](int tile, int u) { return min(tile + 16 * u + 4 * g, static_cast<int>(a.logit_pitch) - 4); };
 
   // Fetch K and V of the TT tokens starting at `tile`: lane (i, g) takes tokens 16u + 4g + r (u < NT, r < 4),
   // 16-byte piece i (+16 per 128-slice) of each row, so a quarter-wave reads one contiguous row.
@@ -196,6 +213,11 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   const uint32_t piece_off = head_off + PIECE_B * static_cast<uint32_t>(piece) + (pair && i >= 8 ? a.kv.head_b : 0u);
   const uint32_t lane_off = static_cast<uint32_t>(4 * g) * stride_b + piece_off;
   auto issue_loads = [&](int tile, raw_t (&kr)[C::NSLOT][C::NS], raw_t (&vr)[C::NSLOT][C::NS]) {
+    if constexpr (kStored) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+        sreg[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_t*>(lrow + static_cast<size_t>(logit_off(tile, u)) * G));
+    }
     if (a.uniform_page && tile + C::TT <= range_hi) {
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
@@ -215,7 +237,8 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           const char* row = sbase + static_cast<uint64_t>(r) * stride_b;
           const char* row_v = row + v_delta;
 #pragma unroll
-          for (int sN = 0; sN < C::NS; ++sN) kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + (lane_off + slice_off[sN]));
+          for (int sN = 0; sN < C::NS; ++sN)
+            if (!kStored) kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + (lane_off + slice_off[sN]));
           if constexpr (C::NS > 1) asm volatile("" ::: "memory");
 #pragma unroll
           for (int sN = 0; sN < C::NS; ++sN)
@@ -238,30 +261,57 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
         const char* row = base + static_cast<uint64_t>(min(r, rlim)) * stride_b;
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
-          kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + slice_off[sN]);
+          if (!kStored) kr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + slice_off[sN]);
           if (kPass != 1) vr[4 * u + r][sN] = *reinterpret_cast<const raw_t*>(row + v_delta + slice_off[sN]);
         }
       }
     }
   };
 
+  f32x4_t skeep[NT];    // kPass 1 with stored logits: the last tile's logits, not yet stored
+  int skeep_tile = -1;
+  auto store_logits = [&]() {
+    if (skeep_tile < 0) return;
+    if (row_valid && skeep_tile + C::TT <= static_cast<int>(a.logit_pitch)) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u)
+        __builtin_nontemporal_store(skeep[u], reinterpret_cast<f32x4_t*>(lrow + static_cast<size_t>(skeep_tile + 16 * u + 4 * g) * G));
+    }
+    skeep_tile = -1;
+  };
   auto body = [&](int tile, raw_t (&vcur)[C::NSLOT][C::NS], raw_t (&vnext)[C::NSLOT][C::NS]) {
+    f32x4_t s_acc[NT];
+    if constexpr (kStored) {
+#pragma unroll
+      for (int u = 0; u < NT; ++u) s_acc[u] = sreg[u];
+    }
     // 1. K rows to the wave-private LDS tile: row = token within the tile, 16-byte piece i (+16 per slice)
+    if constexpr (!kStored)
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN) {
+          // the statistics launch fetches no V: its K rows alternate between the two V buffers, two tiles ahead
+          const raw_t kraw = kPass == 1 ? vcur[4 * u + r][sN] : kreg[4 * u + r][sN];
           u32x4_t kw;
-          if constexpr (kKv != 0) kw = fp8x8_to_bf16x8<kKv>(kreg[4 * u + r][sN]);
-          else kw = kreg[4 * u + r][sN];
+          if constexpr (kKv != 0) kw = fp8x8_to_bf16x8<kKv>(kraw);
+          else kw = kraw;
           *reinterpret_cast<u32x4_t*>(lds_k + (16 * u + 4 * g + r) * C::ROWB + 16 * (i + 16 * sN)) = kw;
         }
+    // The logits of the tile before go out ahead of this iteration's loads: the wait for those loads at the top of the
+    // next iteration then finds the stores a whole iteration old (stores and loads leave one counter in order; issued
+    // after the loads, a store would be waited for when it has only just left).
+    if constexpr (kPass == 1) store_logits();
     // 2. next tile's K and V are requested now, a full iteration before they are needed
-    if (tile + C::TT < range_hi) issue_loads(tile + C::TT, kreg, vnext);
+    if constexpr (kPass == 1) {
+      if (tile + 2 * C::TT < range_hi) issue_loads(tile + 2 * C::TT, vcur, vnext);
+    } else {
+      if (tile + C::TT < range_hi) issue_loads(tile + C::TT, kreg, vnext);
+    }
     // 3. S^T = K Q^T: lane (token i of sub-tile u, group g) reads piece 4 ks + g of its row
-    f32x4_t s_acc[NT];
+    if constexpr (!kStored)
 #pragma unroll
     for (int u = 0; u < NT; ++u) {
       s_acc[u] = f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -278,15 +328,15 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
 #pragma unroll
     for (int u = 0; u < NT; ++u)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) sv[u][r] = kMimic ? rbf(s_acc[u][r]) : s_acc[u][r] * post_scale;
-    if (cap != 0.f) {
+      for (int r = 0; r < 4; ++r) sv[u][r] = kStored ? s_acc[u][r] : kMimic ? rbf(s_acc[u][r]) : s_acc[u][r] * post_scale;
+    if (!kStored && cap != 0.f) {
       asm volatile("" : "+v"(sv[0][0]));  // keeps the soft cap inside this wave-uniform branch (it is not cheap)
 #pragma unroll
       for (int u = 0; u < NT; ++u)
 #pragma unroll
         for (int r = 0; r < 4; r += 2) soft_cap2<kMimic>(sv[u][r], sv[u][r + 1], cap, inv_cap);
     }
-    if (need_mask) {
+    if (!kStored && need_mask) {
 #pragma unroll
       for (int u = 0; u < NT; ++u)
 #pragma unroll
@@ -296,8 +346,16 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           sv[u][r] = keep ? sv[u][r] : -INFINITY;
         }
     }
+    if constexpr (kPass == 1) {
+      // the logits as the next launch needs them, capped and masked; stored by the next iteration
+      if (a.logits != nullptr) {
+#pragma unroll
+        for (int u = 0; u < NT; ++u) skeep[u] = f32x4_t{sv[u][0], sv[u][1], sv[u][2], sv[u][3]};
+        skeep_tile = tile;
+      }
+    }
     uint32_t pw[2 * NT];
-    if constexpr (kPass == 2) {
+    if constexpr (kNorm) {
       // normalised probabilities, rounded to the cache dtype
 #pragma unroll
       for (int u = 0; u < NT; ++u) {
@@ -424,16 +482,22 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   }
 
   if (range_hi > range_lo) {
-    issue_loads(range_lo, kreg, vbuf0);
+    if constexpr (kPass == 1) {
+      issue_loads(range_lo, vbuf0, vbuf1);
+      if (range_lo + C::TT < range_hi) issue_loads(range_lo + C::TT, vbuf1, vbuf0);
+    } else {
+      issue_loads(range_lo, kreg, vbuf0);
+    }
     for (int tile = range_lo; tile < range_hi; tile += 2 * C::TT) {
       body(tile, vbuf0, vbuf1);
       if (tile + C::TT >= range_hi) break;
       body(tile + C::TT, vbuf1, vbuf0);
     }
+    if constexpr (kPass == 1) store_logits();
   }
 
   // ---- row sum across the four lane groups
-  if constexpr (kPass != 2) l_run = row_groups_sum(l_run);
+  if constexpr (!kNorm) l_run = row_groups_sum(l_run);
 
   if constexpr (kWaveOnly && kPass == 0 && kKv == 0) {
     if (sink_part) {
@@ -765,7 +829,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     num_scale = m_run == -INFINITY ? 0.f : expf(m_run - mt);
     denom = num_scale * l_run + ssum;
   }
-  const float inv = kPass == 2 ? out_scale(p) : num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
+  const float inv = kNorm ? out_scale(p) : num_scale * out_scale(p) / fmaxf(denom, 1e-6f);
   bf16_t* orow = out + q_row_off;
 #pragma unroll
   for (int sN = 0; sN < C::NS; ++sN)

@@ -95,7 +95,11 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl);
 int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre = PreState());
 // The same for an 8-bit cache described by `kv` (kv_elem 1 = e4m3, 2 = e5m2): two launches, row statistics into
 // `stats` [total_tokens, num_q_heads, 2] and then the attention (RPA_FLAG_FP32_LOGITS arithmetic, no sinks).
-int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, hipStream_t stream);
+// `logits` (null, or logit_stash_bytes(p) bytes): where the statistics launch leaves its logits for the second launch.
+int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, float* logits, hipStream_t stream);
+// Bytes of fp32 logits a two-launch call on an 8-bit cache keeps between its launches, 0 where it does not (batches
+// that run on prefill tiles, or more than kLogitStashMaxBytes).
+uint64_t logit_stash_bytes(const RpaParams& p);
 
 // Compute units of the current device (cached per device).
 int device_cu_count();

@@ -447,6 +447,7 @@ struct Tune {
   int pipe;                // RPA_TUNE_PIPE: 0 = never use the software-pipelined prefill tile (head_dim 128)
   int pipe_stream_wgs;     // RPA_TUNE_PIPE_STREAM_WGS: workgroups (of one per compute unit) that take the decode stream first
   int pipe_min_tokens_per_seq;  // RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ: average query tokens per sequence from which it is used
+  int no_logit_stash;      // RPA_TUNE_NO_LOGIT_STASH: two-launch calls read K in both launches (experiments)
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -468,6 +469,7 @@ static const Tune& tune() {
     x.pipe = env_int("RPA_TUNE_PIPE", 1);
     x.pipe_min_tokens_per_seq = max(1, env_int("RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ", 128));
     x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
+    x.no_logit_stash = env_int("RPA_TUNE_NO_LOGIT_STASH", 0);
     return x;
   }();
   return t;
@@ -502,6 +504,31 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
 }
 
+// Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
+// of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
+// alone gets a register allocation without spills, and short prefill chunks spread over four times as many
+// wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
+static bool small_batch_of(const RpaParams& p) {
+  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
+  return p.query_start_loc == nullptr ||
+         ((p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) == 0 && rows <= tune().wave_only_rows);
+}
+
+constexpr uint64_t kLogitStashMaxBytes = 2ull << 30;
+static uint32_t logit_pitch_of(const RpaParams& p) {
+  const uint64_t cap = static_cast<uint64_t>(p.pages_per_seq > 0 ? p.pages_per_seq : 0) * static_cast<uint64_t>(p.page_size);
+  return static_cast<uint32_t>(std::min<uint64_t>((cap + 63) & ~63ull, 1u << 30));
+}
+uint64_t logit_stash_bytes(const RpaParams& p) {
+  // decided by the sizes alone: a size query may come before the pointers are set
+  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
+  if (tune().no_logit_stash != 0 || rows <= 0 || rows > tune().wave_only_rows ||
+      (p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES | RPA_FLAG_NO_LOGIT_STASH)) != 0)
+    return 0;
+  const uint64_t bytes = static_cast<uint64_t>(p.total_tokens) * p.num_q_heads * logit_pitch_of(p) * 4ull;
+  return bytes <= kLogitStashMaxBytes ? bytes : 0;
+}
+
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<(D < 128 ? 128 : D), NT, kMimic>;
@@ -529,14 +556,20 @@ static int launch_two_pass(int kv_elem, const TileArgs& a, int grid, hipStream_t
   int rc;
   if (kv_elem == 2) {
     rc = launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 1>(a, grid, stream);
-    return rc != RPA_OK ? rc : launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 2>(a, grid, stream);
+    if (rc != RPA_OK) return rc;
+    if constexpr (kWaveOnly)
+      if (a.logits != nullptr) return launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 3>(a, grid, stream);
+    return launch_cfg<D, NT, MRT, false, kWaveOnly, 2, 2>(a, grid, stream);
   }
   rc = launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 1>(a, grid, stream);
-  return rc != RPA_OK ? rc : launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 2>(a, grid, stream);
+  if (rc != RPA_OK) return rc;
+  if constexpr (kWaveOnly)
+    if (a.logits != nullptr) return launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 3>(a, grid, stream);
+  return launch_cfg<D, NT, MRT, false, kWaveOnly, 1, 2>(a, grid, stream);
 }
 
 static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre, float* stats,
-                             int kv_elem = 0) {
+                             int kv_elem = 0, float* logits = nullptr) {
   WorkspaceLayout wl;
   tiled_workspace_layout(p, &wl);
   if (p.workspace == nullptr || p.workspace_bytes < wl.total_bytes) return RPA_ERR_WORKSPACE;
@@ -545,6 +578,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.kv = kv;
   a.pre = pre;
   a.stats = stats;
+  a.logits = nullptr;
+  a.logit_pitch = 0;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.min_share_tiles = tune().min_share_tiles;
   // a part costs about as much as streaming 128 keys: 4 tiles of 32 keys, 8 of 16 (head_dim 256)
@@ -565,13 +600,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.partial_ml = reinterpret_cast<float*>(ws + wl.partial_ml_off);
   const int grid = tiled_grid();
   const bool mimic = (p.flags & RPA_FLAG_FP32_LOGITS) == 0 && tune().no_mimic == 0;
-  // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
-  // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
-  // alone gets a register allocation without spills, and short prefill chunks spread over four times as many
-  // wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
-  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
-  const bool small_batch = p.query_start_loc == nullptr || ((p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) == 0 &&
-                                                            rows <= tune().wave_only_rows);
+  const bool small_batch = small_batch_of(p);
   // Prefill tiles address one paged cache with a token's K and V rows side by side, [page][slot][combined head][row]
   // (rows may be padded beyond head_dim and tokens beyond 2 * kv heads: the plain tile takes the pitches from the
   // layout; the pipelined tile's instruction stream has the unpadded ones built in); any other layout (two caches, one
@@ -595,6 +624,12 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
       return launch_two_pass<256, 1, 1, false>(kv_elem, a, grid, stream);
     }
     a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 2);
+    // The statistics launch leaves its logits for the second one, which then reads no K rows: per key, 4 bytes
+    // written and 4 read per query head against a K row of head_dim bytes per kv head.
+    if (logits != nullptr && logit_stash_bytes(p) != 0) {
+      a.logits = logits;
+      a.logit_pitch = logit_pitch_of(p);
+    }
     return p.head_dim <= 128 ? launch_two_pass<128, 2, 2, true>(kv_elem, a, grid, stream)
                              : launch_two_pass<256, 1, 1, true>(kv_elem, a, grid, stream);
   }
@@ -637,8 +672,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
 int launch_tiled(const RpaParams& p, const KvLayout& kv, hipStream_t stream, const PreState& pre) {
   return launch_tiled_impl(p, kv, stream, pre, nullptr);
 }
-int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, hipStream_t stream) {
-  return launch_tiled_impl(p, kv, stream, PreState(), stats, kv_elem);
+int launch_tiled_fp8(const RpaParams& p, const KvLayout& kv, int kv_elem, float* stats, float* logits, hipStream_t stream) {
+  return launch_tiled_impl(p, kv, stream, PreState(), stats, kv_elem, logits);
 }
 
 }  // namespace rpa

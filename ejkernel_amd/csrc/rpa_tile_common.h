@@ -34,6 +34,9 @@ struct TileArgs {
   float* partial_o;   // [2 * wavefronts of the grid][16][D]
   float* partial_ml;  // [2 * wavefronts of the grid][16][2]
   float* stats;       // row maximum and row sum per (token, query head) of a two-launch call (null otherwise)
+  float* logits;      // two-launch call: the first launch's logits, [token][kv head][logit_pitch / 4][query head of the
+                      // kv head][4] (null: K is read twice)
+  uint32_t logit_pitch;  // keys per (token, query head) of `logits`: a multiple of 64 that covers a block-table row
   PreState pre;       // state accumulated by an earlier kernel, merged by the wave-level loop (null: none)
   // head_dim 64, instantiation without prefill tiles: a wave-level item covers two kv heads (2 j, 2 j + 1) at once.
   // The 128-wide loop then reads, per token, [K of head 2j | K of head 2j+1] as one K row and the two V rows as one V

@@ -57,6 +57,11 @@ extern "C" {
                                   /* software-pipelined (by default chosen for batches of long chunks: at least 128    */
                                   /* query tokens per sequence on average); implies RPA_FLAG_PREFILL_TILES            */
 #define RPA_FLAG_PLAIN_TILES 16u  /* never those: prefill tiles of 128 rows, two workgroups per compute unit          */
+#define RPA_FLAG_NO_LOGIT_STASH 32u /* rpa_v3_launch with an 8-bit cache: both launches read K.  By default, batches  */
+                                  /* of up to 20480 (token, query head) rows keep the first launch's fp32 logits in   */
+                                  /* the workspace (4 bytes per row and position a block-table row can hold, 2 GiB   */
+                                  /* at most: rpa_v3_workspace_bytes counts them) and the second launch reads those   */
+                                  /* instead of K -- the same numbers, bit for bit                                    */
 
 typedef struct RpaParams {
   /* ---- device buffers (argument names follow ragged_page_attention.py:540-547).  queries, kv_pages and out are   */

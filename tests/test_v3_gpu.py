@@ -299,9 +299,11 @@ E4M3_CASES = dict(CASES)
 E4M3_CASES["long_decode"] = ([1, 1, 1, 1], [4000, 2500, 4096, 777], dict(pages_per_seq=256))
 
 
-# an 8-bit cache on the wave-level loop alone (what small batches get) and with prefill tiles forced (chunks of more
-# than 64 rows per kv head then run on the tiles, in both passes)
-F8_PATHS = [pytest.param(0, id="items"), pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles")]
+# an 8-bit cache on the wave-level loop alone (what small batches get: the second launch reads the first one's logits,
+# or K again where the caller asks for that) and with prefill tiles forced (chunks of more than 64 rows per kv head
+# then run on the tiles, in both passes)
+F8_PATHS = [pytest.param(0, id="items"), pytest.param(_native.RPA_FLAG_NO_LOGIT_STASH, id="items_k_twice"),
+            pytest.param(_native.RPA_FLAG_PREFILL_TILES, id="tiles")]
 
 
 @pytest.mark.parametrize("flags", F8_PATHS)
@@ -322,6 +324,21 @@ def test_e4m3_cache_parity_and_cache_update(case, scales, f8, flags):
         got, ref = got / 2.0, ref / 2.0          # v_scale doubles the outputs
     assert_bf16_parity(got, ref, rows, case)
     assert not out[rows:].any()
+
+
+@pytest.mark.parametrize("f8", BOTH_F8)
+@pytest.mark.parametrize("case", list(E4M3_CASES))
+def test_e4m3_second_launch_on_stored_logits_equals_the_one_that_reads_k_again(case, f8):
+    """Small batches keep the first launch's fp32 logits in the workspace and the second launch reads those instead
+    of K: the same arithmetic on the same numbers, so the output is that of the launch pair that reads K twice, bit for
+    bit (window, cap, scales, pages of 4 tokens, head_dim 256, chunks of several row tiles)."""
+    q_lens, kv_lens, kw = E4M3_CASES[case]
+    outs = []
+    for flags in (0, _native.RPA_FLAG_NO_LOGIT_STASH):
+        v = small_e4m3(q_lens, kv_lens, f8=f8, **kw)
+        out, _ = run_hip(v, flags, q_scale=0.05, k_scale=0.5, v_scale=2.0)
+        outs.append(out.clone())
+    assert torch.equal(outs[0], outs[1])
 
 
 def test_e4m3_probabilities_below_half_the_smallest_subnormal_vanish():
