@@ -76,6 +76,42 @@ def test_ragged_decode_sink_arguments_are_checked_before_any_launch():
     assert lib.rpa_ragged_decode_launch(ctypes.byref(p), None) == -3 and b"too small" in lib.rpa_last_error()
 
 
+def test_python_constants_are_the_header_s():
+    """Every RPA_* constant of the ctypes layer has the value the C header defines."""
+    import pathlib
+    import re
+    text = (pathlib.Path(__file__).resolve().parents[1] / "include" / "rpa_mi355x.h").read_text()
+    defines = {m.group(1): m.group(2) for m in re.finditer(r"^#define (RPA_[A-Z0-9_]+) \(?(-?\d+)u?\)?", text, re.M)}
+    names = [n for n in dir(_native) if n.startswith("RPA_") and isinstance(getattr(_native, n), int)]
+    assert len(names) >= 12
+    for n in names:
+        assert n in defines, f"{n} is not defined in the header"
+        assert int(defines[n]) == getattr(_native, n), n
+
+
+def test_v3_workspace_counts_the_stored_logits_of_an_8_bit_cache():
+    lib = _native.load()
+    v = _native.RpaV3Params()
+    p = v.attn
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = 16, 8, 2, 128
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = 16, 64, 16, 10   # a block-table row holds 160 positions
+    p.dtype, p.compute = _native.RPA_DTYPE_BF16, _native.RPA_COMPUTE_BF16
+    v.cache_dtype = _native.RPA_DTYPE_FP8_E4M3
+    with_logits = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    p.flags = _native.RPA_FLAG_NO_LOGIT_STASH
+    without = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    assert with_logits - without == 16 * 8 * 192 * 4          # fp32 per (token, query head) and position, pitch 192
+    p.flags = 0
+    p.total_tokens = 20480 // 8 + 1                            # batches that run on prefill tiles read K twice
+    grown = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    p.flags = _native.RPA_FLAG_NO_LOGIT_STASH
+    assert grown == lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    p.flags, p.total_tokens, p.pages_per_seq = 0, 2560, 1 << 16  # 2560 * 8 rows * 2**20 positions * 4 bytes: over the limit
+    big = lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+    p.flags = _native.RPA_FLAG_NO_LOGIT_STASH
+    assert big == lib.rpa_v3_workspace_bytes(ctypes.byref(v))
+
+
 def test_v3_cache_dtype_arguments_are_checked_before_any_launch():
     lib = _native.load()
     v = _native.RpaV3Params()
