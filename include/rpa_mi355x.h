@@ -133,8 +133,8 @@ typedef struct RpaV3Params {
                           /* bf16 queries.  An 8-bit cache follows the program's casts (_kernel.py:249-254, :279):  */
                           /* with q_scale, q / q_scale is rounded to the query dtype, clipped to the 8-bit type's   */
                           /* finite range (+-448 / +-57344) and cast to it; the normalised probabilities are cast   */
-                          /* to it before P V.  It runs as two passes over                                          */
-                          /* the keys (row maximum and sum, then the attention) on the MFMA kernel only, and needs  */
+                          /* to it before P V.  It runs as two launches (row                                        */
+                          /* maximum and sum, then the attention) on the MFMA kernel only, and needs                */
                           /* rpa_v3_workspace_bytes() of workspace.                                                 */
   int32_t cache_head_dim; /* elements per cache row: align_to(head_dim, 128) as merge_kv pads it (_kernel.py:44-57), or 0  */
                           /* for head_dim.  With padded rows (head_dim 64 in rows of 128) the cache is                 */
@@ -170,8 +170,8 @@ int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
 uint64_t rpa_static_scratch_bytes(void);
 int rpa_fwd_launch_static(const RpaParams* params, void* hip_stream);
 
-/* Bytes of workspace rpa_v3_launch needs (rpa_workspace_bytes() of `attn`, plus the row statistics of an 8-bit
- * cache). */
+/* Bytes of workspace rpa_v3_launch needs (rpa_workspace_bytes() of `attn`; with an 8-bit cache also the row
+ * statistics and, unless RPA_FLAG_NO_LOGIT_STASH is set, the logits kept between its two launches). */
 uint64_t rpa_v3_workspace_bytes(const RpaV3Params* dims);
 
 /* Enqueues the cache update (token t of sequence s goes to position kv_len - q_len + (t - q_start) of s) and then
