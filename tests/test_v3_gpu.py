@@ -341,6 +341,31 @@ def test_e4m3_second_launch_on_stored_logits_equals_the_one_that_reads_k_again(c
     assert torch.equal(outs[0], outs[1])
 
 
+def test_e4m3_launch_pair_recorded_in_a_hip_graph_replays_correctly():
+    """Cache update, statistics launch and attention on the stored logits only enqueue, so the call can be captured;
+    every replay on new queries equals the eager result bit for bit (the update rewrites the same rows)."""
+    q_lens, kv_lens, kw = E4M3_CASES["long_decode"]
+    v = small_e4m3(q_lens, kv_lens, **kw)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            ragged_page_attention_v3(*v.args(), **v.kwargs())
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g, _ = ragged_page_attention_v3(*v.args(), **v.kwargs())
+    gen = torch.Generator(device=DEV).manual_seed(7)
+    for rep in range(3):
+        v.queries.copy_(torch.randn(v.queries.shape, generator=gen, device=DEV).to(v.queries.dtype))
+        want, _ = ragged_page_attention_v3(*v.args(), **v.kwargs())
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, want), rep
+
+
 def test_e4m3_probabilities_below_half_the_smallest_subnormal_vanish():
     # q = 0 over 1024 keys: p = 2**-10 rounds to zero in e4m3, the row is zero; over 64 keys p = 2**-6 survives and
     # the row is the mean of V.  An implementation that rounds exp(s - max) instead of the normalised value fails this.
