@@ -79,10 +79,6 @@ def parse():
     ap.add_argument("--gemm-probe", type=int, default=0, metavar="N",
                     help="instead of the benchmark, time the vendor library's bf16 N x N x N matrix product (what the "
                          "matrix cores of this box sustain under its power limit; context for the MFMA-bound figures)")
-    ap.add_argument("--mfma-mix-probe", type=float, default=0.0, metavar="SECONDS",
-                    help="instead of the benchmark, run a register-resident loop of 32x32x16 bf16 MFMAs with and without "
-                         "a prefill tile's share of vector work and LDS reads back to back, SECONDS per mix: what the "
-                         "board's power limit lets that instruction mix sustain")
     return ap.parse_args()
 
 
@@ -532,45 +528,6 @@ def sustain(fn, seconds, what, flops=None, nbytes=None, quiet=False):
     return res
 
 
-# (vector elements, LDS operand reads) per block of 32 MFMAs that csrc/probe_mfma_mix.hip instantiates; an element is
-# 5.5 vector instructions, so 24 elements with 16 reads is about the mix of the pipelined prefill tile's key loop
-MFMA_MIXES = [(0, 0), (-16, 0), (0, 16), (24, 0), (24, 16), (48, 0), (48, 16), (64, 16)]  # -16: 64 MFMAs of 16x16x32 instead
-
-
-def mfma_mix_probe(seconds):
-    """What the board sustains, under its power limit, for a register-resident loop of v_mfma_f32_32x32x16_bf16 with
-    a prefill tile's share of softmax-like vector work and LDS operand reads, and for the MFMAs alone: one JSON line
-    with the rate and the power of each mix."""
-    import ctypes
-
-    import torch
-
-    from ejkernel_amd.build import PROBE_LIB_PATH
-
-    lib = ctypes.CDLL(str(PROBE_LIB_PATH))
-    lib.mfma_mix_probe_src_bytes.restype = ctypes.c_uint64
-    lib.mfma_mix_probe_launch.restype = ctypes.c_double
-    lib.mfma_mix_probe_launch.argtypes = [ctypes.c_int] * 4 + [ctypes.c_void_p] * 4
-    grid, iters = torch.cuda.get_device_properties(0).multi_processor_count, 1000
-    src = torch.randn(lib.mfma_mix_probe_src_bytes() // 2, device="cuda:0", dtype=torch.float32).to(torch.bfloat16)
-    dst = torch.empty(grid * 256, device="cuda:0", dtype=torch.float32)
-    clocks = torch.zeros(grid * 2, device="cuda:0", dtype=torch.int64)
-    stream = torch.cuda.current_stream().cuda_stream
-    out = []
-    for elems, reads in MFMA_MIXES:
-        flops = lib.mfma_mix_probe_launch(elems, reads, grid, iters, src.data_ptr(), dst.data_ptr(), clocks.data_ptr(), stream)
-        assert flops > 0, (elems, reads)
-        torch.cuda.synchronize()
-        r = sustain(lambda: lib.mfma_mix_probe_launch(elems, reads, grid, iters, src.data_ptr(), dst.data_ptr(), clocks.data_ptr(), stream),
-                    seconds, f"{elems} vector elements, {reads} LDS reads per 32 MFMAs", flops=flops, quiet=True)
-        c = clocks.view(grid, 2).double().cpu()  # the last launch: shader cycles and 100 MHz ticks per workgroup
-        out.append({"vector_elements": elems, "lds_reads": reads, "tflops": r["tflops"], "ms_per_launch": r["ms_per_launch"],
-                    "power_w_median": r["power_w_median"], "shader_clock_ghz": float((c[:, 0] / c[:, 1]).mean()) * 0.1,
-                    "cycles_per_32_mfma": float(c[:, 0].mean()) / iters})
-    print(json.dumps({"mfma_mix_probe": out, "seconds_each": seconds, "workgroups": grid, "unit": "TFLOP/s",
-                      "dtype": "bf16", "power_cap_w": board_power_watts()[1]}))
-
-
 def measure_config(name, steps, warmup, want_parity):
     """One entry of "configs": the named workload at full size, timed like the headline one and checked against the
     CPU restatement on a small sample of its sequences."""
@@ -642,8 +599,6 @@ def main():
     dev = "cuda:0"
     if args.op in ("page_attention", "ragged_decode"):
         return page_attention_main(args)
-    if args.mfma_mix_probe > 0:
-        return mfma_mix_probe(args.mfma_mix_probe)
     if args.gemm_probe and args.sustain > 0:
         n = args.gemm_probe
         ga = torch.randn(n, n, device=dev, dtype=torch.bfloat16)

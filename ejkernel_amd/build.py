@@ -21,11 +21,6 @@ LIB_PATH = LIB_DIR / "librpa_mi355x.so"
 OBJ_DIR = PKG_DIR / "build"
 
 SOURCES = ["rpa_api.hip", "rpa_generic.hip", "rpa_kv_update.hip", "rpa_sink_keys.hip", "rpa_tile.hip"]
-# A measurement aid of bench.py (a register-resident loop with a prefill tile's instruction mix); a library of its
-# own, so the op's library exports the op's entry points and nothing else.
-PROBE_SOURCE = "probe_mfma_mix.hip"
-PROBE_LIB_PATH = LIB_DIR / "libmfma_mix_probe.so"
-
 # -packed-fp32-ops is switched off on purpose: the compiler must not form v_pk_*_f32.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -70,14 +65,6 @@ def build(verbose: bool = True, extra_flags: list[str] | None = None, jobs: int 
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} ({LIB_PATH.stat().st_size} bytes)")
-    tmp = PROBE_LIB_PATH.with_suffix(".so.tmp")
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-shared", str(CSRC / PROBE_SOURCE), "-o", str(tmp)]
-    r = subprocess.run(cmd, capture_output=True, text=True)
-    if r.returncode != 0:
-        raise RuntimeError(f"hipcc failed for {PROBE_SOURCE}:\n{r.stdout}\n{r.stderr}")
-    os.replace(tmp, PROBE_LIB_PATH)
-    if verbose:
-        print(f"built {PROBE_LIB_PATH} ({PROBE_LIB_PATH.stat().st_size} bytes)")
     return LIB_PATH
 
 

@@ -1,5 +1,5 @@
 """bench.py's modes as child processes on the device: the JSON line of a short run carries the fields the contract asks
-for, and the measurement aids (back-to-back launches, the instruction-mix probe, the copy probe) run."""
+for, and the measurement aids (back-to-back launches, the copy probe) run."""
 
 import json
 import subprocess
@@ -41,9 +41,5 @@ def test_other_operations_and_cache_dtypes():
 def test_measurement_aids():
     d = run_bench("--workload", "decode_small", "--sustain", "0.2")
     assert d["launches"] >= 50 and d["ms_per_launch"] > 0
-    d = run_bench("--mfma-mix-probe", "0.2")
-    mixes = {(m["vector_elements"], m["lds_reads"]): m for m in d["mfma_mix_probe"]}
-    assert mixes[(0, 0)]["tflops"] > mixes[(64, 16)]["tflops"] > 100
-    assert 0.5 < mixes[(0, 0)]["shader_clock_ghz"] < 3.0 and 1000 <= mixes[(0, 0)]["cycles_per_32_mfma"] < 1300
     d = run_bench("--copy-probe", "64", "--steps", "3")
     assert d["copy_probe_bytes_read"] == 64 << 20

@@ -309,17 +309,6 @@ def test_xla_ffi_handlers_type_check_against_the_api_stand_in():
         assert f"XLA_FFI_DEFINE_HANDLER_SYMBOL({symbol}," in text, symbol
 
 
-def test_mfma_mix_probe_library_is_built_and_exports_its_entry_points():
-    """bench.py --mfma-mix-probe loads a library of its own (a measurement aid, not part of the op's ABI)."""
-    from ejkernel_amd.build import PROBE_LIB_PATH
-
-    lib = ctypes.CDLL(str(PROBE_LIB_PATH))
-    lib.mfma_mix_probe_src_bytes.restype = ctypes.c_uint64
-    assert lib.mfma_mix_probe_src_bytes() == (2048 + 2048) * 16
-    assert hasattr(lib, "mfma_mix_probe_launch")
-    assert not hasattr(_native.load(), "mfma_mix_probe_launch")
-
-
 def test_bench_long_prompt_parity_leg_detects_damage():
     """bench.py checks prompts too long for the restatement on a prefix (against it) and on sampled deep rows (float64):
     the float64 result passes, a damaged prefix row and a damaged sampled row (the last one is always sampled) fail."""
