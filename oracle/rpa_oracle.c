@@ -58,6 +58,7 @@ typedef struct {
   const float* sinks;
   void* out;
   int T, Hq, Hkv, D, page, P, pps, n_sinks, bf16, window;
+  int aux_bf16; /* the sinks' dtype is as narrow as the carry's: the epilogue rounds to bf16 at every op */
   float scale, cap;
 } Args;
 
@@ -94,7 +95,7 @@ CLONES static void pv_block(const float* restrict p, const float* restrict vb, f
 /* One (sequence, query block, kv head): the body of _process_query_block restricted to one kv head
  * (the reference carries all kv heads at once; they do not interact). */
 static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, float* sc, float* qs, float* o, float* upd) {
-  const int G = a->Hq / a->Hkv, D = a->D, bf = a->bf16;
+  const int G = a->Hq / a->Hkv, D = a->D, bf = a->bf16, ebf = a->bf16 && a->aux_bf16;
   const int q0 = a->cu[s], q_len = a->cu[s + 1] - q0, kv_len = a->ctx[s];
   const int kvblocks = a->pps >= 64 ? 64 : (a->pps > 1 ? a->pps : 1);
   const int kv_tok = a->page * kvblocks;
@@ -185,14 +186,15 @@ static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, 
       const float* orow = o + (size_t)r * D;
       float num = 1.f, den;
       if (a->sinks && a->n_sinks > 0) { /* :161-172 */
+        /* float32 sinks promote the epilogue of a bf16 carry to float32 (jnp.maximum at :166 and all after it) */
         const float* sk = a->sinks + (size_t)h * a->n_sinks;
         float smax = -INFINITY, ssum = 0.f;
-        for (int k = 0; k < a->n_sinks; ++k) smax = rb(sk[k], bf) > smax ? rb(sk[k], bf) : smax;
+        for (int k = 0; k < a->n_sinks; ++k) smax = rb(sk[k], ebf) > smax ? rb(sk[k], ebf) : smax;
         const float mt = m[r] > smax ? m[r] : smax;
-        for (int k = 0; k < a->n_sinks; ++k) ssum += rb(expf(rb(rb(sk[k], bf) - mt, bf)), bf);
-        num = rb(expf(rb(m[r] - mt, bf)), bf);
-        den = rb(rb(num * l[r], bf) + rb(ssum, bf), bf);
-        const float floor_ = rb(1e-6f, bf);
+        for (int k = 0; k < a->n_sinks; ++k) ssum += rb(expf(rb(rb(sk[k], ebf) - mt, ebf)), ebf);
+        num = rb(expf(rb(m[r] - mt, ebf)), ebf);
+        den = rb(rb(num * l[r], ebf) + rb(ssum, ebf), ebf);
+        const float floor_ = rb(1e-6f, ebf);
         den = den > floor_ ? den : floor_;
       } else {
         const float floor_ = rb(1e-6f, bf); /* :174, the weakly typed 1e-6 in the carry's dtype */
@@ -201,7 +203,7 @@ static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, 
       }
       const size_t dst = ((size_t)row * a->Hq + h) * D;
       for (int d = 0; d < D; ++d) {
-        float v = a->sinks && a->n_sinks > 0 ? rb(rb(num * orow[d], bf) / den, bf) : rb(orow[d] / den, bf);
+        float v = a->sinks && a->n_sinks > 0 ? rb(rb(rb(num * orow[d], ebf) / den, ebf), bf) : rb(orow[d] / den, bf);
         if (bf) ((uint16_t*)a->out)[dst + d] = f32_to_bf16(v);
         else ((float*)a->out)[dst + d] = v;
       }
@@ -212,9 +214,9 @@ static void run_item(const Args* a, int s, int qb, int j, float* kb, float* vb, 
 /* Returns 0, or -1 on bad arguments / allocation failure.  `threads` <= 0 keeps OpenMP's default. */
 int rpa_oracle_strict(const void* q, const void* kv, const int32_t* ctx, const int32_t* bt, const int32_t* cu, int num_seqs,
                       int T, int Hq, int Hkv, int D, int page, int P, int pps, float scale, float cap, int window,
-                      const float* sinks, int n_sinks, int is_bf16, void* out, int threads) {
+                      const float* sinks, int n_sinks, int is_bf16, void* out, int threads, int aux_is_bf16) {
   if (Hq % Hkv || Hq / Hkv > 64 || D <= 0 || page <= 0) return -1;
-  Args a = {q, kv, ctx, bt, cu, sinks, out, T, Hq, Hkv, D, page, P, pps, n_sinks, is_bf16, window, scale, cap};
+  Args a = {q, kv, ctx, bt, cu, sinks, out, T, Hq, Hkv, D, page, P, pps, n_sinks, is_bf16, window, aux_is_bf16, scale, cap};
   const int G = Hq / Hkv;
   const int kvblocks = pps >= 64 ? 64 : (pps > 1 ? pps : 1);
   const size_t kv_tok = (size_t)page * kvblocks, rows = (size_t)QBLK * G;

@@ -109,6 +109,11 @@ def _rounder(dtype):
     raise ValueError(f"unsupported dtype {dtype!r}")
 
 
+def _is_f32(dtype):
+    name = np.dtype(dtype).name if not isinstance(dtype, str) else dtype
+    return name in ("float32", "f32")
+
+
 def _clamp_start(start, size, total):
     """Start index of a lax.dynamic_slice window of `size` in an axis of length `total`."""
     return int(min(max(int(start), 0), total - size))
@@ -153,15 +158,26 @@ def rpa_strict(
     sliding_window=None,
     softmax_aux=None,
     io_dtype="bfloat16",
+    aux_dtype="float32",
 ):
     """Restates ``_ragged_paged_attention`` (_xla_impl_fwd.py:25-201).
 
     ``queries`` / ``kv_pages`` are float32 arrays whose values are representable in
     ``io_dtype`` (the storage dtype the reference would see).  Returns float32 holding
     ``io_dtype``-representable values, shape ``[T, Hq, D]``.
+
+    ``aux_dtype`` is the dtype the reference would see ``softmax_aux`` in.  The program keeps the sinks in
+    that dtype (:60-77), so JAX's promotion decides the precision of the sinks epilogue (:161-172): with
+    float32 sinks and a bfloat16 carry, ``jnp.maximum(max_block, s_max)`` is float32 and so is everything
+    after it, with the single cast of :179 at the end; with sinks as narrow as the carry every op of the
+    epilogue rounds to ``compute_dtype``.  float32 is what the device ABI takes.
     """
     Rq = _rounder(io_dtype)
     Rc = _rounder(compute_dtype)
+    # the epilogue's dtype: the wider of the carry's and the sinks' (bf16 with f32 promotes to f32)
+    wide_aux = _is_f32(aux_dtype) and not _is_f32(compute_dtype)
+    Re = _rounder("float32") if wide_aux else Rc
+    Ra = _rounder(aux_dtype)
     queries = np.asarray(queries, dtype=np.float32)
     kv_pages = np.asarray(kv_pages, dtype=np.float32)
     context_lens = np.asarray(context_lens)
@@ -251,14 +267,14 @@ def rpa_strict(
                     m = new_m
 
                 if sinks is not None:  # :161-172
-                    sb = np.broadcast_to(Rc(sinks)[None], (qblocks, Hkv, G, sinks.shape[-1]))
+                    sb = np.broadcast_to(Ra(sinks)[None], (qblocks, Hkv, G, sinks.shape[-1]))
                     s_max = sb.max(axis=3)
-                    m_tot = np.maximum(m, s_max)
-                    e_m = Rc(np.exp(Rc(m - m_tot)))
-                    e_s = Rc(np.exp(Rc(sb - m_tot[..., None])))
-                    denom = Rc(Rc(e_m * l) + Rc(e_s.sum(axis=3, dtype=np.float32)))
-                    denom = np.maximum(denom, Rc(np.float32(1e-6)))
-                    res = Rc(Rc(e_m[..., None] * o) / denom[..., None])
+                    m_tot = np.maximum(m, s_max)  # :166, in the promoted dtype
+                    e_m = Re(np.exp(Re(m - m_tot)))
+                    e_s = Re(np.exp(Re(sb - m_tot[..., None])))
+                    denom = Re(Re(e_m * l) + Re(e_s.sum(axis=3, dtype=np.float32)))
+                    denom = np.maximum(denom, Re(np.float32(1e-6)))
+                    res = Re(Re(e_m[..., None] * o) / denom[..., None])
                 else:  # :173-177
                     l = np.maximum(l, Rc(np.float32(1e-6)))
                     res = Rc(o / l[..., None])

@@ -29,7 +29,7 @@ def load():
         lib.rpa_oracle_strict.restype = ctypes.c_int
         lib.rpa_oracle_strict.argtypes = [ctypes.c_void_p] * 5 + [ctypes.c_int] * 8 + [
             ctypes.c_float, ctypes.c_float, ctypes.c_int, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
-            ctypes.c_void_p, ctypes.c_int]
+            ctypes.c_void_p, ctypes.c_int, ctypes.c_int]
         lib.rpa_oracle_max_threads.restype = ctypes.c_int
         _lib = lib
     return _lib
@@ -40,7 +40,8 @@ def max_threads() -> int:
 
 
 def rpa_strict_c(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, softmax_scale=None,
-                 logits_soft_cap=None, sliding_window=None, softmax_aux=None, io_dtype="bfloat16", threads=0):
+                 logits_soft_cap=None, sliding_window=None, softmax_aux=None, io_dtype="bfloat16", threads=0,
+                 aux_dtype="float32"):
     """Same contract as ``rpa_oracle.rpa_strict`` (compute dtype == io dtype): float32 arrays holding
     ``io_dtype``-representable values in, float32 ``[T, Hq, D]`` out."""
     lib = load()
@@ -69,7 +70,7 @@ def rpa_strict_c(queries, kv_pages, context_lens, block_tables, query_start_loc,
         q_buf.ctypes.data, kv_buf.ctypes.data, ctx.ctypes.data, bt.ctypes.data, cu.ctypes.data, n, T, Hq, Hkv, D, page, P,
         bt.shape[-1], scale, 0.0 if logits_soft_cap is None else float(logits_soft_cap),
         0 if sliding_window is None else int(sliding_window), None if sinks is None else sinks.ctypes.data, n_sinks,
-        1 if bf else 0, out.ctypes.data, int(threads))
+        1 if bf else 0, out.ctypes.data, int(threads), 1 if aux_dtype in ("bfloat16", "bf16") else 0)
     if rc != 0:
         raise RuntimeError("rpa_oracle_strict failed")
     return bf16_from_bits(out) if bf else out

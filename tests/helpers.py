@@ -40,11 +40,14 @@ def io_dtype(batch):
     return "bfloat16" if batch.queries.dtype == torch.bfloat16 else "float32"
 
 
-def run_strict(batch, compute_dtype=None, softmax_aux=None):
+def run_strict(batch, compute_dtype=None, softmax_aux=None, aux_dtype="float32"):
+    """`aux_dtype`: the dtype the reference would hold `softmax_aux` in (float32 is what the device ABI takes; sinks
+    as narrow as a bf16 carry keep the reference's whole epilogue in bf16)."""
     dt = io_dtype(batch)
     return rpa_oracle.rpa_strict(*oracle_args(batch), softmax_scale=batch.softmax_scale,
                                  logits_soft_cap=batch.logits_soft_cap, compute_dtype=compute_dtype or dt,
-                                 sliding_window=batch.sliding_window, softmax_aux=softmax_aux, io_dtype=dt)
+                                 sliding_window=batch.sliding_window, softmax_aux=softmax_aux, io_dtype=dt,
+                                 aux_dtype=aux_dtype)
 
 
 def run_exact(batch, softmax_aux=None):

@@ -142,6 +142,70 @@ def test_one_key_one_sink_closed_form():
             np.testing.assert_allclose(out[0, h], w * kv[pg, 0, 1], rtol=3e-6, atol=1e-6, err_msg=name)
 
 
+def _one_key_one_sink_bf16(sink):
+    """One bf16 decode row over one key with logit 0.5 exactly, and V values across five binades."""
+    b = _batch([1], [1], num_q_heads=1, num_kv_heads=1, head_dim=8, pages_per_seq=1, softmax_scale=1.0,
+               dtype=torch.bfloat16)
+    pg = int(b.block_tables[0, 0])
+    b.queries.zero_()
+    b.queries[0, 0, 0] = 1.0
+    b.kv_pages.zero_()
+    b.kv_pages[pg, 0, 0, 0] = 0.5
+    v = torch.tensor([1.0, 3.0, 100.0, -7.5, 0.4375, 21.0, -1.25, 13.0])
+    b.kv_pages[pg, 0, 1] = v.to(torch.bfloat16)
+    return b, v.double().numpy(), np.float32([[sink]])
+
+
+def test_float32_sinks_promote_the_epilogue_of_a_bf16_carry():
+    """The reference keeps `softmax_aux` in its own dtype (_xla_impl_fwd.py:60-77), so with float32 sinks and a bf16
+    carry `jnp.maximum(max_block, s_max)` (:166) is float32 and everything after it too, with one cast at the end
+    (:179): the result is the float64 closed form rounded to bf16 once.  With sinks as narrow as the carry every op
+    of :166-172 rounds to bf16, which here lands 1.3 % away: sink 5.3 becomes 5.3125, exp(-4.8125) and 1 + that
+    round again.  A restatement that rounds the epilogue whatever the sinks' dtype fails the first half."""
+    b, v, sink = _one_key_one_sink_bf16(5.3)
+    w = math.exp(0.5) / (math.exp(0.5) + math.exp(float(np.float32(5.3))))
+    want = w * v
+    rounded = O.bf16_round(want.astype(np.float32)).astype(np.float64)
+    step = 2.0 ** (np.floor(np.log2(np.abs(want))) - 7)
+    # the closed form is not within float32 noise of a rounding boundary, so one final cast decides the result
+    assert (np.abs(np.abs(want - rounded) - step / 2) > 1e-4 * step).all()
+    wide = run_strict(b, softmax_aux=sink, aux_dtype="float32")[0, 0].astype(np.float64)
+    np.testing.assert_array_equal(wide, rounded)
+    # by hand, every op rounded to bf16: m_tot = 5.3125, e_m = bf16(exp(-4.8125)) = 133 * 2**-14,
+    # denom = bf16(e_m * 1 + 1) = 1.0078125, out = bf16(bf16(e_m * v) / denom)
+    e_m, denom = 133 * 2.0 ** -14, 1.0078125
+    assert O.bf16_round(np.float32([math.exp(-4.8125)]))[0] == e_m and O.bf16_round(np.float32([e_m + 1]))[0] == denom
+    by_hand = O.bf16_round((O.bf16_round((e_m * v).astype(np.float32)).astype(np.float64) / denom).astype(np.float32))
+    narrow = run_strict(b, softmax_aux=sink, aux_dtype="bfloat16")[0, 0].astype(np.float64)
+    np.testing.assert_array_equal(narrow, by_hand.astype(np.float64))
+    assert (np.abs(narrow - wide) >= step).all(), (narrow, wide)  # the two epilogues are at least one bf16 step apart
+    # float32 storage has one epilogue whatever the sinks' dtype says
+    b32, _, _ = _one_key_one_sink_bf16(5.3)
+    b32.queries, b32.kv_pages = b32.queries.float(), b32.kv_pages.float()
+    np.testing.assert_allclose(run_strict(b32, softmax_aux=sink)[0, 0], want, rtol=3e-6)
+
+
+@pytest.mark.parametrize("aux_dtype", ["float32", "bfloat16"])
+def test_c_restatement_follows_the_sinks_dtype(aux_dtype):
+    from oracle.rpa_oracle_c import rpa_strict_c
+
+    b, _, sink = _one_key_one_sink_bf16(5.3)
+    got = rpa_strict_c(*oracle_args(b), softmax_scale=1.0, softmax_aux=sink, io_dtype="bfloat16", threads=1,
+                       aux_dtype=aux_dtype)
+    np.testing.assert_array_equal(got[0], run_strict(b, softmax_aux=sink, aux_dtype=aux_dtype)[0])
+    rng = np.random.default_rng(5)
+    b = make_batch([5, 1, 12], [300, 1000, 12], num_q_heads=4, num_kv_heads=2, head_dim=64, page_size=8,
+                   pages_per_seq=128, seed=12, dtype=torch.bfloat16)
+    aux = (3.0 * rng.standard_normal((4, 3))).astype(np.float32)
+    if aux_dtype == "bfloat16":
+        aux = O.bf16_round(aux)
+    got = rpa_strict_c(*oracle_args(b), softmax_scale=b.softmax_scale, softmax_aux=aux, io_dtype="bfloat16", threads=2,
+                       aux_dtype=aux_dtype)
+    want = run_strict(b, softmax_aux=aux, aux_dtype=aux_dtype)
+    d = np.abs(got - want)[: b.total_valid_tokens]
+    assert d.max() <= 8e-3 and (d > 0).mean() < 2e-3, (d.max(), (d > 0).mean())
+
+
 # ----------------------------------------------------------------------------- invariants
 
 

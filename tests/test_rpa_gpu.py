@@ -214,7 +214,7 @@ def test_bf16_head_dim_64_prefill_tiles(page, hq, hkv, window, sinks):
     out = to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES, softmax_aux=None if aux is None else aux.to(DEV)))
     aux_np = None if aux is None else aux.float().numpy()
     rows, what = b.total_valid_tokens, f"D=64 tiles page {page} {hq}/{hkv} W={window} sinks={sinks}"
-    strict, exact = run_strict(b, softmax_aux=aux_np)[:rows], run_exact(b, softmax_aux=aux_np)[:rows]
+    strict, exact = run_strict(b, softmax_aux=aux_np, aux_dtype="bfloat16")[:rows], run_exact(b, softmax_aux=aux_np)[:rows]
     finite = np.isfinite(strict).all(axis=(1, 2))  # short pages: the restatement's first KV block under a window is NaN
     assert finite.mean() > 0.5
     assert_bf16_parity_stepwise(out[:rows][finite], strict[finite], what)
@@ -324,9 +324,14 @@ def test_bf16_sinks(flags, shape):
     rng = np.random.default_rng(3)
     aux = {"per_q": rng.standard_normal((8, 2)), "per_kv": rng.standard_normal((2, 3)),
            "shared": rng.standard_normal(2)}[shape].astype(np.float32)
+    # float32 sinks (what the ABI takes): the reference's epilogue is float32 with one final cast
+    out32 = to_np(run_hip(b, flags, softmax_aux=torch.from_numpy(aux).to(DEV)))
+    assert_bf16_parity(out32, run_strict(b, softmax_aux=aux, aux_dtype="float32"), b.total_valid_tokens,
+                       f"float32 sinks {shape}")
+    # sinks in the queries' bf16: the reference rounds every op of the epilogue to bf16
     aux_bf = torch.from_numpy(aux).to(torch.bfloat16)
     out = to_np(run_hip(b, flags, softmax_aux=aux_bf.to(DEV)))
-    ref = run_strict(b, softmax_aux=aux_bf.float().numpy())
+    ref = run_strict(b, softmax_aux=aux_bf.float().numpy(), aux_dtype="bfloat16")
     assert_bf16_parity(out, ref, b.total_valid_tokens, f"sinks {shape}")
     base = to_np(run_hip(b, flags))
     assert np.abs(base - out)[: b.total_valid_tokens].max() > 1e-3  # sinks change the result
