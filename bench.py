@@ -162,7 +162,8 @@ def long_prompt_parity(batch, out, prefix_tokens=768, sampled_tokens=48):
     """Parity for a workload of few, very long prompts, which the CPU restatement cannot walk in seconds.  Causal
     attention makes the first `prefix_tokens` rows of a prompt the attention of that prefix alone: those rows are checked
     against the restatement of the reference program on the prefix as a prompt of its own (the parity bound, widened to
-    two bf16 steps of the value where that is larger).  Rows deep
+    two bf16 steps of the value where that is larger; the record also carries the count against the plain 2e-2 with
+    the smallest and largest |reference value| among those elements and the most keys any of their rows sees).  Rows deep
     in the prompt are checked, `sampled_tokens` positions per prompt, against a float64 evaluation on the device (plain
     torch: gather the prompt's K / V rows, scores, softmax, product) with the bound the tests use against float64."""
     import numpy as np
@@ -177,7 +178,8 @@ def long_prompt_parity(batch, out, prefix_tokens=768, sampled_tokens=48):
     page = m["page_size"]
     cu = batch.query_start_loc.cpu().numpy()
     worst = {"prefix_max_abs": 0.0, "prefix_mean_abs": 0.0, "deep_max_abs": 0.0, "deep_mean_abs": 0.0}
-    rows_prefix = rows_deep = over_bound = 0
+    rows_prefix = rows_deep = over_bound = over_plain = 0
+    plain_min_value, plain_max_value, plain_max_keys = None, None, 0
     rng = np.random.default_rng(0)
     for s in range(len(batch.q_lens)):
         L, q0 = int(batch.kv_lens[s]), int(cu[s])
@@ -204,7 +206,18 @@ def long_prompt_parity(batch, out, prefix_tokens=768, sampled_tokens=48):
         # tests.helpers.assert_bf16_parity_stepwise, which the prefill tiles are held to in the tests).
         ref64 = np.asarray(ref[:n0], np.float64)
         step = 2.0 ** (np.floor(np.log2(np.maximum(np.abs(ref64), 1e-30))) - 7)
-        over_bound += int((np.abs(np.asarray(got[:n0], np.float64) - ref64) > np.maximum(2e-2, 2 * step)).sum())
+        diff = np.abs(np.asarray(got[:n0], np.float64) - ref64)
+        over_bound += int((diff > np.maximum(2e-2, 2 * step)).sum())
+        # the same count against the plain bound, with what the elements over it have in common: the magnitude of the
+        # reference value there (a bf16 step of 2e-2 / 1.28 or more needs |value| >= 2) and how many keys the row sees
+        plain = diff > 2e-2
+        if plain.any():
+            over_plain += int(plain.sum())
+            vals = np.abs(ref64[plain])
+            plain_min_value = float(vals.min()) if plain_min_value is None else min(plain_min_value, float(vals.min()))
+            plain_max_value = float(vals.max()) if plain_max_value is None else max(plain_max_value, float(vals.max()))
+            first_key = 0 if not batch.sliding_window else np.maximum(0, np.nonzero(plain)[0] + 1 - batch.sliding_window)
+            plain_max_keys = max(plain_max_keys, int((np.nonzero(plain)[0] + 1 - first_key).max()))
         rows_prefix += n0
         # rows deep in the prompt, in float64 on the device
         pages = batch.kv_pages[batch.block_tables[s, : -(-L // page)].long()]          # [pages, page, 2 Hkv, D]
@@ -226,6 +239,8 @@ def long_prompt_parity(batch, out, prefix_tokens=768, sampled_tokens=48):
         del pages, kv, k, v
     worst["deep_mean_abs"] /= max(rows_deep, 1)
     worst.update({"rows_prefix": rows_prefix, "rows_deep": rows_deep, "prefix_elements_over_bound": over_bound,
+                  "prefix_elements_over_2e-2": over_plain, "over_2e-2_min_abs_value": plain_min_value,
+                  "over_2e-2_max_abs_value": plain_max_value, "over_2e-2_max_visible_keys": plain_max_keys,
                   "ok": bool(over_bound == 0 and worst["prefix_mean_abs"] <= 2e-3 and
                              worst["deep_max_abs"] <= 4e-2 and worst["deep_mean_abs"] <= 2e-3)})
     return worst

@@ -321,11 +321,21 @@ def test_bench_long_prompt_parity_leg_detects_damage():
     out = torch.from_numpy(np.asarray(run_exact(b), np.float32)).to(torch.bfloat16)
     r = bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)
     assert r["ok"] and r["rows_prefix"] == 100 and 1 <= r["rows_deep"] <= 6
+    assert r["prefix_elements_over_2e-2"] >= r["prefix_elements_over_bound"] == 0
     out[L - 1] += 0.25
     assert not bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)["ok"]
     out[L - 1] -= 0.25
     out[7] += 0.5
     assert not bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)["ok"]
+    out[7] -= 0.5
+    # the widened bound only ever applies to values of magnitude 2 or more: an element below 2 that is off by 0.021
+    # fails, and the record counts it against the plain bound and names its magnitude and its row's key count
+    ref = np.asarray(run_exact(b), np.float32)
+    t, h, d = [(t, h, d) for t in range(40, 60) for h in range(2) for d in range(8) if 0.3 < abs(ref[t, h, d]) < 1.0][0]
+    out[t, h, d] = float(out[t, h, d]) + 0.0215 * (1 if ref[t, h, d] > 0 else -1)
+    r = bench.long_prompt_parity(b, out, prefix_tokens=100, sampled_tokens=6)
+    assert not r["ok"] and r["prefix_elements_over_bound"] >= 1 and r["prefix_elements_over_2e-2"] >= 1
+    assert r["over_2e-2_min_abs_value"] < 1.0 and r["over_2e-2_max_visible_keys"] >= t + 1
 
 
 def test_bench_power_sensor_and_gpu_count_guard():
