@@ -39,7 +39,13 @@ def measured_traffic_bytes(workload: str):
 # gets, and pools allocated early in a process get what a process of their own would (gemma2_local 0.386 ms as the
 # second workload of a process, 0.392-0.398 ms as the fifth; 0.380 ms alone).
 EXTRA_CONFIGS = ["gemma2_local", "decode_long_context", "decode_small", "mixed_prefill_decode", "mixed_prefill_only",
-                 "prefill_single_16k"]
+                 "prefill_single_16k",
+                 # What a serving caller with padded static shapes gets (max_num_seqs 512, query rows rounded up to
+                 # 8192 / 16384, num_seqs as is): the library's own choice of kernel instantiation, made from those
+                 # shapes, and the choice the caller names through RaggedPageAttentionConfig.num_queries_per_block.
+                 ("decode_llama3_8b_padded", None), ("decode_llama3_8b_padded", 16),
+                 ("mixed_prefill_decode_padded", None), ("mixed_prefill_decode_padded", 128),
+                 ("mixed_prefill_only_padded", None), ("mixed_prefill_only_padded", 256)]
 # Prompts too long for the CPU restatement: checked on a prefix against it and on sampled rows against float64
 # (long_prompt_parity).  prefill_single_16k is not one of the five benchmark configurations: it shows the prefill tile
 # where a tile walks up to 16384 keys and what a tile costs besides its key loop no longer counts.
@@ -433,12 +439,12 @@ def settle(fn, seconds=SETTLE_S):
         torch.cuda.synchronize()
 
 
-def time_steps(step, steps, warmup):
+def time_steps(step, steps, warmup, settle_s=SETTLE_S):
     """`warmup` untimed calls, then `steps` calls bracketed by synchronisation: wall time per step, the per-call
     durations between HIP events on the stream the op launches on (torch's current one), and the last output."""
     import torch
 
-    settle(step)
+    settle(step, settle_s)
     out = None
     for _ in range(warmup):
         out = step()
@@ -543,49 +549,122 @@ def sustain(fn, seconds, what, flops=None, nbytes=None, quiet=False):
     return res
 
 
-def measure_config(name, steps, warmup, want_parity):
-    """One entry of "configs": the named workload at full size, timed like the headline one and checked against the
-    CPU restatement on a small sample of its sequences."""
+def graph_replay_ms(step, reps):
+    """The call captured in a HIP graph and replayed `reps` times: milliseconds per replay (no host code per step)."""
+    import torch
+
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+        side.synchronize()
+        with torch.cuda.graph(g, stream=side):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for _ in range(5):
+        g.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        g.replay()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / reps
+
+
+def measure_ref_bench(steps, warmup, want_parity, want_baseline):
+    """The reference's own benchmark grid (benchmarks/benchmark_ragged_page_attn.py:148-185: max_num_seqs {8, 16, 32} x
+    page_size {8 .. 128}, 16 pages per sequence, 16 / 4 heads, head_dim 128, q_len ~ U[1, kv_len]), one entry per shape:
+    microseconds per call and per HIP-graph replay (these batches are launch-latency bound), parity of every row against
+    the CPU restatement of the reference program and that restatement's time for the whole batch on the host cores."""
     import torch
 
     from ejkernel_amd.modules import ragged_page_attention
     from ejkernel_amd.roofline import algorithmic_counts
+    from ejkernel_amd.workloads import REF_BENCH_GRID, make_workload
+    from oracle import rpa_oracle_c
+    from tests.helpers import err_stats, oracle_args, to_np
+
+    out_entries = []
+    threads = rpa_oracle_c.max_threads()
+    for S, page in REF_BENCH_GRID:
+        name = f"ref_bench_{S}_{page}"
+        batch = make_workload(name, device="cuda:0")
+        m = batch.meta
+        counts = algorithmic_counts(batch.q_lens, batch.kv_lens, num_q_heads=m["num_q_heads"], num_kv_heads=m["num_kv_heads"],
+                                    head_dim=m["head_dim"], page_size=m["page_size"], sliding_window=None)
+
+        def step():
+            return ragged_page_attention(*batch.args(), **batch.kwargs())
+
+        ms_per_step, ev_ms, out = time_steps(step, steps, warmup, settle_s=0.05)
+        entry = {"workload": name, "max_num_seqs": S, "page_size": page, "query_tokens": counts["tokens"],
+                 "kv_tokens": int(batch.kv_lens.sum()), "us_per_call": ms_per_step * 1e3,
+                 "kernel_us_avg": sum(ev_ms) / len(ev_ms) * 1e3, "kernel_us_min": ev_ms[0] * 1e3,
+                 "graph_replay_us": graph_replay_ms(step, max(steps, 50)) * 1e3,
+                 "tokens_per_s": counts["tokens"] / (ms_per_step * 1e-3),
+                 "gflops": counts["flops"] / 1e9, "mbytes": counts["bytes"] / 1e6}
+        if want_parity or want_baseline:
+            args = oracle_args(batch)
+            t0 = time.perf_counter()
+            ref = rpa_oracle_c.rpa_strict_c(*args, softmax_scale=batch.softmax_scale, io_dtype="bfloat16", threads=threads)
+            dt = time.perf_counter() - t0
+            rows = batch.total_valid_tokens
+            if want_parity:
+                mx, mean = err_stats(to_np(out), ref, rows)
+                over = int((np_abs_diff(to_np(out)[:rows], ref[:rows]) > 2e-2).sum())
+                entry["parity"] = {"max_abs": mx, "mean_abs": mean, "rows": rows, "elements_over_2e-2": over,
+                                   "ok": bool(mx <= 2e-2 and mean <= 2e-3)}
+            if want_baseline:
+                entry["cpu_us_per_call"] = dt * 1e6
+                entry["cpu_cores"] = int(threads)
+        out_entries.append(entry)
+        del batch, out
+    torch.cuda.empty_cache()
+    return out_entries
+
+
+def np_abs_diff(a, b):
+    import numpy as np
+
+    return np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64))
+
+
+def measure_config(name, steps, warmup, want_parity, queries_per_block=None):
+    """One entry of "configs": the named workload at full size, timed like the headline one and checked against the
+    CPU restatement on a small sample of its sequences.  `queries_per_block` is passed on as
+    RaggedPageAttentionConfig.num_queries_per_block (the caller's hint for the kernel instantiation)."""
+    import torch
+
+    from ejkernel_amd.modules import RaggedPageAttentionConfig, ragged_page_attention
+    from ejkernel_amd.roofline import algorithmic_counts
     from ejkernel_amd.workloads import make_workload
 
     batch = make_workload(name, device="cuda:0")
+    cfg = None if queries_per_block is None else RaggedPageAttentionConfig(num_queries_per_block=queries_per_block)
     m = batch.meta
     counts = algorithmic_counts(batch.q_lens, batch.kv_lens, num_q_heads=m["num_q_heads"], num_kv_heads=m["num_kv_heads"],
                                 head_dim=m["head_dim"], page_size=m["page_size"], sliding_window=batch.sliding_window)
 
     def step():
-        return ragged_page_attention(*batch.args(), **batch.kwargs())
+        return ragged_page_attention(*batch.args(), cfg=cfg, **batch.kwargs())
 
     ms_per_step, ev_ms, out = time_steps(step, steps, warmup)
     roof = roofline_of(counts, ev_ms)
     roof["traffic"] = measured_traffic_bytes(name)
-    if roof["bound"] == "mfma":
+    if roof["bound"] == "mfma" and not name.endswith("_padded"):
         roof["library_gemm_tflops"] = library_gemm_tflops()
     entry = {"workload": name, "ms_per_step": ms_per_step, "kernel_ms_avg": roof["kernel_ms_avg"],
              "tokens_per_s": counts["tokens"] / (ms_per_step * 1e-3), "roofline": roof,
              "host_overhead_ms": ms_per_step - roof["kernel_ms_avg"]}
+    if name.endswith("_padded"):
+        entry["static_shapes"] = {"total_tokens": int(batch.queries.shape[0]), "max_num_seqs": int(m["max_num_seqs"]),
+                                  "num_seqs": len(batch.q_lens)}
+        entry["num_queries_per_block"] = queries_per_block
     if name == "decode_small":
         # the launch-bound configuration: the same call replayed from a HIP graph, where no host code runs per step
-        g = torch.cuda.CUDAGraph()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            step()
-            side.synchronize()
-            with torch.cuda.graph(g, stream=side):
-                step()
-        torch.cuda.current_stream().wait_stream(side)
-        torch.cuda.synchronize()
-        reps = max(steps, 50)
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            g.replay()
-        torch.cuda.synchronize()
-        entry["graph_replay_ms"] = (time.perf_counter() - t0) * 1e3 / reps
+        entry["graph_replay_ms"] = graph_replay_ms(step, max(steps, 50))
     if want_parity:
         if name in LONG_PROMPT_CONFIGS:
             entry["parity"] = long_prompt_parity(batch, out)
@@ -697,12 +776,17 @@ def main():
         # A failure in one of the other configurations must not cost the headline line: it is reported in place of the
         # entry (the exception's text; nothing is retried, and a device fault would end the process anyway).
         line["configs"] = []
-        for name in EXTRA_CONFIGS:
+        for item in EXTRA_CONFIGS:
+            name, hint = item if isinstance(item, tuple) else (item, None)
             try:
-                line["configs"].append(measure_config(name, args.steps, args.warmup, not args.no_parity))
+                line["configs"].append(measure_config(name, args.steps, args.warmup, not args.no_parity, hint))
             except Exception as e:  # noqa: BLE001
                 line["configs"].append({"workload": name, "error": f"{type(e).__name__}: {e}"[:500]})
                 torch.cuda.empty_cache()
+        try:
+            line["ref_bench"] = measure_ref_bench(args.steps, args.warmup, not args.no_parity, not args.no_cpu_baseline)
+        except Exception as e:  # noqa: BLE001
+            line["ref_bench"] = {"error": f"{type(e).__name__}: {e}"[:500]}
     print(json.dumps(line))
 
 

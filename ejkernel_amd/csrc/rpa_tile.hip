@@ -196,20 +196,38 @@ void rpa_tile_kernel(TileArgs a) {
     }
   }
 
-  // ---- rows past the ragged batch are zero
-  {
-    const int total_rows = batch_rows(p, nseq);
-    const int row_u4 = p.num_q_heads * p.head_dim / 8;  // 16-byte pieces per row
-    u32x4_t* o4 = static_cast<u32x4_t*>(p.out);
-    for (int row = total_rows + blockIdx.x; row < p.total_tokens; row += gridDim.x)
-      for (int k = tid; k < row_u4; k += kWgThreads) o4[static_cast<size_t>(row) * row_u4 + k] = u32x4_t{0u, 0u, 0u, 0u};
-  }
+  // ---- rows past the ragged batch are zero.  A caller with padded static shapes has thousands of them (8192 rows
+  // allocated for 256 decode tokens are 65 MB of zeros), so they are written where they cost least: by the workgroups
+  // that have nothing else to do when there are such, otherwise by every workgroup after its work, when the
+  // workgroups that finish early would idle.
+  // The loop reads everything it needs afresh from the kernel arguments (through a pointer the compiler cannot see
+  // through), so that placing it after the work keeps no value of the schedule alive across the hot loops.
+  auto zero_rows_past_batch = [](int first, int stride) {
+    typedef const __attribute__((address_space(4))) TileArgs* KernArgs;
+    KernArgs ap = (KernArgs)__builtin_amdgcn_kernarg_segment_ptr();
+    asm volatile("" : "+s"(ap));
+    RpaParams pp;  // the fields the row arithmetic reads
+    pp.num_seqs = ap->p.num_seqs;
+    pp.query_start_loc = ap->p.query_start_loc;
+    pp.max_num_seqs = ap->p.max_num_seqs;
+    pp.total_tokens = ap->p.total_tokens;
+    const int total_rows = batch_rows(pp, seq_count(pp));
+    const int row_u4 = ap->p.num_q_heads * ap->p.head_dim / 8;  // 16-byte pieces per row
+    u32x4_t* o4 = static_cast<u32x4_t*>(ap->p.out);
+    for (int row = total_rows + first; row < pp.total_tokens; row += stride)
+      for (int k = threadIdx.x; k < row_u4; k += kWgThreads)
+        __builtin_nontemporal_store(u32x4_t{0u, 0u, 0u, 0u}, &o4[static_cast<size_t>(row) * row_u4 + k]);
+  };
 
   // A batch without prefill tiles is pure streaming: it runs fastest with one workgroup per compute unit, so
-  // the second half of the grid (dispatched after every unit has one workgroup) leaves at once.
+  // the second half of the grid (dispatched after every unit has one workgroup) does not stream.
   const int grid_all = static_cast<int>(gridDim.x);
   const int grid_wgs = total_wg == 0 ? min(grid_all, a.stream_grid) : grid_all;
-  if (static_cast<int>(blockIdx.x) >= grid_wgs) return;
+  const bool idle_wgs_exist = grid_wgs < grid_all;
+  if (static_cast<int>(blockIdx.x) >= grid_wgs) {
+    zero_rows_past_batch(static_cast<int>(blockIdx.x) - grid_wgs, grid_all - grid_wgs);
+    return;
+  }
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
   // `kind` says which count the array sums (0 items, 1 stream tiles, 2 prefill tiles); `base` receives start[s].
@@ -427,6 +445,7 @@ void rpa_tile_kernel(TileArgs a) {
       }
     }
   }
+  if (!idle_wgs_exist) zero_rows_past_batch(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
 }
 
 // ----------------------------------------------------------------------------- host side
@@ -504,15 +523,31 @@ void tiled_workspace_layout(const RpaParams& p, WorkspaceLayout* wl) {
   wl->total_bytes = wl->partial_ml_off + wl->partial_ml_bytes;
 }
 
+// What RaggedPageAttentionConfig.num_queries_per_block (RpaParams::num_queries_per_block) asks for.  The host sees
+// padded static shapes only -- total_tokens and max_num_seqs of a serving batch are upper bounds, the lengths live on
+// the device -- so a caller that knows its batch names the tile shape here: up to 16 query rows per tile is the
+// wave-level loop alone (decode steps, short chunks), up to 128 the 128-row workgroup tiles, more the 256-row
+// software-pipelined tiles where they exist (head_dim 128, no soft cap, pages of 16 tokens or more; the 128-row tiles
+// otherwise).  0 leaves the choice to the rules below.  RPA_FLAG_* tile flags, when set, come first.
+static bool tiles_flagged(const RpaParams& p) { return (p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) != 0; }
+// +1 the pipelined tile is asked for, -1 it is ruled out, 0 the size rule decides
+static int pipe_choice_of(const RpaParams& p) {
+  if ((p.flags & RPA_FLAG_PLAIN_TILES) != 0) return -1;
+  if ((p.flags & RPA_FLAG_PIPE_TILES) != 0) return 1;
+  if (p.num_queries_per_block <= 0) return 0;
+  return p.num_queries_per_block > 128 ? 1 : -1;
+}
+
 // Small batches -- one query token per sequence by construction, or so few (token, head) rows that prefill tiles
 // of 128 rows would leave most of the grid idle -- take the instantiation without prefill tiles: the decode loop
 // alone gets a register allocation without spills, and short prefill chunks spread over four times as many
 // wavefronts as wave-level items (512 tokens from scratch at 32 heads: 30 us against 65 us with tiles).
-static bool small_batch_of(const RpaParams& p) {
-  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
-  return p.query_start_loc == nullptr ||
-         ((p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES)) == 0 && rows <= tune().wave_only_rows);
+static bool wave_only_by_sizes(const RpaParams& p) {
+  if (tiles_flagged(p)) return false;
+  if (p.num_queries_per_block > 0) return p.num_queries_per_block <= 16;
+  return static_cast<int64_t>(p.total_tokens) * p.num_q_heads <= tune().wave_only_rows;
 }
+static bool small_batch_of(const RpaParams& p) { return p.query_start_loc == nullptr || wave_only_by_sizes(p); }
 
 constexpr uint64_t kLogitStashMaxBytes = 2ull << 30;
 static uint32_t logit_pitch_of(const RpaParams& p) {
@@ -521,9 +556,8 @@ static uint32_t logit_pitch_of(const RpaParams& p) {
 }
 uint64_t logit_stash_bytes(const RpaParams& p) {
   // decided by the sizes alone: a size query may come before the pointers are set
-  const int64_t rows = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
-  if (tune().no_logit_stash != 0 || rows <= 0 || rows > tune().wave_only_rows ||
-      (p.flags & (RPA_FLAG_PREFILL_TILES | RPA_FLAG_PIPE_TILES | RPA_FLAG_NO_LOGIT_STASH)) != 0)
+  if (tune().no_logit_stash != 0 || p.total_tokens <= 0 || p.num_q_heads <= 0 || !wave_only_by_sizes(p) ||
+      (p.flags & RPA_FLAG_NO_LOGIT_STASH) != 0)
     return 0;
   const uint64_t bytes = static_cast<uint64_t>(p.total_tokens) * p.num_q_heads * logit_pitch_of(p) * 4ull;
   return bytes <= kLogitStashMaxBytes ? bytes : 0;
@@ -582,6 +616,12 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.logit_pitch = 0;
   a.sched_shift = sched_shift_for(p.max_num_seqs);
   a.min_share_tiles = tune().min_share_tiles;
+  // RaggedPageAttentionConfig.num_kv_pages_per_block: the least stretch of a sequence, in pages, that a streaming
+  // wavefront takes before a batch is spread over more wavefronts (split-K granularity of small batches)
+  if (p.num_kv_pages_per_block > 0) {
+    const int64_t keys = static_cast<int64_t>(p.num_kv_pages_per_block) * p.page_size;
+    a.min_share_tiles = static_cast<int>(std::min<int64_t>(4096, std::max<int64_t>(1, keys / (p.head_dim > 128 ? 16 : 32))));
+  }
   // a part costs about as much as streaming 128 keys: 4 tiles of 32 keys, 8 of 16 (head_dim 256)
   a.item_pad_tiles = tune().item_pad_tiles >= 0 ? tune().item_pad_tiles : (p.head_dim > 128 ? 8 : 4);
   a.page_shift = __builtin_ctz(p.page_size);
@@ -653,9 +693,10 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // so it goes by the average number of query tokens per sequence.
     const bool pipe_ok = p.head_dim == 128 && p.page_size >= 16 && p.logits_soft_cap == 0.f &&
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
-    const bool pipe_wanted = (p.flags & RPA_FLAG_PLAIN_TILES) == 0 &&
-                             ((p.flags & RPA_FLAG_PIPE_TILES) != 0 ||
-                              (tune().pipe != 0 && static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs));
+    const int pipe_choice = pipe_choice_of(p);
+    const bool pipe_wanted = pipe_choice > 0 ||
+                             (pipe_choice == 0 && tune().pipe != 0 &&
+                              static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs);
     if (pipe_wanted && pipe_ok && canonical) {
       // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
       // number on every XCD) take the decode stream first and join the prefill queues when it is done

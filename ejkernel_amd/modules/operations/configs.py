@@ -6,10 +6,17 @@ Field names, order and defaults are those of
 can be passed here unchanged.  With a single HIP implementation behind the op the fields
 mean:
 
-``num_queries_per_block``   query tokens per prefill tile (None = library default)
-``num_kv_pages_per_block``  pages per decode split (None = chosen from the batch on device)
-``num_warps``               wavefronts per workgroup (only 4 is built; other values are ignored)
-``num_stages``              accepted, unused
+``num_queries_per_block``   query rows of a sequence per tile, a hint for the choice of kernel instantiation, which
+                            the library otherwise makes from the (possibly padded) static shapes: 1..16 = the
+                            wave-level loop alone (decode steps, short chunks); 17..128 = 128-row workgroup tiles
+                            for long chunks; above 128 = 256-row software-pipelined tiles where they exist
+                            (head_dim 128, no soft cap, pages of 16 tokens or more).  None = library default
+                            (wave-level loop up to 20480 (token, query head) rows, pipelined tiles from 128
+                            tokens per ``max_num_seqs``).  Results stay within the same tolerance either way.
+``num_kv_pages_per_block``  the least stretch of a sequence, in pages, one streaming wavefront takes before a small
+                            batch is spread over more wavefronts (None = 2 tiles of 32 keys, more for long sequences)
+``num_warps``               accepted, ignored (workgroups have 4 wavefronts)
+``num_stages``              accepted, ignored (2 LDS stages in the 128-row tile, 4 in the pipelined one)
 ``platform`` / ``backend``  accepted and validated, never used for dispatch
 """
 

@@ -29,7 +29,11 @@ from .configs import _PLATFORMS, RaggedPageAttentionConfig
 __all__ = ["RaggedPageAttention", "ragged_page_attention"]
 
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
-_MAX_WORKSPACES = 16  # (device, stream) pairs kept; the least recently used one goes first (about 35 MB each)
+# (device, stream) pairs kept; the least recently used one goes first.  A workspace is about 35 MB (70 MB at head_dim
+# 256) unless ragged_page_attention_v3 keeps the logits of an 8-bit cache between its two launches (up to 2 GiB, 268 MB
+# for 256 decode steps over 8192-token block-table rows), so the cache is bounded in bytes as well.
+_MAX_WORKSPACES = 16
+_MAX_WORKSPACE_BYTES = 4 << 30
 _workspaces_lock = threading.Lock()  # host threads launch on streams of their own at the same time
 
 
@@ -138,7 +142,9 @@ def _workspace(device: torch.device, nbytes: int, stream_ptr: int) -> torch.Tens
             # A stream that no longer exists leaves its workspace behind (torch has no hook for a stream's end), so the
             # cache is bounded.  The evicted tensor's memory goes back to torch's caching allocator, which keeps it away
             # from other streams until the work queued on this one has finished.
-            while len(_workspaces) >= _MAX_WORKSPACES:
+            want = max(nbytes, 256)
+            while _workspaces and (len(_workspaces) >= _MAX_WORKSPACES or
+                                   sum(t.numel() for t in _workspaces.values()) + want > _MAX_WORKSPACE_BYTES):
                 _workspaces.pop(next(iter(_workspaces)))
             ws = torch.empty(max(nbytes, 256), dtype=torch.uint8, device=device)
             rc = _native.load().rpa_workspace_init(ctypes.c_void_p(ws.data_ptr()), ws.numel(), ctypes.c_void_p(stream_ptr))

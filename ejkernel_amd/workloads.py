@@ -265,8 +265,15 @@ def _randn_chunked(shape, gen, device, dtype, chunk_elems=1 << 27):
 
 def make_batch(q_lens, kv_lens, *, num_q_heads, num_kv_heads, head_dim, page_size, pages_per_seq, num_pages=None,
                seed=0, device="cpu", dtype=torch.bfloat16, max_num_seqs=None, sliding_window=None,
-               logits_soft_cap=None, softmax_scale=None, slack_rows=8, permute_pages=True, name="") -> Batch:
-    """Build one ragged batch. ``q_lens[i] <= kv_lens[i]``; pages of different sequences are distinct."""
+               logits_soft_cap=None, softmax_scale=None, slack_rows=8, permute_pages=True, name="",
+               total_tokens=None, pool_seqs=None) -> Batch:
+    """Build one ragged batch. ``q_lens[i] <= kv_lens[i]``; pages of different sequences are distinct.
+
+    ``max_num_seqs`` and ``total_tokens`` pad the static shapes the way a serving caller does (block table, lengths and
+    query rows allocated for the largest batch, ``num_seqs`` saying how many sequences are present).  ``pool_seqs``
+    sizes the page pool and the permutation for that many block-table rows (default ``max_num_seqs``); rows past it
+    point at page 0 and belong to no sequence, so a padded batch can share the pool, the pages and the queries of the
+    unpadded one with the same seed."""
     q_lens = np.asarray(q_lens, dtype=np.int64)
     kv_lens = np.asarray(kv_lens, dtype=np.int64)
     S = len(q_lens)
@@ -274,14 +281,20 @@ def make_batch(q_lens, kv_lens, *, num_q_heads, num_kv_heads, head_dim, page_siz
     assert max_num_seqs >= S and len(kv_lens) == S
     assert (q_lens <= kv_lens).all(), "q_len must not exceed kv_len"
     assert kv_lens.max(initial=0) <= pages_per_seq * page_size, "pages_per_seq too small for kv_lens"
-    num_pages = num_pages or max_num_seqs * pages_per_seq
-    assert num_pages >= max_num_seqs * pages_per_seq
+    pool_seqs = pool_seqs or max_num_seqs
+    assert S <= pool_seqs <= max_num_seqs
+    num_pages = num_pages or pool_seqs * pages_per_seq
+    assert num_pages >= pool_seqs * pages_per_seq
     rng = np.random.Generator(np.random.PCG64(seed))
     perm = rng.permutation(num_pages) if permute_pages else np.arange(num_pages)
-    block_tables = perm[: max_num_seqs * pages_per_seq].reshape(max_num_seqs, pages_per_seq).astype(np.int32)
+    block_tables = np.zeros((max_num_seqs, pages_per_seq), np.int32)
+    block_tables[:pool_seqs] = perm[: pool_seqs * pages_per_seq].reshape(pool_seqs, pages_per_seq)
 
     total = int(q_lens.sum())
     t_alloc = ((total + 7) // 8) * 8 + slack_rows if slack_rows else total
+    if total_tokens is not None:
+        assert total_tokens >= t_alloc, "total_tokens must cover the query rows and their slack"
+        t_alloc = int(total_tokens)
     cu = np.zeros(max_num_seqs + 1, dtype=np.int32)
     cu[1:S + 1] = np.cumsum(q_lens)
     cu[S + 1:] = total
@@ -347,12 +360,32 @@ WORKLOADS = {
     "mixed_head_dim_96": "16 chunks x 256 tokens (prior 0..2048) + 112 decode seqs (kv 256..4096), 32q/8kv heads, D=96, page 32",
     # one long prompt: 512 prefill tiles of 256 rows that walk up to 16384 keys each (per-tile costs vanish)
     "prefill_single_16k": "1 prompt x 16384 tokens from scratch, 32q/8kv heads, D=128, page 32",
+    # the static shapes of a serving caller: the same sequences, pages and queries as the unpadded workloads inside
+    # arrays allocated for the largest batch (max_num_seqs 512, query rows rounded up), num_seqs as is
+    "decode_llama3_8b_padded": "decode_llama3_8b inside max_num_seqs 512 and 8192 query rows",
+    "mixed_prefill_decode_padded": "mixed_prefill_decode inside max_num_seqs 512 and 16384 query rows",
+    "mixed_prefill_only_padded": "mixed_prefill_only inside max_num_seqs 512 and 16384 query rows",
 }
+
+# The reference's own benchmark grid (benchmarks/benchmark_ragged_page_attn.py:148-185): max_num_seqs x page_size at
+# 16 pages per sequence, 16 query / 4 kv heads, head_dim 128; "ref_bench_<max_num_seqs>_<page_size>".
+REF_BENCH_GRID = [(s, p) for s in (8, 16, 32) for p in (8, 16, 32, 64, 128)]
+for _s, _p in REF_BENCH_GRID:
+    WORKLOADS[f"ref_bench_{_s}_{_p}"] = (f"the reference benchmark's shape: {_s} seqs, kv 1..{16 * _p}, q 1..kv, 16q/4kv heads, "
+                                         f"D=128, page {_p}, 16 pages per sequence, identity block table")
 
 
 def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bfloat16) -> Batch:
     """Build a named workload. ``scale`` < 1 shrinks sequence counts and lengths for tests."""
     only = None
+    padded = None
+    if name.endswith("_padded"):  # the unpadded workload's draw inside larger static shapes
+        name = name[: -len("_padded")]
+        padded = dict(max_num_seqs=512, total_tokens=8192 if name == "decode_llama3_8b" else 16384)
+        if scale != 1.0:
+            padded = dict(max_num_seqs=max(8, int(512 * scale)), total_tokens=max(64, int(padded["total_tokens"] * scale)))
+    if name.startswith("ref_bench_"):
+        return _ref_bench_workload(name, device=device, dtype=dtype)
     if name in ("mixed_prefill_only", "mixed_decode_only"):
         only, name = name, "mixed_prefill_decode"
     idx = list(WORKLOADS).index(name) + 1
@@ -377,8 +410,11 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         kv = rng.integers(n(512), n(8192) + 1, size=S)
         pps = pages(n(8192), 16)
         pool = max(S * pps, n(160000))
+        pad = {} if padded is None else dict(pool_seqs=S, max_num_seqs=max(S, padded["max_num_seqs"]),
+                                             total_tokens=max(S + 16, padded["total_tokens"]))
         return make_batch(np.ones(S, int), kv, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
-                          pages_per_seq=pps, num_pages=pool, seed=seed, device=device, dtype=dtype, name=name)
+                          pages_per_seq=pps, num_pages=pool, seed=seed, device=device, dtype=dtype,
+                          name=name + ("_padded" if padded else ""), **pad)
     if name == "mixed_prefill_decode":
         n_pre, n_dec = n(16), n(240)
         chunk = n(512)
@@ -390,8 +426,12 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         if only is not None:
             order = np.array([o for o in order if (o < n_pre) == (only == "mixed_prefill_only")])
         pps = pages(max(n(8192), n(4096) + chunk), 32)
+        S = len(order)
+        pad = {} if padded is None else dict(pool_seqs=S, max_num_seqs=max(S, padded["max_num_seqs"]),
+                                             total_tokens=max(int(q[order].sum()) + 16, padded["total_tokens"]))
         return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
-                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype, name=only or name)
+                          pages_per_seq=pps, seed=seed, device=device, dtype=dtype,
+                          name=(only or name) + ("_padded" if padded else ""), **pad)
     if name == "prefill_long":
         L = n(8192)
         return make_batch(np.full(2, L), np.full(2, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
@@ -445,6 +485,25 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         return make_batch(np.ones(S, int), kv, num_q_heads=64, num_kv_heads=8, head_dim=128, page_size=64,
                           pages_per_seq=pps, num_pages=pool, seed=seed, device=device, dtype=dtype, name=name)
     raise KeyError(name)
+
+
+def _ref_bench_workload(name: str, *, device="cpu", dtype=torch.bfloat16) -> Batch:
+    """One shape of the reference's benchmark grid, drawn the way its input generator draws
+    (benchmarks/benchmark_ragged_page_attn.py:40-129): ``num_seqs = max_num_seqs``, ``kv_len ~ U[1, pages_per_seq *
+    page_size]``, ``q_len ~ U[1, kv_len]``, identity block table, 16 query / 4 kv heads, head_dim 128, 16 pages per
+    sequence, N(0,1) data.  Different here: NumPy's generator instead of jax.random, and the query array carries the
+    slack rows that keep the reference program's 8-row query blocks inside the array (its generator allocates exactly
+    ``sum(q_len)`` rows, where the program's clamped block windows overwrite rows of earlier sequences)."""
+    _, _, s, page = name.split("_")
+    S, page = int(s), int(page)
+    if (S, page) not in REF_BENCH_GRID:
+        raise KeyError(name)
+    seed = 3000 + S * 1000 + page
+    rng = np.random.Generator(np.random.PCG64(seed))
+    kv = rng.integers(1, 16 * page + 1, size=S)
+    q = np.array([rng.integers(1, int(k) + 1) for k in kv])
+    return make_batch(q, kv, num_q_heads=16, num_kv_heads=4, head_dim=128, page_size=page, pages_per_seq=16, seed=seed,
+                      device=device, dtype=dtype, permute_pages=False, name=name)
 
 
 def compact_for_host(batch: Batch, seq_ids) -> Batch:

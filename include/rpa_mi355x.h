@@ -97,12 +97,23 @@ typedef struct RpaParams {
   int32_t dtype;          /* RPA_DTYPE_*                                        */
   int32_t compute;        /* RPA_COMPUTE_*                                      */
 
-  /* ---- tile overrides, 0 = library default.  They carry the fields of            */
-  /*      RaggedPageAttentionConfig (modules/operations/configs.py:242-258).        */
-  int32_t num_queries_per_block;  /* query tokens per prefill tile                   */
-  int32_t num_kv_pages_per_block; /* split length of a decode sequence, in pages      */
-  int32_t num_warps;              /* wavefronts per workgroup                         */
-  int32_t num_stages;             /* reserved                                         */
+  /* ---- tile hints, 0 = library default.  They carry the fields of RaggedPageAttentionConfig                       */
+  /*      (modules/operations/configs.py:242-258), which the reference hands to its backends                        */
+  /*      (modules/operations/ragged_page_attention.py:299-318).  The library sees static, possibly padded shapes   */
+  /*      only (total_tokens and max_num_seqs are upper bounds, the lengths live on the device), so its own choice  */
+  /*      of kernel instantiation goes by those; a caller that knows its batch names the shape here.  Hints never   */
+  /*      change which rows are computed, only how the work is cut.                                                  */
+  int32_t num_queries_per_block;  /* query rows of a sequence per tile: 1..16 = the wave-level loop alone (decode     */
+                                  /* steps and short chunks; by default batches of up to 20480 (token, query head)   */
+                                  /* rows); 17..128 = 128-row workgroup tiles for long chunks; above 128 = 256-row    */
+                                  /* software-pipelined tiles where they exist (head_dim 128, no soft cap, pages of   */
+                                  /* 16 tokens or more; by default at least 128 tokens per max_num_seqs), 128-row     */
+                                  /* tiles otherwise.  RPA_FLAG_PREFILL_TILES / PIPE_TILES / PLAIN_TILES come first.  */
+  int32_t num_kv_pages_per_block; /* the least stretch of a sequence, in pages, that one streaming wavefront takes     */
+                                  /* before a small batch is spread over more wavefronts (split-K granularity;        */
+                                  /* default: 2 tiles of 32 keys, more for long sequences)                            */
+  int32_t num_warps;              /* accepted, ignored: workgroups have 4 wavefronts                                   */
+  int32_t num_stages;             /* accepted, ignored: 2 LDS stages in the 128-row tile, 4 in the pipelined one      */
   uint32_t flags;                 /* RPA_FLAG_*                                       */
 
   /* ---- quantisation scales of ragged_page_attention_v3 (_kernel.py:221-226,232-235,258-259); 0 = absent.   */

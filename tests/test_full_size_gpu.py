@@ -17,7 +17,8 @@ import torch
 from ejkernel_amd.modules import ragged_page_attention
 from ejkernel_amd.workloads import Batch, compact_for_host, make_workload
 from oracle import rpa_oracle_c
-from tests.helpers import BF16_MAX_ABS, BF16_MEAN_ABS, err_stats, oracle_args, run_exact, to_np
+from tests.helpers import (BF16_MAX_ABS, BF16_MEAN_ABS, assert_bf16_parity_stepwise, err_stats, oracle_args, run_exact,
+                           to_np)
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -83,6 +84,52 @@ def test_full_size_workload(name, n_sample, permute):
     assert (got - want).abs().max().item() <= 2.0 ** -7 * max(1.0, want.abs().max().item())
     del b, out
     torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("name,hint,n_sample", [("decode_llama3_8b", 16, 12), ("mixed_prefill_decode", 128, 14),
+                                                ("mixed_prefill_only", 256, 3)])
+def test_padded_static_shapes_with_and_without_the_config_hint(name, hint, n_sample):
+    """The same sequences, pages and queries inside the static shapes of a serving caller (max_num_seqs 512, query rows
+    rounded up to 8192 / 16384, num_seqs as is).  With RaggedPageAttentionConfig.num_queries_per_block naming the tile
+    shape the padded call runs the instantiation the unpadded call gets by default: the rows of the batch are bitwise
+    those.  Without the hint the library goes by the padded shapes (another instantiation for two of the three): the
+    sample must still meet the parity bound.  Either way every row past the batch is zero."""
+    from ejkernel_amd.modules import RaggedPageAttentionConfig
+
+    base = make_workload(name, device=DEV)
+    want = run(base)
+    total = base.total_valid_tokens
+    del base
+    torch.cuda.empty_cache()
+    b = make_workload(name + "_padded", device=DEV)
+    assert b.block_tables.shape[0] == 512 and b.queries.shape[0] in (8192, 16384) and b.total_valid_tokens == total
+    hinted = ragged_page_attention(*b.args(), cfg=RaggedPageAttentionConfig(num_queries_per_block=hint), **b.kwargs())
+    torch.cuda.synchronize()
+    assert torch.equal(hinted[:total], want[:total])
+    assert not hinted[total:].any()
+    plain = run(b)
+    assert torch.isfinite(plain.float()).all() and not plain[total:].any()
+    check_sample(b, plain, n_sample)
+    check_sample(b, hinted, n_sample)
+    del b, want, hinted, plain
+    torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("S,page", [(8, 8), (8, 128), (16, 16), (16, 64), (32, 8), (32, 32), (32, 128)])
+def test_reference_benchmark_grid_shapes(S, page):
+    """Shapes of the reference's own benchmark (max_num_seqs x page_size at 16 pages per sequence, 16 / 4 heads,
+    q_len ~ U[1, kv_len], identity block table): every row against the C restatement, on the library's choice of
+    instantiation and on the forced prefill tiles."""
+    from ejkernel_amd.modules import RaggedPageAttentionConfig
+
+    b = make_workload(f"ref_bench_{S}_{page}", device=DEV)
+    ref = rpa_oracle_c.rpa_strict_c(*oracle_args(b), softmax_scale=b.softmax_scale)
+    rows = b.total_valid_tokens
+    for hint in (None, 16, 128, 256):
+        out = ragged_page_attention(*b.args(), cfg=RaggedPageAttentionConfig(num_queries_per_block=hint), **b.kwargs())
+        torch.cuda.synchronize()
+        assert_bf16_parity_stepwise(to_np(out)[:rows], ref[:rows], f"ref_bench {S} x page {page}, hint {hint}")
+        assert not out[rows:].any()
 
 
 def test_long_prompts_on_pipelined_and_plain_tiles():
