@@ -57,8 +57,13 @@ __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
 // of rpa_prefill_pipe.h, which runs one workgroup per compute unit (one wavefront per SIMD, up to 512 registers).
 template <int D, int MRT>
 constexpr bool kPipeTile = D == 128 && MRT == 4;
-template <int D, int MRT>
-constexpr int kWavesPerSimd = kPipeTile<D, MRT> ? 1 : 2;
+// One workgroup per compute unit (one wavefront per SIMD, up to 512 registers) also for the head_dim-256 decode loop
+// over a 16-bit cache: at two wavefronts per SIMD its 256 registers spill 65 of the loop's values, and a streaming
+// batch runs one workgroup per unit anyway.
+template <int D, int MRT, bool kWaveOnly, int kKv>
+constexpr bool kWideDecode = D == 256 && kWaveOnly && kKv == 0;
+template <int D, int MRT, bool kWaveOnly, int kKv>
+constexpr int kWavesPerSimd = kPipeTile<D, MRT> || kWideDecode<D, MRT, kWaveOnly, kKv> ? 1 : 2;
 
 template <int D, int MRT, bool kMimic, int kKv, int kPass>
 __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt) {
@@ -71,7 +76,7 @@ __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, c
 }
 
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
-__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D, MRT>, kWavesPerSimd<D, MRT>)))
+__global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D, MRT, kWaveOnly, kKv>, kWavesPerSimd<D, MRT, kWaveOnly, kKv>)))
 void rpa_tile_kernel(TileArgs a) {
   constexpr int DD = D < 128 ? 128 : D;  // head_dim 64: the wave-level loop works 128 wide, prefill tiles 64 wide
   using C = Cfg<DD, NT, kMimic>;
@@ -681,7 +686,9 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     if (a.pair) a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 1);
     if (p.head_dim <= 128)
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);
-    return mimic ? launch_cfg<256, 1, 1, true, true>(a, grid, stream) : launch_cfg<256, 1, 1, false, true>(a, grid, stream);
+    // head_dim 256: one workgroup per compute unit with the whole register file
+    a.stream_grid = device_cu_count();
+    return mimic ? launch_cfg<256, 1, 1, true, true>(a, a.stream_grid, stream) : launch_cfg<256, 1, 1, false, true>(a, a.stream_grid, stream);
   }
   if (p.head_dim == 64)
     return mimic ? launch_cfg<64, 2, 4, true>(a, grid, stream) : launch_cfg<64, 2, 4, false>(a, grid, stream);
