@@ -167,8 +167,12 @@ def sm2_pack(cur: int, rg: int, s: int, k: int) -> list[str]:
     return [f"v_cvt_pk_bf16_f32 {PWE(rg, s, k)}, {SE(cur, rg, q, r)}, {SE(cur, rg, q, r + 1)}"]
 
 
-def rowsum(rg: int, s: int, k: int) -> list[str]:
-    return [f"v_dot2_f32_bf16 {LSUM(rg)}, {PWE(rg, s, k)}, {ONES2}, {LSUM(rg)}"]
+def rowsum(cur: int, rg: int, s: int, k: int) -> list[str]:
+    """Pair k of P(rg, s) joins the lane's row sum: two fp32 additions of the exponentials themselves.  (A
+    v_dot2_f32_bf16 of the packed pair against two ones is one instruction instead of two, but it issues at a quarter
+    of the rate and, reading an MFMA operand, has to wait for the MFMAs in flight: it cost 3.7 additions' time.)"""
+    q, r = 2 * s + (k >> 1), 2 * (k & 1)
+    return [f"v_add_f32 {LSUM(rg)}, {LSUM(rg)}, {SE(cur, rg, q, r)}", f"v_add_f32 {LSUM(rg)}, {LSUM(rg)}, {SE(cur, rg, q, r + 1)}"]
 
 
 def block_b(h: int) -> list[str]:
@@ -177,14 +181,14 @@ def block_b(h: int) -> list[str]:
     Rules the order obeys: the result of a transcendental instruction may not be read by the very next instruction
     (the hardware does not wait); a register written by a vector instruction may not be read by an MFMA within two
     wait states; and a vector instruction that touches a register an MFMA in flight reads waits for that MFMA, so
-    the row sums of an operand are added before its MFMAs start, not beside them."""
+    the row sums read the exponentials, not the packed operand."""
     cur = 0 if h == 0 else 32
     groups = [(rg, s) for rg in range(NRG) for s in range(2)]
     out = kload(h) + ["s_waitcnt lgkmcnt(8)"]
     rg, s = groups[0]
-    out += sm2_exp(cur, rg, s, 0) + sm2_exp(cur, rg, s, 1) + sm2_pack(cur, rg, s, 0) + sm2_exp(cur, rg, s, 2) + sm2_pack(cur, rg, s, 1)
-    out += rowsum(rg, s, 0) + sm2_exp(cur, rg, s, 3) + sm2_pack(cur, rg, s, 2) + rowsum(rg, s, 1) + sm2_pack(cur, rg, s, 3)
-    out += rowsum(rg, s, 2) + rowsum(rg, s, 3)
+    out += sm2_exp(cur, rg, s, 0) + sm2_exp(cur, rg, s, 1) + sm2_pack(cur, rg, s, 0) + rowsum(cur, rg, s, 0)
+    out += sm2_exp(cur, rg, s, 2) + sm2_pack(cur, rg, s, 1) + rowsum(cur, rg, s, 1)
+    out += sm2_exp(cur, rg, s, 3) + sm2_pack(cur, rg, s, 2) + rowsum(cur, rg, s, 2) + sm2_pack(cur, rg, s, 3) + rowsum(cur, rg, s, 3)
     for gi, (rg, s) in enumerate(groups):
         nx = groups[gi + 1] if gi + 1 < len(groups) else None
         for blk in range(NBLK):
@@ -192,12 +196,10 @@ def block_b(h: int) -> list[str]:
             if nx is None:
                 continue
             out += sm2_exp(cur, nx[0], nx[1], blk)
-            if blk == 1:
-                out += sm2_pack(cur, *nx, 0)
-            if blk == 2:
-                out += sm2_pack(cur, *nx, 1) + rowsum(*nx, 0)
+            if blk >= 1:
+                out += sm2_pack(cur, *nx, blk - 1) + rowsum(cur, *nx, blk - 1)
             if blk == 3:
-                out += sm2_pack(cur, *nx, 2) + rowsum(*nx, 1) + sm2_pack(cur, *nx, 3) + rowsum(*nx, 2) + rowsum(*nx, 3)
+                out += sm2_pack(cur, *nx, 3) + rowsum(cur, *nx, 3)
     return out
 
 

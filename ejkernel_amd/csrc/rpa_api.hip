@@ -127,10 +127,13 @@ static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static std::mutex g_scratch_mu;
 static std::atomic<void*> g_scratch_ptr[64];  // per device; null until the first call there
 
-// Address of this device's copy of `scratch`; the first call on a device looks it up and clears the ticket region
-// (the loader zero-fills the array and every launch leaves the tickets at zero again, so this is belt and braces for
-// a process that aborted a launch half way).  Enqueue-only, no allocation.
-static int static_scratch(hipStream_t stream, void** out) {
+// Address of this device's copy of `scratch`; the first call on a device looks it up.  Nothing is enqueued: the
+// tickets and queue counters at the head of the array are zero when the code object is loaded (a zero-initialised
+// device variable) and every launch leaves them at zero again, and no other part of the array needs an initial
+// value (a partial state is written before the ticket that publishes it).  So a first call made under stream capture
+// records the attention kernel and nothing else, and first calls on two streams cannot reset each other's tickets.
+// The lookup itself may load the code object: make the first call on a device outside any capture.
+static int static_scratch(void** out) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return fail(RPA_ERR_LAUNCH, "hipGetDevice failed or device index above 63");
   void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
@@ -141,9 +144,6 @@ static int static_scratch(hipStream_t stream, void** out) {
       const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
       if (e != hipSuccess || p == nullptr)
         return fail(RPA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
-      hipLaunchKernelGGL(zero_fill_kernel, dim3(64), dim3(256), 0, stream, static_cast<uint4*>(p),
-                         static_cast<size_t>(kWorkspaceTicketBytes / 16));
-      if (hipGetLastError() != hipSuccess) return fail(RPA_ERR_LAUNCH, "clearing the static scratch tickets failed");
       g_scratch_ptr[dev].store(p, std::memory_order_release);
     }
   }
@@ -170,7 +170,7 @@ int rpa_fwd_launch_static(const RpaParams* params, void* hip_stream) {
                        "use rpa_fwd_launch with a workspace",
                        (unsigned long long)need, (unsigned long long)rpa::kStaticScratchBytes);
     void* ptr = nullptr;
-    rc = rpa::static_scratch(static_cast<hipStream_t>(hip_stream), &ptr);
+    rc = rpa::static_scratch(&ptr);
     if (rc != RPA_OK) return rc;
     p.workspace = ptr;
     p.workspace_bytes = rpa::kStaticScratchBytes;

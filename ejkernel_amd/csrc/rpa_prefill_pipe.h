@@ -64,6 +64,7 @@ struct PipeCfg {
 
 typedef __attribute__((ext_vector_type(32))) float f32x32_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(2))) float f32x2_t;
 typedef __attribute__((ext_vector_type(4))) int i32x4_t;
 typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 
@@ -73,8 +74,8 @@ typedef __attribute__((ext_vector_type(8))) int i32x8_t;
 // (register map in gen_prefill_pipe_asm.py).
 struct PipeIo {
   f32x32_t o0, o1, o2, o3;  // out: O^T accumulators, row group 0 blocks 0-1, 2-3, row group 1 blocks 0-1, 2-3
-  f32x4_t lsum;             // out: row sums of the lane's keys per row group ([0], [1])
-  f32x4_t mneg, mthr;       // out: exp2 offset and threshold per row group ([0], [1])
+  f32x2_t lsum;             // out: row sums of the lane's keys per row group ([0], [1])
+  f32x2_t mneg, mthr;       // out: exp2 offset and threshold per row group ([0], [1])
   f32x32_t q0, q1;          // in: Q operands of row group 0, 1
   i32x4_t mspan, rowlo;     // in: per-lane bounds of the visible keys per row group ([0], [1])
   i32x4_t kbase0, kbase1;   // in: LDS addresses of the K operand reads per k-step
@@ -118,8 +119,8 @@ struct PipeIo {
 template <bool kRound>
 __device__ __forceinline__ void pipe_key_loop(PipeIo& R) {
 #define RPA_PPA_OPERANDS                                                                                                  \
-  : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={v[144:147]}"(R.lsum),       \
-    "={v[148:151]}"(R.mneg), "={v[172:175]}"(R.mthr) RPA_PPA_PROF_OUT                                                  \
+  : "={a[0:31]}"(R.o0), "={a[32:63]}"(R.o1), "={a[64:95]}"(R.o2), "={a[96:127]}"(R.o3), "={v[144:145]}"(R.lsum),       \
+    "={v[148:149]}"(R.mneg), "={v[172:173]}"(R.mthr) RPA_PPA_PROF_OUT                                                  \
   : "{v[64:95]}"(R.q0), "{v[96:127]}"(R.q1), "{v[160:163]}"(R.mspan), "{v[178:181]}"(R.rowlo), "{v[224:227]}"(R.kbase0), \
     "{v[228:231]}"(R.kbase1), "{v[186:189]}"(R.misc), "{v[190:193]}"(R.kpiece), "{v169}"(R.cfac), "{s[36:43]}"(R.s0),   \
     "{s[44:51]}"(R.s1)                                                                                                 \

@@ -176,7 +176,9 @@ int rpa_fwd_launch(const RpaParams* params, void* hip_stream);
  * call allocates and frees nothing and never synchronises; results are those of rpa_fwd_launch, bit for bit.
  * Shapes whose rpa_workspace_bytes() exceeds the array are rejected with RPA_ERR_WORKSPACE (head_dim 256 on the
  * MFMA kernel, today).  All calls on one GPU share that GPU's array: calls that overlap in time on one GPU, on
- * whatever streams, race -- serialise them (one stream, or events between streams).
+ * whatever streams, race -- serialise them (one stream, or events between streams).  The call may be captured in a
+ * HIP graph (it records the attention kernel and nothing else); make the first call on a device outside any capture,
+ * since looking up the array's address may load the library's code object.
  */
 uint64_t rpa_static_scratch_bytes(void);
 int rpa_fwd_launch_static(const RpaParams* params, void* hip_stream);

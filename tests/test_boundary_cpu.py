@@ -271,6 +271,53 @@ def test_generated_instruction_stream_is_up_to_date():
     assert (csrc / "rpa_prefill_pipe_asm.inc").read_text() == gen.render()
 
 
+def _regs(tok):
+    """Registers an assembler operand names: 'v[4:7]' -> {v4..v7}, 'a12' -> {a12}, anything else -> {}."""
+    m = re.fullmatch(r"([vas])\[(\d+):(\d+)\]", tok)
+    if m:
+        return {f"{m.group(1)}{k}" for k in range(int(m.group(2)), int(m.group(3)) + 1)}
+    m = re.fullmatch(r"([vas])(\d+)", tok)
+    return {tok} if m else set()
+
+
+def test_instruction_stream_writes_only_what_its_constraints_declare():
+    """The generated key loop is one asm statement with physical-register operands.  Every register an instruction of
+    the stream writes must be an output or a clobber of that statement, none may be an input (the compiler assumes
+    inputs survive), and no register is both output and clobber.  m0 is saved and restored by the stream itself."""
+    csrc = Path(_native.__file__).resolve().parent / "csrc"
+    inc = (csrc / "rpa_prefill_pipe_asm.inc").read_text()
+    hdr = (csrc / "rpa_prefill_pipe.h").read_text()
+    ops = hdr[hdr.index("#define RPA_PPA_OPERANDS"):hdr.index("if constexpr (kRound) asm volatile")]
+    outs_txt, ins_txt = ops.split("\n  : ")[1], ops.split("\n  : ")[2]
+    outputs = set().union(*[_regs(t) for t in re.findall(r'"=\{([^}]+)\}"', outs_txt)])
+    inputs = set().union(*[_regs(t) for t in re.findall(r'"\{([^}]+)\}"', ins_txt)])
+    clob_txt = hdr[hdr.index("#define RPA_PPA_CLOBBERS"):hdr.index("// The key loop of one tile for one wavefront.")]
+    clobbers = set(re.findall(r'"([vas]\d+)"', clob_txt))
+    assert len(outputs) == 128 + 6 and len(inputs) >= 64 + 8
+    assert not (outputs & clobbers), sorted(outputs & clobbers)
+    assert not (outputs & inputs) and not (inputs & clobbers), sorted(inputs & clobbers)
+    no_dest = ("s_waitcnt", "s_barrier", "s_nop", "s_branch", "s_cbranch", "s_cmp", "buffer_load", "s_setprio", "s_sleep")
+    written = set()
+    for line in re.findall(r'"([^"\\]+)\\n\\t"', inc):
+        line = line.strip()
+        if not line or line.endswith(":") or line.startswith(no_dest):
+            continue
+        mnem, _, rest = line.partition(" ")
+        toks = [t.strip() for t in rest.split(",")]
+        if mnem.startswith("v_cmp"):
+            dst = toks[:1] if toks[0] != "vcc" else []   # a scalar pair or vcc
+        elif mnem.startswith("v_permlane32_swap") or mnem.startswith("v_permlane16_swap"):
+            dst = toks[:2]
+        else:
+            dst = toks[:1]
+        for t in dst:
+            written |= _regs(t)
+    assert written, "no instruction parsed"
+    undeclared = written - outputs - clobbers
+    assert not undeclared, f"written but neither output nor clobber: {sorted(undeclared)}"
+    assert not (written & inputs), f"inputs written by the stream: {sorted(written & inputs)}"
+
+
 def test_hbm_traffic_file_is_well_formed():
     """profiles/hbm_traffic.json (read by bench.py for roofline.traffic): bytes = scaled counters, per workload."""
     import json

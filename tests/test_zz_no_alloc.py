@@ -70,3 +70,46 @@ def test_static_scratch_rejects_what_does_not_fit():
     # the scalar kernel needs no scratch at all
     g = run(b, True, _native.RPA_FLAG_FORCE_GENERIC)
     assert torch.equal(g, run(b, False, _native.RPA_FLAG_FORCE_GENERIC))
+
+
+def test_static_entry_point_allocates_nothing_and_replays_from_a_hip_graph():
+    """What the entry point is for: a call under HIP graph capture, where nothing may allocate.  After one eager call
+    (the first call on a device looks up the scratch array's address) the call is captured, replayed on new queries
+    three times with eager work in between, and every replay must equal the eager result of the workspace entry
+    point bit for bit.  Across the C call itself neither torch's allocator nor the device's free memory moves."""
+    import ctypes
+
+    b = make_batch([1, 1, 1, 3], [9000, 300, 5000, 64], num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16,
+                   pages_per_seq=640, seed=41, device=DEV)
+    out = torch.zeros_like(b.queries)
+    kw = dict(softmax_scale=b.softmax_scale, cfg=RaggedPageAttentionConfig(), _out=out, _static_scratch=True)
+    RaggedPageAttention().run(*b.args(), **kw)   # first call on the device: outside capture
+    torch.cuda.synchronize()
+    hip = ctypes.CDLL("libamdhip64.so")
+    free0, total = ctypes.c_size_t(), ctypes.c_size_t()
+    free1 = ctypes.c_size_t()
+    assert hip.hipMemGetInfo(ctypes.byref(free0), ctypes.byref(total)) == 0
+    allocated, reserved = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    RaggedPageAttention().run(*b.args(), **kw)
+    torch.cuda.synchronize()
+    assert hip.hipMemGetInfo(ctypes.byref(free1), ctypes.byref(total)) == 0
+    assert free1.value == free0.value, "device memory moved across rpa_fwd_launch_static"
+    assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (allocated, reserved)
+
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            RaggedPageAttention().run(*b.args(), **kw)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    gen = torch.Generator(device=DEV).manual_seed(5)
+    for k in range(3):
+        b.queries[: b.total_valid_tokens] = torch.randn(b.total_valid_tokens, 8, 128, device=DEV, generator=gen).to(torch.bfloat16)
+        out.fill_(3.0)
+        g.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        want = run(b, False)   # eager, workspace entry point, allocations and synchronisation between the replays
+        assert torch.equal(got, want), f"replay {k} differs from the eager result"
