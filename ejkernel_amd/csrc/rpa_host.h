@@ -79,9 +79,12 @@ inline int sched_shift_for(int max_num_seqs) {
 constexpr int kTiledMaxWgsPerCu = 4;        // persistent grid = compute units x this, at most
 
 constexpr uint64_t kWorkspaceTicketBytes = 1u << 20;  // head of the workspace, cleared by rpa_workspace_init
-// The last 16 words of the ticket region hold the prefill queue counters (8 queues, 1 exit count); the split
-// tickets, one word per (sequence, kv head), lie below them.
-constexpr uint32_t kQueueCounterIndex = (1u << 20) / 4 - 16;
+// The last 512 words of the ticket region hold the counters of the prefill queues, each in a 64-byte line of its
+// own (counters that share a line queue up behind each other where the atomics execute): the ticket counter of queue
+// x at word 16 x, the count of XCDs whose workgroups have all left at word 128, and at word 144 + 16 x the count of
+// workgroups of XCD x that have left.  The split tickets, one word per (sequence, kv head), lie below them.
+constexpr uint32_t kQueueCounterIndex = (1u << 20) / 4 - 512;
+constexpr uint32_t kQueueStride = 16, kQueueExitIndex = 128, kQueueXcdExitIndex = 144;
 
 struct WorkspaceLayout {
   uint64_t counters_bytes;                   // split tickets at offset 0

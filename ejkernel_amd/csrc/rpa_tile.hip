@@ -296,25 +296,63 @@ void rpa_tile_kernel(TileArgs a) {
         // workgroup draws from the queue of its own XCD until that is empty, then from the others.  Within a
         // (sequence, kv head) the late causal tiles (most keys) come first.  The last workgroup to find every
         // queue empty clears the counters for the next launch.
+        // Atomics on one word execute one after the other where the XCDs' memory paths meet, a hundred workgroups
+        // asking at the same moment wait tens of microseconds, and a batch of a few tiles is all such moments.  So
+        // the workgroups that begin with the prefill tiles own the first tickets of their home queue without asking
+        // (workgroup b: ticket b / 8), the counters hand out the tickets after those, and a workgroup that leaves
+        // its home queue reads all eight counters at once (plain loads, which do not queue up) and asks only where
+        // the count says items are left.
         uint32_t* qctr = a.counters + kQueueCounterIndex;
         const int home = blockIdx.x & 7;
+        const int n_first = split && (total_tiles > 0 || total_items > 0) ? a.decode_grid : grid_all;  // begin with tiles
+        auto owned = [&](int x) { return n_first > x ? (n_first - x + 7) >> 3 : 0; };    // ... and have home queue x
+        // items of queue x: its full runs (run r belongs to queue r % 8) and the partial last run if it is x's
+        auto items_of = [&](int x) {
+          const int runs = total_wg / kQueueRun, rem = total_wg - runs * kQueueRun;
+          return (runs > x ? (runs - x + 7) >> 3 : 0) * kQueueRun + ((runs & 7) == x ? rem : 0);
+        };
         int probe = 0;
+        bool first = static_cast<int>(blockIdx.x) < n_first;
         while (true) {
-          int w = -1;
-          while (probe < 8) {
-            const int x = (home + probe) & 7;
-            if (tid == 0)
-              scratch[0] = static_cast<int>(__hip_atomic_fetch_add(&qctr[x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-            __syncthreads();
-            const int t = __builtin_amdgcn_readfirstlane(scratch[0]);
-            __syncthreads();
-            const int cand = ((t / kQueueRun) * 8 + x) * kQueueRun + t % kQueueRun;
-            if (cand < total_wg) {
-              w = cand;
-              break;
+          // counters of the queues in this workgroup's order, read when the home queue is known to be empty
+          uint32_t left = 0;  // bit k: the k-th queue in this workgroup's order has items left by its counter
+          if (probe > 0 && wave == 0) {
+            const int lane = tid & (kWave - 1);
+            const int seen = static_cast<int>(__hip_atomic_load(&qctr[kQueueStride * ((home + (lane & 7)) & 7)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+              const int x = (home + k) & 7;
+              if (__builtin_amdgcn_readlane(seen, k) + owned(x) < items_of(x)) left |= 1u << k;
             }
-            ++probe;
           }
+          if (tid == 0) {
+            int res = -1;
+            while (probe < 8) {
+              const int x = (home + probe) & 7;
+              int t = -1;
+              if (first) {
+                t = static_cast<int>(blockIdx.x) >> 3;
+              } else if (probe == 0 || ((left >> probe) & 1u) != 0) {
+                t = owned(x) + static_cast<int>(__hip_atomic_fetch_add(&qctr[kQueueStride * x], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+              }
+              first = false;
+              if (t >= 0) {
+                const int cand = ((t / kQueueRun) * 8 + x) * kQueueRun + t % kQueueRun;
+                if (cand < total_wg) {
+                  res = cand;
+                  break;
+                }
+              }
+              ++probe;
+            }
+            scratch[0] = res;
+            scratch[1] = probe;
+          }
+          first = false;
+          __syncthreads();
+          const int w = __builtin_amdgcn_readfirstlane(scratch[0]);
+          probe = __builtin_amdgcn_readfirstlane(scratch[1]);
+          __syncthreads();
           if (w < 0) break;
           int s_base, s;
           if (n_sorted > 0) {
@@ -349,10 +387,22 @@ void rpa_tile_kernel(TileArgs a) {
           }
           run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, n_qt - 1 - member);
         }
+        // The last workgroup out clears the counters for the next launch; the exit counts are kept per XCD and
+        // then over the XCDs, so that the workgroups of a small batch, which all leave at once, do not queue up on one word.
         if (tid == 0) {
-          const uint32_t done = __hip_atomic_fetch_add(&qctr[8], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (done == static_cast<uint32_t>(grid_all) - 1)
-            for (int i = 0; i < 9; ++i) __hip_atomic_store(&qctr[i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const uint32_t n_home = (static_cast<uint32_t>(grid_all) - home + 7) >> 3;  // workgroups b with b % 8 == home
+          const uint32_t gone = __hip_atomic_fetch_add(&qctr[kQueueXcdExitIndex + kQueueStride * home], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (gone == n_home - 1) {
+            const uint32_t n_groups = static_cast<uint32_t>(min(grid_all, 8));
+            const uint32_t done = __hip_atomic_fetch_add(&qctr[kQueueExitIndex], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (done == n_groups - 1) {
+              for (int i = 0; i < 8; ++i) {
+                __hip_atomic_store(&qctr[kQueueStride * i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(&qctr[kQueueXcdExitIndex + kQueueStride * i], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+              }
+              __hip_atomic_store(&qctr[kQueueExitIndex], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+          }
         }
       } else {
         // Static split: numbering the workgroups XCD by XCD keeps the row tiles of one K/V stream on one XCD; within
