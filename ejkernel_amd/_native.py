@@ -27,6 +27,7 @@ EXPORTED_SYMBOLS = (
     "rpa_abi_version",
     "rpa_last_error",
     "rpa_workspace_bytes",
+    "rpa_kernel_path",
     "rpa_workspace_init",
     "rpa_fwd_launch",
     "rpa_fwd_launch_static",
@@ -182,6 +183,8 @@ def load() -> ctypes.CDLL:
     lib.rpa_last_error.argtypes = []
     lib.rpa_workspace_bytes.restype = ctypes.c_uint64
     lib.rpa_workspace_bytes.argtypes = [ctypes.POINTER(RpaParams)]
+    lib.rpa_kernel_path.restype = ctypes.c_int
+    lib.rpa_kernel_path.argtypes = [ctypes.POINTER(RpaParams)]
     lib.rpa_workspace_init.restype = ctypes.c_int
     lib.rpa_workspace_init.argtypes = [ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     lib.rpa_fwd_launch.restype = ctypes.c_int

@@ -95,6 +95,11 @@ uint64_t rpa_workspace_bytes(const RpaParams* dims) {
   return wl.total_bytes;
 }
 
+int rpa_kernel_path(const RpaParams* dims) {
+  if (dims == nullptr || rpa::validate(*dims, false) != RPA_OK) return -1;
+  return rpa::tiled_supported(*dims) ? 1 : 0;
+}
+
 int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stream) {
   // Only the split tickets need a defined value; they sit at the head of the workspace and every launch
   // leaves them at zero again.

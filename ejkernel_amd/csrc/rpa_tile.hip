@@ -147,6 +147,32 @@ void rpa_tile_kernel(TileArgs a) {
   }
   __syncthreads();
 
+  // ---- two launches, one call (TileArgs::select).  The 128-row tiles run beside a streaming workgroup on every
+  // compute unit and win where the decode stream sets the time; the pipelined tiles own their units and win where
+  // the prefill work does (16 chunks of 512 tokens beside 64 decode sequences: 0.45 against 0.53 ms; beside 240:
+  // 1.08 against 0.92 ms).  The host sees padded shapes only, so where it cannot tell it enqueues both kernels and
+  // every workgroup of both decides here, from the same sums: prefill work in units of 1024 (query row, key) pairs
+  // against the stream's tiles of 32 keys -- 0.6 ns against 3 ns apiece at the rates the two kernels reach, and the
+  // pipelined tiles are worth it from seven tenths of the stream's time on.
+  if constexpr (!kWaveOnly && kKv == 0) {
+    if (a.select != 0) {
+      int my_cost = 0;
+      for (int s = s_begin; s < s_end; ++s) {
+        const SeqInfo si = seq_info<C::TT>(a, s, G);
+        if (!si.eligible && si.n_rt > kWaveItemMaxRowTiles) {
+          const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
+          my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
+        }
+      }
+      int total_cost;
+      block_excl_scan(my_cost, scratch, total_cost);
+      total_cost = __builtin_amdgcn_readfirstlane(total_cost);
+      const bool pick_pipe = 10ll * total_cost >= 35ll * total_tiles;
+      __syncthreads();
+      if ((a.select == 2) != pick_pipe) return;
+    }
+  }
+
   // ---- prefill order.  Tiles are drawn from the queues in item order and a tile's cost grows with the number of
   // keys it can see, so the longest sequences go first (as in longest-processing-time-first scheduling: the work left
   // for the end is the short tiles).  wg_start is rebuilt over the sequences that have prefill tiles, by descending
@@ -522,6 +548,7 @@ struct Tune {
   int pipe_stream_wgs;     // RPA_TUNE_PIPE_STREAM_WGS: workgroups (of one per compute unit) that take the decode stream first
   int pipe_min_tokens_per_seq;  // RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ: average query tokens per sequence from which it is used
   int no_logit_stash;      // RPA_TUNE_NO_LOGIT_STASH: two-launch calls read K in both launches (experiments)
+  int device_select;       // RPA_TUNE_DEVICE_SELECT: 0 = never enqueue both tile kernels and let the device pick
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -544,6 +571,7 @@ static const Tune& tune() {
     x.pipe_min_tokens_per_seq = max(1, env_int("RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ", 128));
     x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
     x.no_logit_stash = env_int("RPA_TUNE_NO_LOGIT_STASH", 0);
+    x.device_select = env_int("RPA_TUNE_DEVICE_SELECT", 1);
     return x;
   }();
   return t;
@@ -683,6 +711,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.uniform_page = p.page_size >= 16;
   a.phase_mode = tune().phase_mode;
   a.pair = 0;
+  a.select = 0;
   a.even_xcd_permille = tune().even_xcd_permille;
   // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
   // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes
@@ -754,6 +783,20 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     const bool pipe_wanted = pipe_choice > 0 ||
                              (pipe_choice == 0 && tune().pipe != 0 &&
                               static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs);
+    // Neither flag nor hint, and the static shapes do not say "long chunks": the batch may still be one (a serving
+    // caller pads total_tokens and max_num_seqs), so both kernels are enqueued and the device picks (TileArgs::select).
+    // The launch that is not picked builds the schedule and ends: a few microseconds.
+    if (pipe_choice == 0 && !pipe_wanted && pipe_ok && canonical && tune().pipe != 0 && tune().device_select != 0) {
+      TileArgs b = a;
+      a.select = 1;
+      int rc = mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
+      if (rc != RPA_OK) return rc;
+      const int g1 = device_cu_count();
+      b.select = 2;
+      b.stream_grid = g1;
+      b.decode_grid = max(0, g1 - tune().pipe_stream_wgs);
+      return mimic ? launch_cfg<128, 2, 4, true>(b, g1, stream) : launch_cfg<128, 2, 4, false>(b, g1, stream);
+    }
     if (pipe_wanted && pipe_ok && canonical) {
       // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
       // number on every XCD) take the decode stream first and join the prefill queues when it is done

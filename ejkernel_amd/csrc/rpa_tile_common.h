@@ -44,6 +44,11 @@ struct TileArgs {
   // rows of the first head zero in the second half of the contraction and vice versa; every row keeps the half of the
   // output that belongs to its head.
   int pair;
+  // Which of two launches of one call does the work, decided on the device, where the lengths are: 0 = this launch
+  // (the host has decided), 1 = this launch holds the 128-row prefill tiles, 2 = this one the pipelined 256-row
+  // tiles.  With 1 or 2 every workgroup weighs the batch's prefill work against its decode stream the same way and
+  // the launch that is not picked ends there.
+  int select;
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the

@@ -6,29 +6,26 @@
 // ejkernel_amd/jax_ffi.py only where JAX is installed and is not part of the default build.
 //
 // Handlers (operands | results | attributes):
-//   RpaFwd           queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs [, sinks] | out |
+//   RpaFwd           queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs [, sinks] | out, scratch |
 //                    softmax_scale f32, logits_soft_cap f32 (0 = none), sliding_window i32 (0 = none), compute i32,
 //                    num_queries_per_block, num_kv_pages_per_block, num_warps, num_stages i32
 //   RpaV3            queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution |
 //                    out, kv_cache (the caller aliases it to operand 3: the reference donates the cache,
-//                    ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:110-126) |
+//                    ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:110-126), scratch |
 //                    softmax_scale, logits_soft_cap, q_scale, k_scale, v_scale f32 (0 = none), sliding_window i32
-//   RpaPageAttn      query, key_cache, value_cache, context_lens, block_tables | out | attn_scale f32
-//   RpaRaggedDecode  query, key, value, sequence_start, sequence_end [, softmax_aux] | out |
+//   RpaPageAttn      query, key_cache, value_cache, context_lens, block_tables | out, scratch | attn_scale f32
+//   RpaRaggedDecode  query, key, value, sequence_start, sequence_end [, softmax_aux] | out, scratch |
 //                    softmax_scale, logits_soft_cap f32, window_left i32 (< 0 = none)
 //
-// Scratch memory: XLA's result buffers are uninitialised and reused for other values between calls, so a workspace
-// handed out by XLA would have to be cleared before every launch.  The handlers keep one workspace per (device,
-// stream) instead, allocated and cleared on the first call there and grown when a shape needs more; launches on
-// one stream are ordered, so they never share a workspace in time.  The first call on a stream allocates: the
-// handlers are not registered as command-buffer compatible.
+// Scratch memory: every handler has one more result than its op, a byte buffer of the size the matching
+// rpa_*_workspace_bytes function names (the Python wrapper declares it and drops it), so XLA owns and places the
+// scratch and a handler allocates nothing, frees nothing and never synchronises: it enqueues the kernel that clears
+// the ticket region (XLA's buffers arrive uninitialised and are reused between calls) and then the op, on the stream
+// XLA hands over.  That is all a command buffer capture may contain.
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
-#include <map>
-#include <mutex>
 #include <string>
-#include <utility>
 
 #include "../../include/rpa_mi355x.h"
 #include "xla/ffi/api/ffi.h"
@@ -39,29 +36,15 @@ static ffi::Error Invalid(const std::string& msg) { return ffi::Error(ffi::Error
 static ffi::Error Failed(const std::string& msg) { return ffi::Error(ffi::ErrorCode::kInternal, msg); }
 
 namespace {
-struct Workspace {
-  void* ptr = nullptr;
-  uint64_t bytes = 0;
-};
-std::mutex g_mu;
-std::map<std::pair<int, hipStream_t>, Workspace> g_workspaces;
-
-// The workspace of this device and stream with at least `bytes` bytes, its tickets zero.
-ffi::Error StreamWorkspace(hipStream_t stream, uint64_t bytes, void** out) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess) return Failed("hipGetDevice failed");
-  std::lock_guard<std::mutex> lock(g_mu);
-  Workspace& w = g_workspaces[{dev, stream}];
-  if (w.bytes < bytes) {
-    if (w.ptr != nullptr) {
-      if (hipStreamSynchronize(stream) != hipSuccess || hipFree(w.ptr) != hipSuccess) return Failed("releasing the old workspace failed");
-      w = Workspace();
-    }
-    if (hipMalloc(&w.ptr, bytes) != hipSuccess) return Failed("hipMalloc of the attention workspace failed");
-    w.bytes = bytes;
-    if (rpa_workspace_init(w.ptr, w.bytes, stream) != RPA_OK) return Failed(rpa_last_error());
-  }
-  *out = w.ptr;
+// Points the launch at the scratch result and clears its tickets on the stream.
+ffi::Error UseScratch(hipStream_t stream, ffi::Result<ffi::AnyBuffer>& scratch, uint64_t need, void** workspace,
+                      uint64_t* workspace_bytes) {
+  const uint64_t have = static_cast<uint64_t>(scratch->size_bytes());
+  if (have < need) return Invalid("the scratch result is smaller than the op's workspace (declare rpa_*_workspace_bytes bytes)");
+  if ((reinterpret_cast<uintptr_t>(scratch->untyped_data()) & 255u) != 0) return Invalid("the scratch result is not 256-byte aligned");
+  if (rpa_workspace_init(scratch->untyped_data(), have, stream) != RPA_OK) return Failed(rpa_last_error());
+  *workspace = scratch->untyped_data();
+  *workspace_bytes = have;
   return ffi::Error::Success();
 }
 
@@ -78,8 +61,8 @@ int DtypeOf(ffi::DataType t) {
 static ffi::Error RpaFwdImpl(hipStream_t stream, ffi::AnyBuffer queries, ffi::AnyBuffer kv_pages,
                              ffi::Buffer<ffi::S32> context_lens, ffi::Buffer<ffi::S32> block_tables,
                              ffi::Buffer<ffi::S32> query_start_loc, ffi::Buffer<ffi::S32> num_seqs,
-                             ffi::RemainingArgs rest, ffi::Result<ffi::AnyBuffer> out, float softmax_scale,
-                             float logits_soft_cap, int32_t sliding_window, int32_t compute,
+                             ffi::RemainingArgs rest, ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> scratch,
+                             float softmax_scale, float logits_soft_cap, int32_t sliding_window, int32_t compute,
                              int32_t num_queries_per_block, int32_t num_kv_pages_per_block, int32_t num_warps,
                              int32_t num_stages) {
   const auto qd = queries.dimensions();
@@ -119,8 +102,7 @@ static ffi::Error RpaFwdImpl(hipStream_t stream, ffi::AnyBuffer queries, ffi::An
   p.num_kv_pages_per_block = num_kv_pages_per_block;
   p.num_warps = num_warps;
   p.num_stages = num_stages;
-  p.workspace_bytes = rpa_workspace_bytes(&p);
-  if (ffi::Error e = StreamWorkspace(stream, p.workspace_bytes, &p.workspace); e.failure()) return e;
+  if (ffi::Error e = UseScratch(stream, scratch, rpa_workspace_bytes(&p), &p.workspace, &p.workspace_bytes); e.failure()) return e;
   if (rpa_fwd_launch(&p, stream) != RPA_OK) return Invalid(rpa_last_error());
   return ffi::Error::Success();
 }
@@ -136,6 +118,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaFwd, RpaFwdImpl,
                                   .Arg<ffi::Buffer<ffi::S32>>()   // num_seqs
                                   .RemainingArgs()                // [sinks]
                                   .Ret<ffi::AnyBuffer>()          // out
+                                  .Ret<ffi::AnyBuffer>()          // scratch
                                   .Attr<float>("softmax_scale")
                                   .Attr<float>("logits_soft_cap")
                                   .Attr<int32_t>("sliding_window")
@@ -149,8 +132,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaFwd, RpaFwdImpl,
 static ffi::Error RpaV3Impl(hipStream_t stream, ffi::AnyBuffer queries, ffi::AnyBuffer keys, ffi::AnyBuffer values,
                             ffi::AnyBuffer kv_cache, ffi::Buffer<ffi::S32> kv_lens, ffi::Buffer<ffi::S32> block_tables,
                             ffi::Buffer<ffi::S32> query_start_loc, ffi::Buffer<ffi::S32> distribution,
-                            ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> cache_out, float softmax_scale,
-                            float logits_soft_cap, float q_scale, float k_scale, float v_scale, int32_t sliding_window) {
+                            ffi::Result<ffi::AnyBuffer> out, ffi::Result<ffi::AnyBuffer> cache_out,
+                            ffi::Result<ffi::AnyBuffer> scratch, float softmax_scale, float logits_soft_cap, float q_scale, float k_scale, float v_scale, int32_t sliding_window) {
   const auto qd = queries.dimensions();
   const auto kd = keys.dimensions();
   const auto cd = kv_cache.dimensions();  // [pages, page_size, 2 * kv heads / packing, packing, aligned head_dim]
@@ -194,8 +177,7 @@ static ffi::Error RpaV3Impl(hipStream_t stream, ffi::AnyBuffer queries, ffi::Any
   v.new_values = values.untyped_data();
   v.cache_head_dim = static_cast<int32_t>(cd[4]);
   v.cache_combined_heads = static_cast<int32_t>(cd[2] * cd[3]);
-  p.workspace_bytes = rpa_v3_workspace_bytes(&v);
-  if (ffi::Error e = StreamWorkspace(stream, p.workspace_bytes, &p.workspace); e.failure()) return e;
+  if (ffi::Error e = UseScratch(stream, scratch, rpa_v3_workspace_bytes(&v), &p.workspace, &p.workspace_bytes); e.failure()) return e;
   if (rpa_v3_launch(&v, stream) != RPA_OK) return Invalid(rpa_last_error());
   return ffi::Error::Success();
 }
@@ -213,6 +195,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaV3, RpaV3Impl,
                                   .Arg<ffi::Buffer<ffi::S32>>()   // distribution
                                   .Ret<ffi::AnyBuffer>()          // out
                                   .Ret<ffi::AnyBuffer>()          // kv_cache, aliased to operand 3
+                                  .Ret<ffi::AnyBuffer>()          // scratch
                                   .Attr<float>("softmax_scale")
                                   .Attr<float>("logits_soft_cap")
                                   .Attr<float>("q_scale")
@@ -223,7 +206,8 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaV3, RpaV3Impl,
 // ------------------------------------------------------------------------------------------------------ page_attention
 static ffi::Error RpaPageAttnImpl(hipStream_t stream, ffi::AnyBuffer query, ffi::AnyBuffer key_cache,
                                   ffi::AnyBuffer value_cache, ffi::Buffer<ffi::S32> context_lens,
-                                  ffi::Buffer<ffi::S32> block_tables, ffi::Result<ffi::AnyBuffer> out, float attn_scale) {
+                                  ffi::Buffer<ffi::S32> block_tables, ffi::Result<ffi::AnyBuffer> out,
+                                  ffi::Result<ffi::AnyBuffer> scratch, float attn_scale) {
   const auto qd = query.dimensions();
   const auto kd = key_cache.dimensions();
   const auto bd = block_tables.dimensions();
@@ -246,8 +230,7 @@ static ffi::Error RpaPageAttnImpl(hipStream_t stream, ffi::AnyBuffer query, ffi:
   p.block_size = static_cast<int32_t>(kd[2]);
   p.max_blocks = static_cast<int32_t>(bd[1]);
   p.attn_scale = attn_scale;
-  p.workspace_bytes = rpa_page_attention_workspace_bytes(&p);
-  if (ffi::Error e = StreamWorkspace(stream, p.workspace_bytes, &p.workspace); e.failure()) return e;
+  if (ffi::Error e = UseScratch(stream, scratch, rpa_page_attention_workspace_bytes(&p), &p.workspace, &p.workspace_bytes); e.failure()) return e;
   if (rpa_page_attention_launch(&p, stream) != RPA_OK) return Invalid(rpa_last_error());
   return ffi::Error::Success();
 }
@@ -261,13 +244,15 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaPageAttn, RpaPageAttnImpl,
                                   .Arg<ffi::Buffer<ffi::S32>>()   // context_lens
                                   .Arg<ffi::Buffer<ffi::S32>>()   // block_tables
                                   .Ret<ffi::AnyBuffer>()          // out
+                                  .Ret<ffi::AnyBuffer>()          // scratch
                                   .Attr<float>("attn_scale"));
 
 // ---------------------------------------------------------------------------------------------- ragged_decode_attention
 static ffi::Error RpaRaggedDecodeImpl(hipStream_t stream, ffi::AnyBuffer query, ffi::AnyBuffer key, ffi::AnyBuffer value,
                                       ffi::Buffer<ffi::S32> sequence_start, ffi::Buffer<ffi::S32> sequence_end,
-                                      ffi::RemainingArgs rest, ffi::Result<ffi::AnyBuffer> out, float softmax_scale,
-                                      float logits_soft_cap, int32_t window_left) {
+                                      ffi::RemainingArgs rest, ffi::Result<ffi::AnyBuffer> out,
+                                      ffi::Result<ffi::AnyBuffer> scratch, float softmax_scale, float logits_soft_cap,
+                                      int32_t window_left) {
   const auto qd = query.dimensions();
   const auto kd = key.dimensions();
   if (qd.size() != 3 || kd.size() != 4) return Invalid("rank mismatch in ragged_decode_attention operands");
@@ -296,8 +281,7 @@ static ffi::Error RpaRaggedDecodeImpl(hipStream_t stream, ffi::AnyBuffer query, 
     p.aux_rows = static_cast<int32_t>(aux->dimensions()[0]);
     p.num_sinks = static_cast<int32_t>(aux->dimensions()[1]);
   }
-  p.workspace_bytes = rpa_ragged_decode_workspace_bytes(&p);
-  if (ffi::Error e = StreamWorkspace(stream, p.workspace_bytes, &p.workspace); e.failure()) return e;
+  if (ffi::Error e = UseScratch(stream, scratch, rpa_ragged_decode_workspace_bytes(&p), &p.workspace, &p.workspace_bytes); e.failure()) return e;
   if (rpa_ragged_decode_launch(&p, stream) != RPA_OK) return Invalid(rpa_last_error());
   return ffi::Error::Success();
 }
@@ -312,6 +296,7 @@ XLA_FFI_DEFINE_HANDLER_SYMBOL(RpaRaggedDecode, RpaRaggedDecodeImpl,
                                   .Arg<ffi::Buffer<ffi::S32>>()   // sequence_end
                                   .RemainingArgs()                // [softmax_aux]
                                   .Ret<ffi::AnyBuffer>()          // out
+                                  .Ret<ffi::AnyBuffer>()          // scratch
                                   .Attr<float>("softmax_scale")
                                   .Attr<float>("logits_soft_cap")
                                   .Attr<int32_t>("window_left"));

@@ -9,6 +9,9 @@ ejkernel/kernels/_xla/ragged_page_attention_v3/_kernel.py:110-126), ``page_atten
 ``ragged_decode_attention``, all traceable under ``jax.jit``.  Like the reference's native call
 (ejkernel/callib/_triton_call.py:760-799) they are forward-only: no JVP and no batching rule.
 
+Scratch memory belongs to XLA: every call declares one more result than the op has, ``uint8[n]`` with ``n`` from
+the library's ``rpa_*_workspace_bytes`` for the call's static shapes, and drops it; the handlers allocate nothing.
+
 This image has no JAX, so this module has not been built or run here; the torch-tensor
 entry point in ``ejkernel_amd.modules`` is the tested one.  Both go through the same C ABI.
 """
@@ -55,6 +58,27 @@ def _register():
     _registered = True
 
 
+def _scratch(nbytes: int):
+    """The extra result every handler takes: the op's workspace, owned and placed by XLA."""
+    return jax.ShapeDtypeStruct((max(int(nbytes), 256),), jnp.uint8)
+
+
+def _rpa_dims(total_tokens, num_q_heads, num_kv_heads, head_dim, page_size, num_pages, max_num_seqs, pages_per_seq, dtype,
+              cfg=None, flags=0):
+    """RpaParams carrying the static shapes only (what the workspace-size queries read)."""
+    p = _native.RpaParams()
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = total_tokens, num_q_heads, num_kv_heads, head_dim
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = page_size, num_pages, max_num_seqs, pages_per_seq
+    bf16 = jnp.dtype(dtype) == jnp.bfloat16
+    p.dtype = _native.RPA_DTYPE_BF16 if bf16 else _native.RPA_DTYPE_F32
+    p.compute = _native.RPA_COMPUTE_BF16 if bf16 else _native.RPA_COMPUTE_F32
+    if cfg is not None:
+        p.num_queries_per_block = cfg.num_queries_per_block or 0
+        p.num_kv_pages_per_block = cfg.num_kv_pages_per_block or 0
+    p.flags = flags
+    return p
+
+
 def ragged_page_attention(queries, kv_pages, context_lens, block_tables, query_start_loc, num_seqs, softmax_aux=None, /,
                           *, softmax_scale=None, logits_soft_cap=None, compute_dtype=jnp.bfloat16, optimized=False,
                           sliding_window=None, mask_value=None, vmem_limit_bytes=None, platform=None, cfg=None,
@@ -78,8 +102,11 @@ def ragged_page_attention(queries, kv_pages, context_lens, block_tables, query_s
         elif aux.shape[0] != num_q_heads:
             aux = jnp.repeat(aux, num_q_heads // aux.shape[0], axis=0)
         operands.append(aux)
-    call = jax.ffi.ffi_call(_TARGET, jax.ShapeDtypeStruct(queries.shape, queries.dtype))
-    out = call(
+    dims = _rpa_dims(total_tokens, num_q_heads, combined // 2, head_dim, page_size, num_pages, max_num_seqs, pages_per_seq,
+                     queries.dtype, cfg)
+    nbytes = _native.load().rpa_workspace_bytes(ctypes.byref(dims))
+    call = jax.ffi.ffi_call(_TARGET, (jax.ShapeDtypeStruct(queries.shape, queries.dtype), _scratch(nbytes)))
+    out, _ = call(
         *operands,
         softmax_scale=np.float32(head_dim**-0.5 if softmax_scale is None else softmax_scale),
         logits_soft_cap=np.float32(0.0 if logits_soft_cap is None else logits_soft_cap),
@@ -99,24 +126,42 @@ def ragged_page_attention_v3(queries, keys, values, kv_cache, kv_lens, block_tab
     """Cache update + attention; returns ``(out, kv_cache)`` with the cache updated in place (operand 3 is aliased to
     the second result, so jit the caller with the cache donated as the reference does)."""
     _register()
+    v = _native.RpaV3Params()
+    v.attn = _rpa_dims(queries.shape[0], queries.shape[1], keys.shape[1], queries.shape[2], kv_cache.shape[1], kv_cache.shape[0],
+                       kv_lens.shape[0], block_tables.size // max(kv_lens.shape[0], 1), queries.dtype,
+                       flags=_native.RPA_FLAG_FP32_LOGITS)
+    cache_dt = jnp.dtype(kv_cache.dtype)
+    v.cache_dtype = {jnp.dtype(jnp.bfloat16): _native.RPA_DTYPE_BF16, jnp.dtype(jnp.float32): _native.RPA_DTYPE_F32,
+                     jnp.dtype(jnp.float8_e4m3fn): _native.RPA_DTYPE_FP8_E4M3,
+                     jnp.dtype(jnp.float8_e5m2): _native.RPA_DTYPE_FP8_E5M2}[cache_dt]
+    v.cache_head_dim, v.cache_combined_heads = kv_cache.shape[4], kv_cache.shape[2] * kv_cache.shape[3]
+    nbytes = _native.load().rpa_v3_workspace_bytes(ctypes.byref(v))
     call = jax.ffi.ffi_call(
         "mi355x_rpa_v3",
-        (jax.ShapeDtypeStruct(queries.shape, queries.dtype), jax.ShapeDtypeStruct(kv_cache.shape, kv_cache.dtype)),
+        (jax.ShapeDtypeStruct(queries.shape, queries.dtype), jax.ShapeDtypeStruct(kv_cache.shape, kv_cache.dtype), _scratch(nbytes)),
         input_output_aliases={3: 1},
     )
     f32 = lambda x: np.float32(0.0 if x is None else x)  # noqa: E731
     return call(queries, keys, values, kv_cache, kv_lens, block_tables, query_start_loc, distribution,
                 softmax_scale=np.float32(queries.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale),
                 logits_soft_cap=f32(logits_soft_cap), q_scale=f32(q_scale), k_scale=f32(k_scale), v_scale=f32(v_scale),
-                sliding_window=np.int32(0 if sliding_window is None else sliding_window))
+                sliding_window=np.int32(0 if sliding_window is None else sliding_window))[:2]
 
 
 def page_attention(query, key_cache, value_cache, context_lens, block_tables, /, *, attn_scale=None):
     """One query token per sequence over separate paged K and V caches ``[blocks, kv heads, block, head_dim]``."""
     _register()
-    call = jax.ffi.ffi_call("mi355x_page_attention", jax.ShapeDtypeStruct(query.shape, query.dtype))
+    p = _native.RpaPageAttnParams()
+    p.num_seqs, p.num_q_heads, p.head_dim = query.shape
+    p.num_blocks, p.num_kv_heads, p.block_size = key_cache.shape[:3]
+    p.max_blocks = block_tables.shape[1]
+    bf16 = jnp.dtype(query.dtype) == jnp.bfloat16
+    p.dtype = _native.RPA_DTYPE_BF16 if bf16 else _native.RPA_DTYPE_F32
+    p.compute = _native.RPA_COMPUTE_BF16 if bf16 else _native.RPA_COMPUTE_F32
+    nbytes = _native.load().rpa_page_attention_workspace_bytes(ctypes.byref(p))
+    call = jax.ffi.ffi_call("mi355x_page_attention", (jax.ShapeDtypeStruct(query.shape, query.dtype), _scratch(nbytes)))
     return call(query, key_cache, value_cache, context_lens, block_tables,
-                attn_scale=np.float32(query.shape[-1] ** -0.5 if attn_scale is None else attn_scale))
+                attn_scale=np.float32(query.shape[-1] ** -0.5 if attn_scale is None else attn_scale))[0]
 
 
 def ragged_decode_attention(query, key, value, sequence_start, sequence_end, softmax_aux=None, /, *, softmax_scale=None,
@@ -128,8 +173,17 @@ def ragged_decode_attention(query, key, value, sequence_start, sequence_end, sof
     if softmax_aux is not None:
         aux = jnp.asarray(softmax_aux, jnp.float32)
         operands.append(aux[None] if aux.ndim == 1 else aux)
-    call = jax.ffi.ffi_call("mi355x_ragged_decode_attention", jax.ShapeDtypeStruct(query.shape, query.dtype))
+    p = _native.RpaRaggedDecodeParams()
+    p.batch, p.num_q_heads, p.head_dim = query.shape
+    p.seq_len, p.num_kv_heads = key.shape[1], key.shape[2]
+    bf16 = jnp.dtype(query.dtype) == jnp.bfloat16
+    p.dtype = _native.RPA_DTYPE_BF16 if bf16 else _native.RPA_DTYPE_F32
+    p.compute = _native.RPA_COMPUTE_BF16 if bf16 else _native.RPA_COMPUTE_F32
+    if softmax_aux is not None:
+        p.aux_rows, p.num_sinks = operands[-1].shape
+    nbytes = _native.load().rpa_ragged_decode_workspace_bytes(ctypes.byref(p))
+    call = jax.ffi.ffi_call("mi355x_ragged_decode_attention", (jax.ShapeDtypeStruct(query.shape, query.dtype), _scratch(nbytes)))
     return call(*operands,
                 softmax_scale=np.float32(query.shape[-1] ** -0.5 if softmax_scale is None else softmax_scale),
                 logits_soft_cap=np.float32(0.0 if logits_soft_cap is None else logits_soft_cap),
-                window_left=np.int32(-1 if sliding_window is None else int(sliding_window[0])))
+                window_left=np.int32(-1 if sliding_window is None else int(sliding_window[0])))[0]

@@ -19,6 +19,7 @@ from __future__ import annotations
 
 import ctypes
 import threading
+import warnings
 from typing import Any, Literal
 
 import torch
@@ -35,6 +36,7 @@ _workspaces: dict[tuple[int, int], torch.Tensor] = {}
 _MAX_WORKSPACES = 16
 _MAX_WORKSPACE_BYTES = 4 << 30
 _workspaces_lock = threading.Lock()  # host threads launch on streams of their own at the same time
+_warned_scalar: set[tuple] = set()   # shapes already reported as running on the scalar kernel
 
 
 def _compute_mode(compute_dtype: Any) -> int:
@@ -221,6 +223,16 @@ def _launch(queries, kv_pages, context_lens, block_tables, query_start_loc, num_
         kv_start = kv_start.to(device=dev, dtype=torch.int32).contiguous()
         p.kv_start = kv_start.data_ptr()
 
+    if p.dtype == _native.RPA_DTYPE_BF16 and p.compute == _native.RPA_COMPUTE_BF16 and not (flags & _native.RPA_FLAG_FORCE_GENERIC):
+        # a bf16 call is expected on the MFMA kernels: say so, once per shape, when it is not
+        shape = (head_dim, page_size, max_num_seqs)
+        if shape not in _warned_scalar and lib.rpa_kernel_path(ctypes.byref(p)) == 0:
+            _warned_scalar.add(shape)
+            warnings.warn(
+                f"ragged_page_attention: head_dim={head_dim}, page_size={page_size}, max_num_seqs={max_num_seqs} runs on "
+                "the scalar kernel (exact, about fifty times slower on a decode batch): the MFMA kernels take head_dim "
+                "64..256 in multiples of 16, page sizes that are powers of two from 4 and up to 16384 sequences",
+                RuntimeWarning, stacklevel=3)
     with torch.cuda.device(dev):
         stream_ptr = torch.cuda.current_stream(dev).cuda_stream
         if static_scratch:  # the entry point that allocates nothing: scratch inside the library, no workspace

@@ -161,6 +161,13 @@ typedef struct RpaV3Params {
 /* Bytes of workspace rpa_fwd_launch needs for these static dims (pointers are ignored). */
 uint64_t rpa_workspace_bytes(const RpaParams* dims);
 
+/* Which kernels rpa_fwd_launch runs for these static dims, dtypes and flags (pointers are ignored): 1 = the MFMA
+ * kernels, 0 = the scalar kernel -- fp32 inputs or compute, head_dim below 64, above 256 or no multiple of 16,
+ * page_size below 4 or no power of two, more than 16384 sequences, RPA_FLAG_FORCE_GENERIC: exact, and some fifty
+ * times slower on a decode batch -- and -1 for dims the launch would reject.  No counterpart in the reference, whose
+ * registry names the backend it picked; a caller can warn, as the Python layer does, or choose another shape. */
+int rpa_kernel_path(const RpaParams* dims);
+
 /* Clears the counters at the head of a freshly allocated workspace (enqueue only).
  * A launch leaves them cleared again, so this is needed once per allocation. */
 int rpa_workspace_init(void* workspace, uint64_t workspace_bytes, void* hip_stream);

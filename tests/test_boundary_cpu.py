@@ -89,6 +89,28 @@ def test_python_constants_are_the_header_s():
         assert int(defines[n]) == getattr(_native, n), n
 
 
+def test_kernel_path_query_names_what_the_mfma_kernels_take():
+    """rpa_kernel_path: 1 where the MFMA kernels run, 0 where the scalar kernel does, -1 for dims a launch rejects."""
+    lib = _native.load()
+    p = _native.RpaParams()
+    p.total_tokens, p.num_q_heads, p.num_kv_heads, p.head_dim = 16, 8, 2, 128
+    p.page_size, p.num_pages, p.max_num_seqs, p.pages_per_seq = 16, 64, 4, 16
+    p.softmax_scale = 0.1
+    p.dtype, p.compute = _native.RPA_DTYPE_BF16, _native.RPA_COMPUTE_BF16
+    assert lib.rpa_kernel_path(ctypes.byref(p)) == 1
+    for field, value in (("head_dim", 48), ("head_dim", 72), ("head_dim", 320), ("page_size", 2), ("page_size", 24),
+                         ("flags", _native.RPA_FLAG_FORCE_GENERIC), ("compute", _native.RPA_COMPUTE_F32)):
+        keep = getattr(p, field)
+        setattr(p, field, value)
+        assert lib.rpa_kernel_path(ctypes.byref(p)) == 0, (field, value)
+        setattr(p, field, keep)
+    for hd in (64, 80, 96, 144, 256):
+        p.head_dim = hd
+        assert lib.rpa_kernel_path(ctypes.byref(p)) == 1, hd
+    p.head_dim, p.num_q_heads = 128, 7   # not a multiple of the kv heads: the launch would reject it
+    assert lib.rpa_kernel_path(ctypes.byref(p)) == -1
+
+
 def test_v3_workspace_counts_the_stored_logits_of_an_8_bit_cache():
     lib = _native.load()
     v = _native.RpaV3Params()

@@ -132,6 +132,55 @@ def test_reference_benchmark_grid_shapes(S, page):
         assert not out[rows:].any()
 
 
+def test_tile_kernel_is_picked_on_the_device_where_the_host_cannot_tell():
+    """Static shapes that say nothing about the batch (many rows, few tokens per max_num_seqs, no flag, no hint): both
+    tile kernels are enqueued and the device picks one from the lengths.  A batch whose prefill work outweighs its
+    decode stream must come out bit for bit as the pipelined tiles give it, one whose stream outweighs the chunks as
+    the 128-row tiles do; and the pair of launches replays from a HIP graph on new queries."""
+    from ejkernel_amd import _native
+    from ejkernel_amd.modules.operations import RaggedPageAttention, RaggedPageAttentionConfig
+    from ejkernel_amd.workloads import make_batch
+
+    def run_flags(bb, flags, out=None):
+        o = RaggedPageAttention().run(*bb.args(), softmax_scale=bb.softmax_scale, cfg=RaggedPageAttentionConfig(), _flags=flags,
+                                      _out=out)
+        torch.cuda.synchronize()
+        return o
+
+    rng = np.random.default_rng(3)
+    chunks = make_batch([600] * 4 + [1] * 8, [900] * 4 + list(rng.integers(1000, 3000, size=8)), num_q_heads=32,
+                        num_kv_heads=8, head_dim=128, page_size=32, pages_per_seq=128, seed=51, device=DEV, max_num_seqs=64)
+    stream = make_batch([600] + [1] * 60, [900] + list(rng.integers(3000, 4096, size=60)), num_q_heads=32, num_kv_heads=8,
+                        head_dim=128, page_size=32, pages_per_seq=128, seed=52, device=DEV, max_num_seqs=64)
+    pipe, plain = _native.RPA_FLAG_PIPE_TILES, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES
+    for b, picked, other in ((chunks, pipe, plain), (stream, plain, pipe)):
+        assert b.queries.shape[0] * 32 > 20480 and b.queries.shape[0] < 128 * 64   # no rule of the host's applies
+        out = run_flags(b, 0)
+        assert torch.equal(out, run_flags(b, picked))
+        assert not torch.equal(out, run_flags(b, other))   # (the other kernel's rounding differs somewhere)
+        sub, _ = check_sample(b, out, 4)
+        assert not out[b.total_valid_tokens:].any()
+    # the two launches of one call in a HIP graph
+    b = chunks
+    out = torch.zeros_like(b.queries)
+    run_flags(b, 0, out)
+    g = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            RaggedPageAttention().run(*b.args(), softmax_scale=b.softmax_scale, cfg=RaggedPageAttentionConfig(), _out=out)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    gen = torch.Generator(device=DEV).manual_seed(9)
+    for k in range(3):
+        b.queries[: b.total_valid_tokens] = torch.randn(b.total_valid_tokens, 32, 128, device=DEV, generator=gen).to(torch.bfloat16)
+        out.fill_(5.0)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out.clone(), run_flags(b, pipe)), f"replay {k}"
+
+
 def test_long_prompts_on_pipelined_and_plain_tiles():
     """prefill_long (2 prompts x 8192 tokens) is too much for the CPU restatement in seconds (its scaled form is checked
     against it elsewhere): here the two tile kernels must agree with each other within the parity bound, each must be

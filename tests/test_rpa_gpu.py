@@ -623,3 +623,29 @@ def test_launch_recorded_in_a_hip_graph_replays_correctly():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out_g, want), rep
+
+
+def test_bf16_call_on_the_scalar_kernel_warns_once_per_shape():
+    """A bf16 call the MFMA kernels do not take (here: pages of 2 tokens) runs on the scalar kernel, exact and far
+    slower: the Python layer says so the first time it sees the shape, and not again."""
+    import warnings
+
+    import importlib
+
+    from ejkernel_amd.modules import ragged_page_attention
+
+    m = importlib.import_module("ejkernel_amd.modules.operations.ragged_page_attention")
+    b = small([3, 1], [9, 30], page_size=2, pages_per_seq=16, head_dim=128)
+    m._warned_scalar.discard((128, 2, b.block_tables.shape[0]))
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        out = ragged_page_attention(*b.args(), **b.kwargs())
+        ragged_page_attention(*b.args(), **b.kwargs())
+    torch.cuda.synchronize()
+    assert len([w for w in seen if "scalar kernel" in str(w.message)]) == 1
+    assert_bf16_parity(to_np(out), run_strict(b), b.total_valid_tokens, "pages of 2 tokens")
+    ok = small([3, 1], [9, 30], page_size=4, pages_per_seq=8, head_dim=128)
+    with warnings.catch_warnings(record=True) as seen:
+        warnings.simplefilter("always")
+        ragged_page_attention(*ok.args(), **ok.kwargs())
+    assert not [w for w in seen if "scalar kernel" in str(w.message)]
