@@ -13,7 +13,8 @@ struct Cfg {
   static constexpr int NKS = D / 32;        // k-steps of the QK^T contraction
   static constexpr int TT = 16 * NT;        // tokens per iteration
   static constexpr int NSLOT = 4 * NT;      // tokens each lane fetches per iteration
-  static constexpr int ROWB = D * 2 + 16;   // LDS bytes per K row (16 B pad: conflict-free b128 reads)
+  static constexpr int ROWB = D * 2 + 32;   // LDS bytes per K row: with a 32-byte pad neither the b128 reads (lane = row) nor
+                                            // the b128 writes (lane = piece) meet a bank conflict; with 16 the reads do, two-way
   static constexpr int LDS_PER_WAVE = TT * ROWB;
   static constexpr int SINK_KEYS = 8;                   // sink keys of ragged_decode_attention staged in LDS per wavefront
   static constexpr int SINK_LDS = SINK_KEYS * 2 * D * 2 + 16 * SINK_KEYS * 4;  // their K rows, their V rows, 16 rows of biases

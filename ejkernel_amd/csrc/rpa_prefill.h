@@ -237,8 +237,16 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // V blocks are laid out for the transposing operand read instead: [32-byte column unit][row of the block], so the
   // lane that fills LDS bytes [16 l, 16 l + 16) of a block fetches half (l & 1) of unit (l / 2) / RB of row (l / 2) % RB.
   // (Without the transposing read the V tile is laid out like the K tile.)
+  // With four rows to a block (256-byte rows) the four 16-lane groups of a transposing read take the same column unit of
+  // four consecutive blocks, 1 KiB apart: the same half of the banks, four groups deep where two is the least a
+  // 512-byte read takes.  So every second block keeps its units in swapped pairs (unit c at position c ^ 1): odd and even
+  // blocks then answer from different halves of the banks.  (With eight rows to a block, 128-byte rows, two groups
+  // share a block and the other two the next one: nothing to swap.)
+  constexpr bool kSwapUnits = C::TRV && C::RB == 4;
   const int v_row = C::TRV ? (lane >> 1) % C::RB : l_row;
-  const uint32_t v_src = PB * piece_of(static_cast<uint32_t>(2 * ((lane >> 1) / C::RB) + (lane & 1)));  // byte offset in the row
+  const uint32_t v_unit = static_cast<uint32_t>((lane >> 1) / C::RB);
+  const uint32_t v_src = PB * piece_of(2 * v_unit + (lane & 1));  // byte offset in the row
+  const uint32_t v_src_odd = kSwapUnits ? PB * piece_of(2 * (v_unit ^ 1u) + (lane & 1)) : v_src;  // ... in an odd block
   // Wavefront w moves rows [GROUP * w, GROUP * (w + 1)) of the K tile and of the V tile: BPW / 2 blocks each.
   constexpr int HB = C::BPW / 2, GROUP = C::RB * HB;
   uint32_t pre_off[HB];  // per-lane byte offset of K block n inside the group: row part + swizzled piece
@@ -248,8 +256,11 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     pre_off[n] = static_cast<uint32_t>(C::RB * n + l_row) * stride_b + PB * piece_of(static_cast<uint32_t>(l_slot ^ C::swz(t_local)));
   }
   const uint32_t v_pre_off = static_cast<uint32_t>(v_row) * stride_b + v_src + v_delta;  // V block 0; block n adds RB rows
+  const uint32_t v_pre_off_odd = static_cast<uint32_t>(v_row) * stride_b + v_src_odd + v_delta;
+  // (a wavefront's group starts at an even block, so block n of the group is an odd block of the tile iff n is odd)
+  static_assert(!kSwapUnits || HB % 2 == 0, "the parity of a block inside its group must be its parity in the tile");
   auto v_src_off = [&](int n) {  // byte offset of this lane's V piece in block n of the group, from the group's first K row
-    return C::TRV ? v_pre_off + n * C::RB * stride_b : pre_off[n] + v_delta;
+    return C::TRV ? ((n & 1) ? v_pre_off_odd : v_pre_off) + n * C::RB * stride_b : pre_off[n] + v_delta;
   };
   const bool group_in_page = p.page_size >= GROUP;
   // 8-bit cache: this lane's K and V pieces of the tile being fetched, and where they go once widened
@@ -299,7 +310,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       const int t_c = min(t_first + C::RB * n, t_last & ~(C::RB - 1));
       const int t_local = GROUP * wave + C::RB * n + l_row;
       const uint32_t k_piece = PB * piece_of(static_cast<uint32_t>(l_slot ^ C::swz(t_local)));
-      const uint32_t v_piece = C::TRV ? v_src : k_piece;
+      const uint32_t v_piece = C::TRV ? ((n & 1) ? v_src_odd : v_src) : k_piece;
       if (C::RB > 4 && p.page_size < C::RB) {
         // pages shorter than a block (pages of 4 tokens under 128-byte rows): every lane looks its own row's page up
         auto row_base = [&](int tok) {
@@ -358,6 +369,9 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // address (half, sub-tile, unit) is a compile-time offset.
   const int v_key = 4 * g + (i >> 2);
   const int v_rd = (v_key / C::RB) * 1024 + (v_key % C::RB) * 32 + 8 * (i & 3);
+  // swapped units: this lane group's block is odd iff g is (sub-tiles and halves start at even blocks), and unit c of
+  // an odd block sits one unit further on for an even c, one back for an odd c
+  const int v_rd_swap = kSwapUnits && (g & 1) ? C::RB * 32 : 0;
   // Row-major V tile: lane (i, g) reads piece i (+ 16 per slice) of rows 4g..4g+3 and transposes in registers.
   int v_off[C::NS][4];
 #pragma unroll
@@ -408,7 +422,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
 #pragma unroll
               for (int u = 0; u < 2; ++u) {
                 const s16x4_t t = __builtin_amdgcn_ds_read_tr16_b64_v4i16((__attribute__((address_space(3))) s16x4_t*)(
-                    vt + v_rd + ((32 * h + 16 * u) / C::RB) * 1024 + (c + C::CB * sN) * (C::RB * 32)));
+                    vt + v_rd + ((c & 1) ? -v_rd_swap : v_rd_swap) + ((32 * h + 16 * u) / C::RB) * 1024 + (c + C::CB * sN) * (C::RB * 32)));
                 const u32x2_t t2 = __builtin_bit_cast(u32x2_t, t);
                 vraw[c][2 * u] = t2[0];
                 vraw[c][2 * u + 1] = t2[1];
