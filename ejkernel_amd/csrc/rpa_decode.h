@@ -578,7 +578,42 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     }
   }
 
-  if (part.partial) {
+  bool merged = false;
+  if constexpr (kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
+    if (part.in_workgroup) {
+      // ---- the four wavefronts of the workgroup hold the four parts of this (sequence, kv head): wavefronts 1..3 leave
+      // their state in their own K tile (accumulator piece c of row i, lane group g at ((16 c + i) * 4 + g) * 16, then
+      // the rows' maxima and sums), wavefront 0 adds them to its own in wavefront order.  Every wavefront of the
+      // workgroup comes here, with or without keys, so the barrier is complete.
+      const int wv = static_cast<int>(threadIdx.x) / kWave;
+      constexpr int kState = 16 * D * 4;
+      if (wv != 0) {
+#pragma unroll
+        for (int c = 0; c < 8; ++c) *reinterpret_cast<f32x4_t*>(lds_k + ((16 * c + i) * 4 + g) * 16) = o_acc[0][c];
+        if (g == 0) *reinterpret_cast<float2*>(lds_k + kState + 8 * i) = float2{m_run, l_run};
+      }
+      __syncthreads();
+      if (wv != 0) return;
+#pragma unroll 1
+      for (int w = 1; w < kWgWaves; ++w) {
+        const char* st = lds_k + w * C::LDS_PER_WAVE;
+        const float2 ml = *reinterpret_cast<const float2*>(st + kState + 8 * i);
+        const float m_new = fmaxf(m_run, ml.x);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float keep = __builtin_amdgcn_exp2f((m_run - m_use) * kLog2e);
+        const float wgt = __builtin_amdgcn_exp2f((ml.x - m_use) * kLog2e);
+        l_run = l_run * keep + wgt * ml.y;
+        m_run = m_new;
+#pragma unroll
+        for (int c = 0; c < 8; ++c) {
+          const f32x4_t ov = *reinterpret_cast<const f32x4_t*>(st + ((16 * c + i) * 4 + g) * 16);
+          o_acc[0][c] = o_acc[0][c] * keep + wgt * ov;
+        }
+      }
+      merged = true;
+    }
+  }
+  if (part.partial && !merged) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
     // Who writes, who reads: this wavefront writes its slot; the wavefront that draws the last ticket of the
     // (sequence, kv head) -- any workgroup, usually on another XCD with another L2 -- reads every slot.  Partials are

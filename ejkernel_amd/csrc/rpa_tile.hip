@@ -106,9 +106,17 @@ void rpa_tile_kernel(TileArgs a) {
   // (more than kWaveItemMaxRowTiles row tiles), or wave-level items (everything else).
   auto classify = [&](const SeqInfo& si, int& tiles, int& items, int& wg_items) {
     tiles = items = wg_items = 0;
-    if (si.eligible) tiles = item_heads * ((si.hi - si.lo_al + C::TT - 1) / C::TT + a.item_pad_tiles);
-    else if (!kWaveOnly && si.n_rt > kWaveItemMaxRowTiles) wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
-    else items = item_heads * si.n_rt;
+    if (si.eligible) {
+      const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
+      tiles = item_heads * (per_head + a.item_pad_tiles);
+      // (a kernel without prefill tiles has no use for the third sum: it counts the sequences that are too long for
+      // one workgroup per (sequence, kv head) there, and in the upper half those longer than half of that)
+      if (kWaveOnly) wg_items = (per_head > a.wg_item_tiles ? 1 : 0) + (2 * per_head > a.wg_item_tiles ? 65536 : 0);
+    } else if (!kWaveOnly && si.n_rt > kWaveItemMaxRowTiles) {
+      wg_items = p.num_kv_heads * ((si.rows + PC::WGROWS - 1) / PC::WGROWS);
+    } else {
+      items = item_heads * si.n_rt;
+    }
   };
   const int per = (((nseq + kWgThreads - 1) / kWgThreads + K - 1) >> shift) << shift;  // a multiple of K per thread
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
@@ -139,6 +147,11 @@ void rpa_tile_kernel(TileArgs a) {
   total_items = __builtin_amdgcn_readfirstlane(total_items);
   total_tiles = __builtin_amdgcn_readfirstlane(total_tiles);
   total_wg = __builtin_amdgcn_readfirstlane(total_wg);
+  int n_long = 0;  // kWaveOnly: sequences of the decode stream with more than wg_item_tiles tiles, and (<< 16) with more than half
+  if constexpr (kWaveOnly) {
+    n_long = total_wg;
+    total_wg = 0;
+  }
   const int nc = (nseq + K - 1) >> shift;  // entries in use
   if (tid == 0) {
     item_start[nc] = total_items;
@@ -259,6 +272,39 @@ void rpa_tile_kernel(TileArgs a) {
     zero_rows_past_batch(static_cast<int>(blockIdx.x) - grid_wgs, grid_all - grid_wgs);
     return;
   }
+  // ---- a small batch of short decode sequences: workgroup b takes (sequence, kv head) number b, a quarter of its
+  // tiles per wavefront, and the four partial states meet in LDS.  Split over the grid's wavefronts instead, the
+  // parts would go through memory: partial state written through, a ticket, the parts read back -- three round trips
+  // of a microsecond or two each, which is most of what such a launch takes.  (The block stands in front of
+  // everything the other kinds of work set up -- shares, queues, look-ups: some eight hundred scalar instructions that a
+  // wavefront alone on its SIMD takes two microseconds to get through.)
+  // Decode steps only: a batch that also holds wave-level items (short chunks, sequences without keys) is split the usual way.
+  bool wg_items_mode = false;
+  if constexpr (kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
+    // A wavefront walks a quarter of its (sequence, kv head): with few of them the longer ones do better cut into
+    // more parts over more wavefronts (one sequence of 1024 keys, 8 kv heads: 20.5 us split over the grid, 22.4
+    // here; 32 such sequences: 34.4 against 31.3).
+    const int n_heads = nseq * item_heads;
+    const int too_long = n_heads >= 32 ? (n_long & 0xffff) : (n_long >> 16);
+    wg_items_mode = total_tiles > 0 && total_items == 0 && a.wg_item_tiles > 0 && nseq < 65536 && too_long == 0 && n_heads <= grid_wgs;
+    if (wg_items_mode) {
+      const int b = static_cast<int>(blockIdx.x);
+      if (b < n_heads) {
+        const int s = b / item_heads, j = b - s * item_heads;
+        const SeqInfo si = seq_info<C::TT>(a, s, G);
+        if (si.eligible) {
+          const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
+          const int per_wave = (per_head + kWgWaves - 1) / kWgWaves;
+          Part part;
+          part.partial = true;
+          part.in_workgroup = true;
+          const int lo = si.lo_al + wave * per_wave * C::TT;
+          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, lo, min(si.hi, lo + per_wave * C::TT), part);
+        }
+      }
+    }
+  }
+  if (!wg_items_mode) {
   // Largest s in [0, nseq) with start[s] <= x; sequences that add nothing share their successor's start and
   // are skipped because the search keeps the last one that does not exceed x.
   // `kind` says which count the array sums (0 items, 1 stream tiles, 2 prefill tiles); `base` receives start[s].
@@ -526,6 +572,7 @@ void rpa_tile_kernel(TileArgs a) {
       }
     }
   }
+  }  // !wg_items_mode
   if (!idle_wgs_exist) zero_rows_past_batch(static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x));
 }
 
@@ -549,6 +596,7 @@ struct Tune {
   int pipe_min_tokens_per_seq;  // RPA_TUNE_PIPE_MIN_TOKENS_PER_SEQ: average query tokens per sequence from which it is used
   int no_logit_stash;      // RPA_TUNE_NO_LOGIT_STASH: two-launch calls read K in both launches (experiments)
   int device_select;       // RPA_TUNE_DEVICE_SELECT: 0 = never enqueue both tile kernels and let the device pick
+  int wg_item_tiles;       // RPA_TUNE_WG_ITEM_TILES: longest (sequence, kv head), in tiles, of a batch that runs one per workgroup
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -572,6 +620,7 @@ static const Tune& tune() {
     x.pipe_stream_wgs = max(8, env_int("RPA_TUNE_PIPE_STREAM_WGS", 160)) & ~7;
     x.no_logit_stash = env_int("RPA_TUNE_NO_LOGIT_STASH", 0);
     x.device_select = env_int("RPA_TUNE_DEVICE_SELECT", 1);
+    x.wg_item_tiles = max(0, env_int("RPA_TUNE_WG_ITEM_TILES", 32));
     return x;
   }();
   return t;
@@ -712,6 +761,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.phase_mode = tune().phase_mode;
   a.pair = 0;
   a.select = 0;
+  a.wg_item_tiles = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_item_tiles;  // a caller that names the split gets the split
   a.even_xcd_permille = tune().even_xcd_permille;
   // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
   // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes

@@ -49,6 +49,9 @@ struct TileArgs {
   // tiles.  With 1 or 2 every workgroup weighs the batch's prefill work against its decode stream the same way and
   // the launch that is not picked ends there.
   int select;
+  // A batch of few, short decode sequences: up to how many tiles a (sequence, kv head) may have for the batch to run
+  // one workgroup per (sequence, kv head), its four wavefronts merging through LDS (0 = never).
+  int wg_item_tiles;
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the
@@ -97,6 +100,7 @@ struct Shares {
 // A wavefront's part of one (sequence, kv head) of the decode stream.
 struct Part {
   bool partial;         // the (sequence, kv head) is shared with other wavefronts
+  bool in_workgroup = false;  // ... with the other wavefronts of this workgroup and no one else: they merge through LDS
   int slot;             // workspace slot of this part
   int first_w, last_w;  // wavefronts sharing it (every one of them holds at least one of its tiles)
   int stream_a;         // stream index of its first tile

@@ -111,7 +111,9 @@ typedef struct RpaParams {
                                   /* tiles otherwise.  RPA_FLAG_PREFILL_TILES / PIPE_TILES / PLAIN_TILES come first.  */
   int32_t num_kv_pages_per_block; /* the least stretch of a sequence, in pages, that one streaming wavefront takes     */
                                   /* before a small batch is spread over more wavefronts (split-K granularity;        */
-                                  /* default: 2 tiles of 32 keys, more for long sequences)                            */
+                                  /* default: 2 tiles of 32 keys, more for long sequences -- and one workgroup per     */
+                                  /* (sequence, kv head), merged in LDS, for a decode batch of at most 256 of them     */
+                                  /* with up to 1024 keys each, which a value here switches off)                      */
   int32_t num_warps;              /* accepted, ignored: workgroups have 4 wavefronts                                   */
   int32_t num_stages;             /* accepted, ignored: 2 LDS stages in the 128-row tile, 4 in the pipelined one      */
   uint32_t flags;                 /* RPA_FLAG_*                                       */

@@ -185,6 +185,38 @@ def test_bf16_head_dim_64_two_kv_heads_per_item(hq, hkv, window, cap, sinks):
         assert_bf16_parity(to_np(run_hip(b)), run_strict(b), b.total_valid_tokens, f"page {page} {hq}/{hkv}")
 
 
+@pytest.mark.parametrize("hq,hkv,D", [(8, 2, 128), (32, 8, 128), (4, 4, 128), (16, 1, 128), (8, 2, 64), (16, 8, 64), (6, 3, 64)])
+@pytest.mark.parametrize("window,cap,sinks", [(None, None, False), (40, 20.0, True), (300, None, False)])
+def test_bf16_small_decode_batches_one_workgroup_per_kv_head(hq, hkv, D, window, cap, sinks):
+    """A decode batch of few short sequences runs one workgroup per (sequence, kv head): each of its four wavefronts
+    walks a quarter of the keys and the partial states are merged in LDS.  Lengths around the tile and quarter
+    boundaries (wavefronts without keys, a last tile of one key) up to 512 keys; up to 1024 in a batch of 32
+    (sequence, kv head)s or more, where the longer limit applies; and the first batch again with a chunk of three
+    tokens and a sequence of one key in it (with more than 16 rows the chunk is a wave-level item and sends the whole
+    batch the usual way; with fewer it is one more row tile of the mode, whose rows belong to three tokens).
+    `num_kv_pages_per_block` names the split and switches the mode off: the split over the grid, with its merge
+    through memory, must agree with it and with the oracle."""
+    aux = (torch.randn(hq, 2, generator=torch.Generator().manual_seed(5)) * 2).numpy() if sinks else None
+    lens = [1, 31, 32, 33, 64, 65, 96, 97, 100, 128, 129, 255, 300, 500, 512]
+    cases = [([1] * 15, lens, 32), ([1] * 15 + [3, 1], lens + [7, 1], 32)]
+    n_more = -(-32 // hkv) + 1   # enough sequences for 32 (sequence, kv head)s
+    rng = np.random.default_rng(11)
+    cases.append(([1] * n_more, [1024, 1000, 513] + rng.integers(1, 1025, size=n_more - 3).tolist(), 64))
+    for ql, kl, pps in cases:
+        b = small(ql, kl, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, pages_per_seq=pps, sliding_window=window,
+                  logits_soft_cap=cap, seed=23)
+        ref = run_strict(b, softmax_aux=aux)
+        out = run_hip(b, softmax_aux=aux)
+        rows = b.total_valid_tokens
+        assert_bf16_parity(to_np(out), ref, rows, f"{hq}/{hkv} D={D} W={window} cap={cap} sinks={sinks}")
+        assert torch.equal(run_hip(b, softmax_aux=aux), out)   # deterministic
+        assert not out[rows:].any()
+        split = run_hip(b, softmax_aux=aux, cfg=RaggedPageAttentionConfig(num_kv_pages_per_block=4))
+        assert_bf16_parity(to_np(split), ref, rows, "split over the grid")
+        # the two ways of cutting a row's keys differ by fp32 summation order only: a bf16 step or two of the largest outputs
+        assert (out[:rows].float() - split[:rows].float()).abs().max().item() <= 2e-2
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128), (8, 2, 64), (4, 4, 64)])
 @pytest.mark.parametrize("window", [None, 48])
