@@ -610,7 +610,7 @@ static const Tune& tune() {
     x.min_share_tiles = max(1, env_int("RPA_TUNE_MIN_SHARE_TILES", kMinShareTiles));
     x.item_pad_tiles = min(64, env_int("RPA_TUNE_ITEM_PAD_TILES", -1));  // negative: 128 keys' worth of tiles
     x.phase_mode = env_int("RPA_TUNE_PHASE_MODE", 4);
-    x.even_xcd_permille = min(900, max(100, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", 540)));
+    x.even_xcd_permille = min(900, env_int("RPA_TUNE_EVEN_XCD_PERMILLE", -1));  // negative: by head_dim, see run_tiled
     x.no_mimic = env_int("RPA_TUNE_NO_MIMIC", 0);
     x.no_wave_only = env_int("RPA_TUNE_NO_WAVE_ONLY", 0);
     x.wave_only_rows = env_int("RPA_TUNE_WAVE_ONLY_ROWS", kWaveOnlyMaxRows);
@@ -762,7 +762,10 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.pair = 0;
   a.select = 0;
   a.wg_item_tiles = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_item_tiles;  // a caller that names the split gets the split
-  a.even_xcd_permille = tune().even_xcd_permille;
+  // The wavefronts on odd XCDs stream about a tenth slower when all eight compete for memory; per-XCD exit times put the
+  // balance at 54.0 % of the stream on the even ones with 256-byte rows and at 54.7 % with 512-byte rows (head_dim 256:
+  // even XCDs left at 329 us, odd ones at 338 with 54.0 %; 0.3571 -> 0.3532 ms with 54.7 %).
+  a.even_xcd_permille = tune().even_xcd_permille >= 100 ? tune().even_xcd_permille : (p.head_dim > 128 ? 547 : 540);
   // Pure streaming runs fastest with one workgroup per compute unit -- unless a wavefront's loads carry half the
   // bytes (head_dim 64: rows of 128 bytes under 16-byte pieces), when it takes both workgroups to keep as many bytes
   // in flight.
