@@ -266,7 +266,19 @@ void rpa_tile_kernel(TileArgs a) {
   // A batch without prefill tiles is pure streaming: it runs fastest with one workgroup per compute unit, so
   // the second half of the grid (dispatched after every unit has one workgroup) does not stream.
   const int grid_all = static_cast<int>(gridDim.x);
-  const int grid_wgs = total_wg == 0 ? min(grid_all, a.stream_grid) : grid_all;
+  // A small batch of decode steps runs one workgroup per (sequence, kv head), see below; such a batch may use the
+  // whole grid, the streaming ones stop at stream_grid workgroups.
+  bool wg_items_mode = false;
+  const int n_heads = nseq * item_heads;
+  if constexpr (kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
+    // A wavefront walks a quarter of its (sequence, kv head): with few of them the longer ones do better cut into
+    // more parts over more wavefronts (one sequence of 1024 keys, 8 kv heads: 20.5 us split over the grid, 22.4
+    // in this mode; 32 such sequences: 34.4 against 31.3).
+    const int too_long = n_heads >= 32 ? (n_long & 0xffff) : (n_long >> 16);
+    wg_items_mode = total_tiles > 0 && total_items == 0 && a.wg_item_tiles > 0 && nseq < 65536 && too_long == 0 && n_heads <= grid_all;
+  }
+  const int grid_wgs = wg_items_mode ? max(n_heads, min(grid_all, a.stream_grid))
+                                     : total_wg == 0 ? min(grid_all, a.stream_grid) : grid_all;
   const bool idle_wgs_exist = grid_wgs < grid_all;
   if (static_cast<int>(blockIdx.x) >= grid_wgs) {
     zero_rows_past_batch(static_cast<int>(blockIdx.x) - grid_wgs, grid_all - grid_wgs);
@@ -279,14 +291,7 @@ void rpa_tile_kernel(TileArgs a) {
   // everything the other kinds of work set up -- shares, queues, look-ups: some eight hundred scalar instructions that a
   // wavefront alone on its SIMD takes two microseconds to get through.)
   // Decode steps only: a batch that also holds wave-level items (short chunks, sequences without keys) is split the usual way.
-  bool wg_items_mode = false;
   if constexpr (kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
-    // A wavefront walks a quarter of its (sequence, kv head): with few of them the longer ones do better cut into
-    // more parts over more wavefronts (one sequence of 1024 keys, 8 kv heads: 20.5 us split over the grid, 22.4
-    // here; 32 such sequences: 34.4 against 31.3).
-    const int n_heads = nseq * item_heads;
-    const int too_long = n_heads >= 32 ? (n_long & 0xffff) : (n_long >> 16);
-    wg_items_mode = total_tiles > 0 && total_items == 0 && a.wg_item_tiles > 0 && nseq < 65536 && too_long == 0 && n_heads <= grid_wgs;
     if (wg_items_mode) {
       const int b = static_cast<int>(blockIdx.x);
       if (b < n_heads) {
@@ -355,8 +360,11 @@ void rpa_tile_kernel(TileArgs a) {
                                             : a.phase_mode == 2 ? (blockIdx.x & 1) != 0
                                             : a.phase_mode == 3 ? ((blockIdx.x >> 3) & 1) != 0
                                             : a.phase_mode == 4);
+  // (Without prefill tiles there is one phase, and no loop: out of a loop the compiler hoists every invariant of every
+  // kind of work in front of it, some eight hundred scalar instructions that a small launch then waits two
+  // microseconds for whatever it holds.)
 #pragma unroll 1
-  for (int phase = 0; phase < 2; ++phase) {
+  for (int phase = kWaveOnly ? 1 : 0; phase < 2; ++phase) {
     if ((phase == 0) != stream_first) {
       if constexpr (!kWaveOnly) {
       // ---- prefill: one item per (sequence, kv head, tile of WGROWS rows), the row tiles of a (sequence, kv head)

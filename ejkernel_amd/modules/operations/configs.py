@@ -15,7 +15,7 @@ mean:
                             tokens per ``max_num_seqs``).  Results stay within the same tolerance either way.
 ``num_kv_pages_per_block``  the least stretch of a sequence, in pages, one streaming wavefront takes before a small
                             batch is spread over more wavefronts (None = 2 tiles of 32 keys, more for long sequences;
-                            and a decode batch of at most 256 (sequence, kv head)s of up to 1024 keys runs one
+                            and a decode batch of at most 512 (sequence, kv head)s of up to 1024 keys runs one
                             workgroup per (sequence, kv head) with the merge in LDS, which a value here switches off)
 ``num_warps``               accepted, ignored (workgroups have 4 wavefronts)
 ``num_stages``              accepted, ignored (2 LDS stages in the 128-row tile, 4 in the pipelined one)

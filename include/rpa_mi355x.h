@@ -112,7 +112,7 @@ typedef struct RpaParams {
   int32_t num_kv_pages_per_block; /* the least stretch of a sequence, in pages, that one streaming wavefront takes     */
                                   /* before a small batch is spread over more wavefronts (split-K granularity;        */
                                   /* default: 2 tiles of 32 keys, more for long sequences -- and one workgroup per     */
-                                  /* (sequence, kv head), merged in LDS, for a decode batch of at most 256 of them     */
+                                  /* (sequence, kv head), merged in LDS, for a decode batch of at most 512 of them     */
                                   /* with up to 1024 keys each, which a value here switches off)                      */
   int32_t num_warps;              /* accepted, ignored: workgroups have 4 wavefronts                                   */
   int32_t num_stages;             /* accepted, ignored: 2 LDS stages in the 128-row tile, 4 in the pipelined one      */

@@ -202,6 +202,9 @@ def test_bf16_small_decode_batches_one_workgroup_per_kv_head(hq, hkv, D, window,
     n_more = -(-32 // hkv) + 1   # enough sequences for 32 (sequence, kv head)s
     rng = np.random.default_rng(11)
     cases.append(([1] * n_more, [1024, 1000, 513] + rng.integers(1, 1025, size=n_more - 3).tolist(), 64))
+    if hkv == 8:   # more (sequence, kv head)s than streaming workgroups: 480 of the grid's 512 workgroups, and all of them
+        cases.append(([1] * 60, rng.integers(1, 700, size=60).tolist(), 64))
+        cases.append(([1] * 64, rng.integers(1, 300, size=64).tolist(), 32))
     for ql, kl, pps in cases:
         b = small(ql, kl, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, pages_per_seq=pps, sliding_window=window,
                   logits_soft_cap=cap, seed=23)
