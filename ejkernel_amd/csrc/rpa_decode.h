@@ -81,7 +81,7 @@ constexpr float fp8_max() { return kKv == 2 ? 57344.f : 448.f; }
 // row of logit_pitch keys per (token, query head)) and the second launch is 3 instead of 2: the same arithmetic on the
 // stored logits, with no K rows read, no Q and no first product -- for a decode step that is 8 bytes of logits written
 // and read per key and query head against a K row of head_dim bytes per key and kv head.
-template <int D, int NT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
+template <int D, int NT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0, bool kFew = false>
 __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict__ lds_k, const SeqInfo& si, int s,
                                              int j, int rt, int range_lo, int range_hi, const Part& part) {
   using C = Cfg<D, NT, kMimic>;
@@ -452,7 +452,7 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
     return kvb + static_cast<uint64_t>(page) * page_b + static_cast<uint64_t>(t & (p.page_size - 1)) * stride_b + head_off;
   };
   if constexpr (kWaveOnly && kPass == 0 && kKv == 0) {
-    if (a.pre.sink_aux != nullptr && (!part.partial || range_lo == si.lo_al)) {
+    if (a.pre.sink_aux != nullptr && (!(part.partial || part.in_workgroup) || range_lo == si.lo_al)) {
       sink_first = kv_start_of(p, s);
       sink_keys = max(0, min(a.pre.sink_n, a.pre.sink_limit - sink_first));
       sink_part = sink_keys > 0;
@@ -581,22 +581,27 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
   bool merged = false;
   if constexpr (kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
     if (part.in_workgroup) {
-      // ---- the four wavefronts of the workgroup hold the four parts of this (sequence, kv head): wavefronts 1..3 leave
-      // their state in their own K tile (accumulator piece c of row i, lane group g at ((16 c + i) * 4 + g) * 16, then
-      // the rows' maxima and sums), wavefront 0 adds them to its own in wavefront order.  Every wavefront of the
-      // workgroup comes here, with or without keys, so the barrier is complete.
+      // ---- the four wavefronts of the workgroup hold a quarter of this part each: all but one leave their state in
+      // their own K tile (accumulator piece c of row i, lane group g at ((16 c + i) * 4 + g) * 16, then the rows'
+      // maxima and sums), the merging one adds them to its own in wavefront order.  Every wavefront of the
+      // workgroup comes here, with or without keys, so the barriers are complete.
       const int wv = static_cast<int>(threadIdx.x) / kWave;
+      const int merger = kFew ? part.merger : 0;
       constexpr int kState = 16 * D * 4;
-      if (wv != 0) {
+      if (wv != merger) {
 #pragma unroll
         for (int c = 0; c < 8; ++c) *reinterpret_cast<f32x4_t*>(lds_k + ((16 * c + i) * 4 + g) * 16) = o_acc[0][c];
         if (g == 0) *reinterpret_cast<float2*>(lds_k + kState + 8 * i) = float2{m_run, l_run};
       }
       __syncthreads();
-      if (wv != 0) return;
+      if (wv != merger) {
+        if (kFew && part.again) __syncthreads();  // (the merging wavefront has read the states: the K tiles may be written again)
+        return;
+      }
 #pragma unroll 1
-      for (int w = 1; w < kWgWaves; ++w) {
-        const char* st = lds_k + w * C::LDS_PER_WAVE;
+      for (int w = 0; w < kWgWaves; ++w) {
+        if (w == wv) continue;
+        const char* st = lds_k + (w - wv) * C::LDS_PER_WAVE;
         const float2 ml = *reinterpret_cast<const float2*>(st + kState + 8 * i);
         const float m_new = fmaxf(m_run, ml.x);
         const float m_use = m_new == -INFINITY ? 0.f : m_new;
@@ -610,10 +615,12 @@ __device__ __forceinline__ void process_item(const TileArgs& a, char* __restrict
           o_acc[0][c] = o_acc[0][c] * keep + wgt * ov;
         }
       }
+      if (kFew && part.again) __syncthreads();
       merged = true;
     }
   }
-  if (part.partial && !merged) {
+  // (kFew: what a workgroup has merged may still be one of several parts of its (sequence, kv head))
+  if (part.partial && !(merged && (!kFew || part.first_w == part.last_w))) {
     // ---- partial to the workspace, then take a ticket; the last part merges all of them in stream order.
     // Who writes, who reads: this wavefront writes its slot; the wavefront that draws the last ticket of the
     // (sequence, kv head) -- any workgroup, usually on another XCD with another L2 -- reads every slot.  Partials are

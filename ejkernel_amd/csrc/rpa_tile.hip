@@ -35,6 +35,7 @@ namespace rpa {
 
 constexpr int kWaveItemMaxRowTiles = 4;  // sequences with more 16-row tiles than this use workgroup tiles
 constexpr int kMaxMinShareTiles = 16;  // ... and the most the length of the (sequence, kv head)s raises that to
+constexpr int kFewHeads = 64;          // (sequence, kv head)s up to which a decode batch takes the kFew instantiation
 constexpr int kMinShareTiles = 2;       // tiles per streaming wavefront before more wavefronts are used
 constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to the same XCD queue
 constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
@@ -75,7 +76,9 @@ __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, c
   }
 }
 
-template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
+// kFew (with kWaveOnly): the instantiation for batches of a few dozen (sequence, kv head)s at most, where the host can
+// tell from max_num_seqs; its decode stream is cut by workgroup or by wavefront.
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0, bool kFew = false>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D, MRT, kWaveOnly, kKv>, kWavesPerSimd<D, MRT, kWaveOnly, kKv>)))
 void rpa_tile_kernel(TileArgs a) {
   constexpr int DD = D < 128 ? 128 : D;  // head_dim 64: the wave-level loop works 128 wide, prefill tiles 64 wide
@@ -301,10 +304,11 @@ void rpa_tile_kernel(TileArgs a) {
           const int per_head = (si.hi - si.lo_al + C::TT - 1) / C::TT;
           const int per_wave = (per_head + kWgWaves - 1) / kWgWaves;
           Part part;
-          part.partial = true;
+          part.partial = true;   // (no part of the split through memory: first_w = last_w)
+          part.first_w = part.last_w = 0;
           part.in_workgroup = true;
           const int lo = si.lo_al + wave * per_wave * C::TT;
-          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, lo, min(si.hi, lo + per_wave * C::TT), part);
+          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass, kFew>(a, lds_k, si, s, j, 0, lo, min(si.hi, lo + per_wave * C::TT), part);
         }
       }
     }
@@ -520,17 +524,33 @@ void rpa_tile_kernel(TileArgs a) {
         const int range_lo = max(p.sliding_window > 0 ? max(0, pos_min - p.sliding_window + 1) : 0, si.start) & ~(C::TT - 1);
         Part part;
         part.partial = false;
-        process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
+        process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass, kFew>(a, lds_k, si, s, j, rt, range_lo, range_hi, part);
       }
 
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
       if (total_tiles > 0) {
+        // Few long sequences are cut into dozens of parts each, and the merge of their partial states by one wavefront
+        // is what takes the time.  There the stream is cut by workgroup: a workgroup's part of a (sequence, kv head) is
+        // walked by its four wavefronts, a quarter each, and merged in LDS by one of them (in turn), which alone takes
+        // part in the split through memory: a quarter of the parts, of the tickets and of what the last one reads.
+        // One sequence of 32768 keys 47.3 -> 42.3 us, of 131072 keys 116 -> 108 us, two of 8192 keys 35.5 -> 30.9 us;
+        // eight of 4096 keys (16 parts each) would lose, 37.4 -> 39.4 us, and are cut by wavefront.  (In an
+        // instantiation of its own, kFew: the loop that serves both cuts costs the large batches registers, 2-4 % of
+        // their time; elsewhere unit_waves is the constant 1.)
+        int unit_waves = 1;
+        if constexpr (kFew && kWaveOnly && kPass == 0 && kKv == 0 && C::NS == 1 && C::LDS_PER_WAVE >= 16 * D * 4 + 128) {
+          const float avg = static_cast<float>(total_tiles) / static_cast<float>(max(1, nseq * item_heads));
+          const int by_len = max(a.min_share_tiles, min(kMaxMinShareTiles, static_cast<int>(__builtin_sqrtf(avg) * (1.f / 3.f))));
+          const int share = max(by_len, total_tiles / n_workers);  // tiles per part, cut by wavefront
+          if (a.wg_unit_parts > 0 && avg >= static_cast<float>(a.wg_unit_parts) * static_cast<float>(share)) unit_waves = kWgWaves;
+        }
+        const int n_units = n_workers / unit_waves, unit = worker / unit_waves;
         Shares sh;
         {
           // Weighted regions when every wavefront gets a few tiles at least.  Small batches use fewer wavefronts
           // instead, kMinShareTiles tiles each: a (sequence, kv head) cut into many one-tile parts would spend its
           // time in the merge, which reads the parts one after the other.
-          const int q = total_tiles / n_workers, half = n_workers / 2;
+          const int q = total_tiles / n_units, half = n_units / 2;
           // With T tiles per (sequence, kv head) cut into P parts a wavefront streams T / P tiles and the merge reads P
           // parts, a few at a time: the sum is smallest near P = 3 sqrt(T), i.e. sqrt(T) / 3 tiles per part.
           int min_share = a.min_share_tiles;
@@ -538,18 +558,20 @@ void rpa_tile_kernel(TileArgs a) {
             const float avg = static_cast<float>(total_tiles) / static_cast<float>(max(1, nseq * item_heads));
             min_share = max(min_share, min(kMaxMinShareTiles, static_cast<int>(__builtin_sqrtf(avg) * (1.f / 3.f))));
           }
+          min_share *= unit_waves;
           if (q >= min_share) {
-            const int rem = total_tiles - q * n_workers;
+            const int rem = total_tiles - q * n_units;
             int first_tiles = half * q + min(half, rem);
             if (by_xcd) first_tiles = static_cast<int>(static_cast<long long>(total_tiles) * a.even_xcd_permille / 1000);
-            sh.set(total_tiles, n_workers, half, first_tiles);
+            sh.set(total_tiles, n_units, half, first_tiles);
           } else {
             const int n_active = max(1, total_tiles / min_share);
             sh.set(total_tiles, n_active, n_active, total_tiles);  // one evenly cut region; the other wavefronts get nothing
           }
         }
-        int x = sh.begin(worker);
-        const int x_end = sh.begin(worker + 1);
+        int x = sh.begin(unit);
+        const int x_end = sh.begin(unit + 1);
+        int n_parts = 0;
         while (x < x_end) {
           int s_base;
           const int s = find(tile_start, 1, x, s_base);
@@ -573,8 +595,20 @@ void rpa_tile_kernel(TileArgs a) {
           part.first_w = sh.owner(part.stream_a);
           part.last_w = sh.owner(part.stream_a + per_head - 1);
           part.partial = part.first_w != part.last_w;
-          part.slot = part_slot(worker, part.stream_a, sh);
-          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass>(a, lds_k, si, s, j, 0, si.lo_al + t0 * C::TT, min(si.hi, si.lo_al + min(t1, per_head) * C::TT), part);
+          part.slot = part_slot(unit, part.stream_a, sh);
+          int lo = t0, hi = min(t1, per_head);
+          if constexpr (kFew) {
+            if (unit_waves > 1) {
+              const int per_wave = (hi - lo + kWgWaves - 1) / kWgWaves;
+              lo += wave * per_wave;
+              hi = min(hi, lo + per_wave);
+              part.in_workgroup = true;
+              part.merger = n_parts & (kWgWaves - 1);
+              part.again = true;
+              ++n_parts;
+            }
+          }
+          process_item<DD, NT, kMimic, kWaveOnly, kKv, kPass, kFew>(a, lds_k, si, s, j, 0, si.lo_al + lo * C::TT, min(si.hi, si.lo_al + hi * C::TT), part);
           x += t1 - t0;
         }
       }
@@ -605,6 +639,7 @@ struct Tune {
   int no_logit_stash;      // RPA_TUNE_NO_LOGIT_STASH: two-launch calls read K in both launches (experiments)
   int device_select;       // RPA_TUNE_DEVICE_SELECT: 0 = never enqueue both tile kernels and let the device pick
   int wg_item_tiles;       // RPA_TUNE_WG_ITEM_TILES: longest (sequence, kv head), in tiles, of a batch that runs one per workgroup
+  int wg_unit_parts;       // RPA_TUNE_WG_UNIT_PARTS: parts per (sequence, kv head) from which few sequences are cut by workgroup
 };
 static const Tune& tune() {
   static const Tune t = [] {
@@ -629,6 +664,7 @@ static const Tune& tune() {
     x.no_logit_stash = env_int("RPA_TUNE_NO_LOGIT_STASH", 0);
     x.device_select = env_int("RPA_TUNE_DEVICE_SELECT", 1);
     x.wg_item_tiles = max(0, env_int("RPA_TUNE_WG_ITEM_TILES", 32));
+    x.wg_unit_parts = max(0, env_int("RPA_TUNE_WG_UNIT_PARTS", 32));
     return x;
   }();
   return t;
@@ -703,7 +739,7 @@ uint64_t logit_stash_bytes(const RpaParams& p) {
   return bytes <= kLogitStashMaxBytes ? bytes : 0;
 }
 
-template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0>
+template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0, bool kFew = false>
 static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   using C = Cfg<(D < 128 ? 128 : D), NT, kMimic>;
   using PC = PCfg<D, MRT>;
@@ -715,12 +751,12 @@ static int launch_cfg(const TileArgs& a, int grid, hipStream_t stream) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
   if (allowed[dev].load(std::memory_order_acquire) < lds) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass, kFew>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(lds)) != hipSuccess)
       return RPA_ERR_LAUNCH;
     allowed[dev].store(lds, std::memory_order_release);
   }
-  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass>), dim3(grid), dim3(kWgThreads), lds, stream, a);
+  hipLaunchKernelGGL((rpa_tile_kernel<D, NT, MRT, kMimic, kWaveOnly, kKv, kPass, kFew>), dim3(grid), dim3(kWgThreads), lds, stream, a);
   return hipGetLastError() == hipSuccess ? RPA_OK : RPA_ERR_LAUNCH;
 }
 
@@ -770,6 +806,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.pair = 0;
   a.select = 0;
   a.wg_item_tiles = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_item_tiles;  // a caller that names the split gets the split
+  a.wg_unit_parts = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_unit_parts;
   // The wavefronts on odd XCDs stream about a tenth slower when all eight compete for memory; per-XCD exit times put the
   // balance at 54.0 % of the stream on the even ones with 256-byte rows and at 54.7 % with 512-byte rows (head_dim 256:
   // even XCDs left at 329 us, odd ones at 338 with 54.0 %; 0.3571 -> 0.3532 ms with 54.7 %).
@@ -824,8 +861,15 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     a.pair = p.head_dim == 64 && p.num_kv_heads % 2 == 0 && 2 * (p.num_q_heads / p.num_kv_heads) <= 16 && pre.ml == nullptr &&
              pre.sink_aux == nullptr && tune().no_pair64 == 0;
     if (a.pair) a.stream_grid = device_cu_count() * (tune().decode_wgs_per_cu > 0 ? tune().decode_wgs_per_cu : 1);
-    if (p.head_dim <= 128)
+    if (p.head_dim <= 128) {
+      // few sequences (what max_num_seqs allows is all the host knows): the instantiation that can also cut the decode
+      // stream by workgroup, for the long ones among them
+      const int heads = a.pair ? p.num_kv_heads / 2 : p.num_kv_heads;
+      if (static_cast<int64_t>(p.max_num_seqs) * heads <= kFewHeads && a.wg_unit_parts > 0)
+        return mimic ? launch_cfg<128, 2, 2, true, true, 0, 0, true>(a, grid, stream)
+                     : launch_cfg<128, 2, 2, false, true, 0, 0, true>(a, grid, stream);
       return mimic ? launch_cfg<128, 2, 2, true, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, true>(a, grid, stream);
+    }
     // head_dim 256: one workgroup per compute unit with the whole register file
     a.stream_grid = device_cu_count();
     return mimic ? launch_cfg<256, 1, 1, true, true>(a, a.stream_grid, stream) : launch_cfg<256, 1, 1, false, true>(a, a.stream_grid, stream);

@@ -52,6 +52,10 @@ struct TileArgs {
   // A batch of few, short decode sequences: up to how many tiles a (sequence, kv head) may have for the batch to run
   // one workgroup per (sequence, kv head), its four wavefronts merging through LDS (0 = never).
   int wg_item_tiles;
+  // Kernels for few sequences (kFew): from how many parts per (sequence, kv head) on, were it cut by wavefront, the decode
+  // stream is cut by workgroup: a workgroup's share of a (sequence, kv head) is walked by its four wavefronts, a quarter
+  // each, and merged in LDS, so a (sequence, kv head) has a quarter of the parts that go through memory (0 = never).
+  int wg_unit_parts;
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the
@@ -100,7 +104,9 @@ struct Shares {
 // A wavefront's part of one (sequence, kv head) of the decode stream.
 struct Part {
   bool partial;         // the (sequence, kv head) is shared with other wavefronts
-  bool in_workgroup = false;  // ... with the other wavefronts of this workgroup and no one else: they merge through LDS
+  bool in_workgroup = false;  // the four wavefronts of the workgroup hold a quarter of this part each and merge through LDS
+  int merger = 0;             // ... into this wavefront, which then stands for the part (kFew kernels; 0 elsewhere)
+  bool again = false;         // ... and the workgroup goes on to another part: a second barrier before the K tiles are written anew
   int slot;             // workspace slot of this part
   int first_w, last_w;  // wavefronts sharing it (every one of them holds at least one of its tiles)
   int stream_a;         // stream index of its first tile

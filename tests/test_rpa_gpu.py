@@ -134,12 +134,18 @@ def test_bf16_gqa_ratios(flags, hq, hkv):
 def test_bf16_few_long_sequences_split_into_many_parts(hq, hkv, q_len, D):
     """One or two long sequences on the whole grid: every (sequence, kv head) is cut into dozens of parts, which the
     last wavefront to arrive merges several at a time on the lanes of the rows a decode tile does not have (1, 2, 4,
-    8 or 16 rows per tile here, 3 and 6 padded to 4 and 8).  Parity, and the same bits on every call."""
+    8 or 16 rows per tile here, 3 and 6 padded to 4 and 8).  Parity, and the same bits on every call.
+    With so few (sequence, kv head)s the stream is cut by workgroup up to head_dim 128 (four wavefronts a quarter of
+    the workgroup's share each, merged in LDS, then the split through memory over a quarter of the parts); a
+    `num_kv_pages_per_block` names the cut and gives the one by wavefront, which must agree."""
     b = small([q_len, q_len], [8192, 5000], num_q_heads=hq, num_kv_heads=hkv, pages_per_seq=512, head_dim=D)
     out = run_hip(b)
     assert_bf16_parity(to_np(out), run_strict(b), b.total_valid_tokens, f"{hq}/{hkv} q_len {q_len} D {D}")
     for _ in range(3):
         assert torch.equal(run_hip(b), out)
+    by_wave = run_hip(b, cfg=RaggedPageAttentionConfig(num_kv_pages_per_block=8))
+    assert_bf16_parity(to_np(by_wave), run_strict(b), b.total_valid_tokens, "cut by wavefront")
+    assert (out.float() - by_wave.float()).abs().max().item() <= 2e-2
     assert_bf16_parity(to_np(run_hip(b, _native.RPA_FLAG_PREFILL_TILES)), run_strict(b), b.total_valid_tokens, "tiles")
 
 
