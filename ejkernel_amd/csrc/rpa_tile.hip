@@ -41,12 +41,12 @@ constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to
 constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
 constexpr int kWaveOnlyMaxRows = 20480;   // (token, query head) rows up to which a batch runs without prefill tiles
 
-// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 8 ints of scratch and the sequences with prefill
+// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 16 ints of scratch and the sequences with prefill
 // tiles in order of length (up to kSortMax ints), then the data region
 // shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
 __host__ __device__ constexpr int sort_entries(int max_num_seqs) { return max_num_seqs < kSortMax ? max_num_seqs : kSortMax; }
 __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
-  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 8 + sort_entries(max_num_seqs)) * sizeof(int) + 15) &
+  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 16 + sort_entries(max_num_seqs)) * sizeof(int) + 15) &
          ~static_cast<size_t>(15);
 }
 
@@ -76,6 +76,15 @@ __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, c
   }
 }
 
+// A wave-uniform value the compiler cannot see through.  The kinds of work of the kernel below sit in one loop over
+// its two phases, and out of a loop the compiler hoists every invariant of every kind in front of it -- shares of the
+// stream, queue sizes, divisions by run-time values, some eight hundred scalar instructions that a small launch then
+// waits two microseconds for whatever it holds.  Sums that enter a section through this stay inside it.
+__device__ __forceinline__ int kept_in_place(int x) {
+  asm volatile("" : "+s"(x));
+  return x;
+}
+
 // kFew (with kWaveOnly): the instantiation for batches of a few dozen (sequence, kv head)s at most, where the host can
 // tell from max_num_seqs; its decode stream is cut by workgroup or by wavefront.
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0, bool kFew = false>
@@ -99,7 +108,7 @@ void rpa_tile_kernel(TileArgs a) {
   int* tile_start = item_start + (sched_n + 1);     // decode stream tiles
   int* wg_start = tile_start + (sched_n + 1);       // workgroup-level prefill tiles
   int* scratch = wg_start + (sched_n + 1);
-  int* wg_seq = scratch + 8;                        // sequence of the r-th entry of wg_start, when those are sorted
+  int* wg_seq = scratch + 16;                       // sequence of the r-th entry of wg_start, when those are sorted
   char* lds_data = smem + sched_bytes(sched_n);
   char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
@@ -124,17 +133,32 @@ void rpa_tile_kernel(TileArgs a) {
   const int per = (((nseq + kWgThreads - 1) / kWgThreads + K - 1) >> shift) << shift;  // a multiple of K per thread
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
   int my_items = 0, my_tiles = 0, my_wg = 0;
+  int my_cost = 0;  // TileArgs::select: prefill work in units of 1024 (query row, key) pairs, see below
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
-    classify(seq_info<C::TT>(a, s, G), t, it, wg);
+    const SeqInfo si = seq_info<C::TT>(a, s, G);
+    classify(si, t, it, wg);
     my_tiles += t;
     my_items += it;
     my_wg += wg;
+    if constexpr (!kWaveOnly && kKv == 0) {
+      if (a.select != 0 && wg > 0) {
+        const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
+        my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
+      }
+    }
   }
-  int total_items, total_tiles, total_wg;
-  int item_base = block_excl_scan(my_items, scratch, total_items);
-  int tile_base = block_excl_scan(my_tiles, scratch, total_tiles);
-  int wg_base = block_excl_scan(my_wg, scratch, total_wg);
+  // (all four sums behind one pair of barriers: a small launch is a chain of such waits)
+  int total_items, total_tiles, total_wg, total_cost;
+  int item_base, tile_base, wg_base;
+  {
+    const int mine[4] = {my_items, my_tiles, my_wg, my_cost};
+    int base[4], total[4];
+    block_excl_scan4(mine, scratch, base, total);
+    item_base = base[0], tile_base = base[1], wg_base = base[2];
+    total_items = total[0], total_tiles = total[1], total_wg = total[2];
+    total_cost = __builtin_amdgcn_readfirstlane(total[3]);
+  }
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
     classify(seq_info<C::TT>(a, s, G), t, it, wg);
@@ -172,19 +196,7 @@ void rpa_tile_kernel(TileArgs a) {
   // pipelined tiles are worth it from seven tenths of the stream's time on.
   if constexpr (!kWaveOnly && kKv == 0) {
     if (a.select != 0) {
-      int my_cost = 0;
-      for (int s = s_begin; s < s_end; ++s) {
-        const SeqInfo si = seq_info<C::TT>(a, s, G);
-        if (!si.eligible && si.n_rt > kWaveItemMaxRowTiles) {
-          const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
-          my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
-        }
-      }
-      int total_cost;
-      block_excl_scan(my_cost, scratch, total_cost);
-      total_cost = __builtin_amdgcn_readfirstlane(total_cost);
       const bool pick_pipe = 10ll * total_cost >= 35ll * total_tiles;
-      __syncthreads();
       if ((a.select == 2) != pick_pipe) return;
     }
   }
@@ -195,7 +207,11 @@ void rpa_tile_kernel(TileArgs a) {
   // length; wg_seq names them.  The data region, not yet in use, holds the temporaries.
   int n_sorted = 0;
   if constexpr (!kWaveOnly) {
-    if (total_wg > 0 && shift == 0 && a.phase_mode == 4) {
+    // (With no more tiles than workgroups that begin with tiles every tile starts at once and the order is of no
+    // consequence: the sort, two microseconds of a launch that takes thirty, is left out.)
+    const int begin_with_tiles = static_cast<int>(gridDim.x) > a.decode_grid && (total_tiles > 0 || total_items > 0)
+                                     ? a.decode_grid : static_cast<int>(gridDim.x);
+    if (total_wg > begin_with_tiles && shift == 0 && a.phase_mode == 4) {
       int mine = 0;
       for (int s = s_begin; s < s_end; ++s) {
         int t, it, wg;
@@ -376,6 +392,7 @@ void rpa_tile_kernel(TileArgs a) {
       // row tiles that share one K/V stream should run at the same time on the same XCD, so that all but the first
       // of them read it from that L2.
       if (queued) {
+        const int total_wg_here = kept_in_place(total_wg);
         // Eight queues, one per XCD: aligned runs of kQueueRun consecutive items go to the queues in turn.  A
         // workgroup draws from the queue of its own XCD until that is empty, then from the others.  Within a
         // (sequence, kv head) the late causal tiles (most keys) come first.  The last workgroup to find every
@@ -392,7 +409,7 @@ void rpa_tile_kernel(TileArgs a) {
         auto owned = [&](int x) { return n_first > x ? (n_first - x + 7) >> 3 : 0; };    // ... and have home queue x
         // items of queue x: its full runs (run r belongs to queue r % 8) and the partial last run if it is x's
         auto items_of = [&](int x) {
-          const int runs = total_wg / kQueueRun, rem = total_wg - runs * kQueueRun;
+          const int runs = total_wg_here / kQueueRun, rem = total_wg_here - runs * kQueueRun;
           return (runs > x ? (runs - x + 7) >> 3 : 0) * kQueueRun + ((runs & 7) == x ? rem : 0);
         };
         int probe = 0;
@@ -422,7 +439,7 @@ void rpa_tile_kernel(TileArgs a) {
               first = false;
               if (t >= 0) {
                 const int cand = ((t / kQueueRun) * 8 + x) * kQueueRun + t % kQueueRun;
-                if (cand < total_wg) {
+                if (cand < total_wg_here) {
                   res = cand;
                   break;
                 }
@@ -511,8 +528,10 @@ void rpa_tile_kernel(TileArgs a) {
       __syncthreads();
       }
     } else if (do_stream) {
+      const int total_items_here = kept_in_place(total_items), total_tiles_here = kept_in_place(total_tiles);
+      const int n_workers_here = kept_in_place(n_workers);
       // ---- sequences with a few row tiles: one item per (sequence, row tile, kv head), strided over the wavefronts
-      for (int w = worker; w < total_items; w += n_workers) {
+      for (int w = worker; w < total_items_here; w += n_workers_here) {
         int s_base;
         const int s = find(item_start, 0, w, s_base);
         const SeqInfo si = seq_info<C::TT>(a, s, G);
@@ -528,7 +547,8 @@ void rpa_tile_kernel(TileArgs a) {
       }
 
       // ---- decode stream: this wavefront's share [x, x_end) of the tiles, cut at (sequence, kv head) boundaries
-      if (total_tiles > 0) {
+      if (total_tiles_here > 0) {
+        const int total_tiles = total_tiles_here, n_workers = n_workers_here;  // (the section's own copies, see kept_in_place)
         // Few long sequences are cut into dozens of parts each, and the merge of their partial states by one wavefront
         // is what takes the time.  There the stream is cut by workgroup: a workgroup's part of a (sequence, kv head) is
         // walked by its four wavefronts, a quarter each, and merged in LDS by one of them (in turn), which alone takes

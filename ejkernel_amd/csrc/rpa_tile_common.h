@@ -169,6 +169,39 @@ __device__ __forceinline__ int block_excl_scan(int v, int* wave_tot, int& total)
   return base + inc - v;
 }
 
+// Four such sums at once behind one pair of barriers (wave_tot: 4 * kWgWaves ints): v and total are arrays of four,
+// base receives the exclusive prefix sums.
+__device__ __forceinline__ void block_excl_scan4(const int (&v)[4], int* wave_tot, int (&base)[4], int (&total)[4]) {
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int inc[4] = {v[0], v[1], v[2], v[3]};
+#pragma unroll
+  for (int o = 1; o < kWave; o <<= 1) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int t = __shfl_up(inc[k], o, kWave);
+      if (lane >= o) inc[k] += t;
+    }
+  }
+  __syncthreads();
+  if (lane == kWave - 1) {
+#pragma unroll
+    for (int k = 0; k < 4; ++k) wave_tot[4 * wave + k] = inc[k];
+  }
+  __syncthreads();
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    int b = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kWgWaves; ++w) {
+      const int t = wave_tot[4 * w + k];
+      if (w < wave) b += t;
+      tot += t;
+    }
+    total[k] = tot;
+    base[k] = b + inc[k] - v[k];
+  }
+}
+
 // Hardware round-to-nearest-even conversions (v_cvt_pk_bf16_f32): branch-free, NaN stays NaN.
 typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2_t;
 __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
