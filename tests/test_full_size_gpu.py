@@ -32,7 +32,16 @@ def run(b):
 
 def check_sample(b, out, n_seqs, seed=0):
     rng = np.random.default_rng(seed)
-    ids = sorted(int(s) for s in rng.permutation(len(b.q_lens))[:n_seqs])
+    order = [int(s) for s in rng.permutation(len(b.q_lens))]
+    if b.sliding_window:
+        # The reference program turns a row NaN when one of its 64-page KV blocks lies entirely left of the row's window,
+        # and such rows can only be held against the float64 evaluation.  Half of the sample is therefore taken from
+        # the sequences short enough to have no such block, so that the restatement of the program itself is what
+        # checks a windowed workload too.
+        short = [s for s in order if b.kv_lens[s] < b.sliding_window + 64 * b.meta["page_size"]]
+        head = short[: n_seqs // 2]
+        order = head + [s for s in order if s not in head]
+    ids = sorted(order[:n_seqs])
     sub = compact_for_host(b, ids)
     ref = rpa_oracle_c.rpa_strict_c(*oracle_args(sub), softmax_scale=sub.softmax_scale,
                                     logits_soft_cap=sub.logits_soft_cap, sliding_window=sub.sliding_window)
@@ -43,6 +52,8 @@ def check_sample(b, out, n_seqs, seed=0):
     got = to_np(out[sub.meta["rows"].to(out.device)])
     mx, mean = err_stats(got, ref, rows)
     assert mx <= BF16_MAX_ABS and mean <= BF16_MEAN_ABS, (b.name, mx, mean)
+    if b.sliding_window and any(b.kv_lens[s] < b.sliding_window + 64 * b.meta["page_size"] for s in ids):
+        assert nan_rows.sum() < rows, "no row of the sample was checked against the restatement of the program"
     return sub, int(nan_rows.sum())
 
 
@@ -59,7 +70,7 @@ def permuted(b, seed=9):
 
 @pytest.mark.parametrize("name,n_sample,permute", [("decode_small", 8, True), ("decode_llama3_8b", 12, True),
                                                    ("mixed_prefill_decode", 14, True), ("mixed_prefill_only", 3, True),
-                                                   ("gemma2_local", 4, False), ("decode_long_context", 2, False),
+                                                   ("gemma2_local", 8, False), ("decode_long_context", 5, False),
                                                    ("decode_head_dim_96", 12, True), ("mixed_head_dim_96", 10, True),
                                                    ("prefill_head_dim_256", 1, True), ("decode_head_dim_64", 12, True)])
 def test_full_size_workload(name, n_sample, permute):
