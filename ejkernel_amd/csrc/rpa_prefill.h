@@ -74,7 +74,7 @@ constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point b
 // them and accumulates P V with no rescaling.
 template <int D, int MRT, bool kMimic, int kKv = 0, int kPass = 0>
 __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
-                                             int qt) {
+                                             int qt, int part = 0, int parts = 1, int tile_id = 0) {
   using C = PCfg<D, MRT>;
   static_assert(kKv == 0 || C::NSTG == 2, "the register stage of an 8-bit cache stands in for one LDS stage ahead");
   static_assert((kKv == 0) == (kPass == 0), "an 8-bit cache runs as two passes, a 16-bit cache as one");
@@ -104,8 +104,15 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // ---- key range of the workgroup's rows
   const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
   const int wg_pos_min = pos0 + wg_row_lo / G, wg_pos_max = pos0 + (wg_row_hi - 1) / G;
-  const int range_hi = min(si.kv_len, wg_pos_max + 1);
-  const int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
+  int range_hi = min(si.kv_len, wg_pos_max + 1);
+  int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
+  // A batch of few tiles (TileArgs::tile_split): the key range is cut into `parts` runs of whole key tiles, one
+  // workgroup each, whose states meet in the workspace (below).  A run may be empty.
+  if (kPass == 0 && parts > 1) {
+    const int n_kt = (max(range_hi - range_lo, 0) + C::TK - 1) / C::TK, per = (n_kt + parts - 1) / parts;
+    range_lo = min(range_lo + part * per * C::TK, range_hi);
+    range_hi = min(range_hi, range_lo + per * C::TK);
+  }
   const int t_last = range_hi - 1;
 
   // ---- this wavefront's rows: row tile m holds rows w_row_lo + 16 m + i
@@ -641,6 +648,89 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     }
   }
 
+  // ---- a part of a split key range: the state of every row -- reference point, sum, unnormalised output -- goes to
+  // the workspace as it sits in registers (accumulator c of row tile m and slice sN of this wavefront: 1 KiB in lane
+  // order), the workgroup takes a ticket of its tile, and the one that draws the last ticket adds the parts up in
+  // part order (its own included, so the result does not depend on who comes last) and goes on to normalise and
+  // store.  Written and read at agent scope like the partial states of the decode stream.
+  float m_merged[MRT], l_merged[MRT];
+  if constexpr (kPass == 0) {
+    if (parts > 1) {
+      // (fresh names for the accumulators: what this seldom-run block does with them must not shape the registers
+      // they have in the key loop)
+#pragma unroll
+      for (int m = 0; m < MRT; ++m)
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int c = 0; c < C::CB; ++c) asm volatile("" : "+v"(o_acc[m][sN][c]));
+      constexpr int kAgentScope = 16;
+      constexpr uint32_t kWaveState = MRT * C::NS * C::CB * 1024, kPartState = kWgWaves * kWaveState;  // bytes
+      const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(a.partial_o, 0, 0x7fffffff, 0x00020000);
+      float2* ml = reinterpret_cast<float2*>(a.partial_ml);
+      const uint32_t my_part = static_cast<uint32_t>(tile_id * parts + part);
+      auto state_off = [&](uint32_t pt, int m, int sN, int c) {
+        return static_cast<int>(pt * kPartState + wave * kWaveState + ((m * C::NS + sN) * C::CB + c) * 1024 + lane * 16);
+      };
+#pragma unroll
+      for (int m = 0; m < MRT; ++m) {
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int c = 0; c < C::CB; ++c)
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, o_acc[m][sN][c]), o_rsrc, state_off(my_part, m, sN, c), 0, kAgentScope);
+        if (g == 0) {
+          const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+          const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_row)) | (static_cast<uint64_t>(__float_as_uint(l_acc[m][0])) << 32);
+          __hip_atomic_store(reinterpret_cast<uint64_t*>(ml) + (my_part * kWgWaves + wave) * (16 * MRT) + 16 * m + i, v,
+                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();  // every wavefront's state has left (and every wavefront is out of the key loop's LDS)
+      uint32_t* ctr = a.counters + a.tile_ticket_base + tile_id;
+      int* flag = reinterpret_cast<int*>(lds);
+      if (threadIdx.x == 0)
+        *flag = static_cast<int>(__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      __syncthreads();
+      const int ticket = *flag;
+      __syncthreads();  // (the flag's word belongs to the next tile's stage from here on)
+      if (ticket != parts - 1) return;
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+      for (int m = 0; m < MRT; ++m) {
+        float M = -INFINITY, L = 0.f;
+#pragma unroll
+        for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+          for (int c = 0; c < C::CB; ++c) o_acc[m][sN][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int pt = 0; pt < parts; ++pt) {
+          const uint32_t src = static_cast<uint32_t>(tile_id * parts + pt);
+          const uint64_t v = __hip_atomic_load(reinterpret_cast<const uint64_t*>(ml) + (src * kWgWaves + wave) * (16 * MRT) + 16 * m + i,
+                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const float mk = __uint_as_float(static_cast<uint32_t>(v)), lk = __uint_as_float(static_cast<uint32_t>(v >> 32));
+          const float m_new = fmaxf(M, mk);
+          const float m_use = m_new == -INFINITY ? 0.f : m_new;
+          const float keep = __builtin_amdgcn_exp2f((M - m_use) * kLog2e);
+          const float w = __builtin_amdgcn_exp2f((mk - m_use) * kLog2e);
+          L = L * keep + w * lk;
+          M = m_new;
+#pragma unroll
+          for (int sN = 0; sN < C::NS; ++sN)
+#pragma unroll
+            for (int c = 0; c < C::CB; ++c) {
+              const u32x4_t ov = __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, state_off(src, m, sN, c), 0, kAgentScope);
+              o_acc[m][sN][c] = o_acc[m][sN][c] * keep + w * __builtin_bit_cast(f32x4_t, ov);
+            }
+        }
+        m_merged[m] = M;
+        l_merged[m] = L;
+      }
+      if (threadIdx.x == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+
   // ---- normalise (with optional sinks) and store
 #pragma unroll
   for (int m = 0; m < MRT; ++m) {
@@ -652,7 +742,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     row_of(m, opaque0, valid, head, q_off);
     const float l_row1 = kPass == 1 ? row_groups_sum(l32[m]) : 0.f;  // the four lanes of a row, every lane taking part
     if (!valid) continue;
-    const float m_row = m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+    const float m_row = kPass == 0 && parts > 1 ? m_merged[m] : m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
     if constexpr (kPass == 1) {
       if (g == 0) {
         float* st = a.stats + 2 * (q_off / hd);  // q_off = ((q0 + qi) * num_q_heads + head) * head_dim
@@ -661,7 +751,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       }
       continue;
     }
-    const float l_run = l_acc[m][0];
+    const float l_run = kPass == 0 && parts > 1 ? l_merged[m] : l_acc[m][0];
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;

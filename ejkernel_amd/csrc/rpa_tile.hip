@@ -67,12 +67,13 @@ template <int D, int MRT, bool kWaveOnly, int kKv>
 constexpr int kWavesPerSimd = kPipeTile<D, MRT> || kWideDecode<D, MRT, kWaveOnly, kKv> ? 1 : 2;
 
 template <int D, int MRT, bool kMimic, int kKv, int kPass>
-__device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt) {
+__device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt,
+                                                 int part = 0, int parts = 1, int tile_id = 0) {
   if constexpr (kPipeTile<D, MRT>) {
     static_assert(kKv == 0, "the pipelined tile reads a 16-bit cache");
     prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
   } else {
-    prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds, si, s, j, qt);
+    prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds, si, s, j, qt, part, parts, tile_id);
   }
 }
 
@@ -142,7 +143,7 @@ void rpa_tile_kernel(TileArgs a) {
     my_items += it;
     my_wg += wg;
     if constexpr (!kWaveOnly && kKv == 0) {
-      if (a.select != 0 && wg > 0) {
+      if ((a.select != 0 || a.tile_split > 1) && wg > 0) {
         const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
         my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
       }
@@ -198,6 +199,20 @@ void rpa_tile_kernel(TileArgs a) {
     if (a.select != 0) {
       const bool pick_pipe = 10ll * total_cost >= 35ll * total_tiles;
       if ((a.select == 2) != pick_pipe) return;
+    }
+  }
+
+  // ---- a launch of few prefill tiles and nothing to stream -- one chunk of 512 tokens after 2048 is 128 tiles for 512
+  // workgroups, each walking 40 key tiles alone: every tile's key range is cut into `key_split` runs, a workgroup each
+  // (TileArgs::tile_split), as many as leaves every part a workgroup of its own and four key tiles by the batch's
+  // average (total_cost counts 1024 (query row, key) pairs).
+  int key_split = 1;
+  if constexpr (!kWaveOnly && kKv == 0 && kPass == 0 && !kPipeTile<D, MRT>) {
+    if (a.tile_split > 1 && total_wg > 0 && total_tiles == 0 && a.phase_mode == 4 && shift == 0 &&
+        a.tile_ticket_base + total_wg <= static_cast<int>(kQueueCounterIndex)) {
+      const long long key_tiles = (static_cast<long long>(total_cost) << 10) / (static_cast<long long>(total_wg) * PC::WGROWS * PC::TK);
+      key_split = min(min(a.tile_split, static_cast<int>(gridDim.x) / total_wg), min(static_cast<int>(key_tiles / 4), a.tile_parts_cap / total_wg));
+      key_split = __builtin_amdgcn_readfirstlane(max(key_split, 1));
     }
   }
 
@@ -392,7 +407,7 @@ void rpa_tile_kernel(TileArgs a) {
       // row tiles that share one K/V stream should run at the same time on the same XCD, so that all but the first
       // of them read it from that L2.
       if (queued) {
-        const int total_wg_here = kept_in_place(total_wg);
+        const int total_wg_here = kept_in_place(total_wg) * key_split;  // work items: the tiles, or the parts of the tiles
         // Eight queues, one per XCD: aligned runs of kQueueRun consecutive items go to the queues in turn.  A
         // workgroup draws from the queue of its own XCD until that is empty, then from the others.  Within a
         // (sequence, kv head) the late causal tiles (most keys) come first.  The last workgroup to find every
@@ -455,18 +470,19 @@ void rpa_tile_kernel(TileArgs a) {
           probe = __builtin_amdgcn_readfirstlane(scratch[1]);
           __syncthreads();
           if (w < 0) break;
+          const int wt = key_split > 1 ? w / key_split : w, part = w - wt * key_split;  // the tile, and which run of its keys
           int s_base, s;
           if (n_sorted > 0) {
             int lo = 0, hi = n_sorted;
             while (hi - lo > 1) {
               const int mid = (lo + hi) >> 1;
-              if (wg_start[mid] <= w) lo = mid; else hi = mid;
+              if (wg_start[mid] <= wt) lo = mid; else hi = mid;
             }
             lo = __builtin_amdgcn_readfirstlane(lo);
             s = __builtin_amdgcn_readfirstlane(wg_seq[lo]);
             s_base = __builtin_amdgcn_readfirstlane(wg_start[lo]);
           } else {
-            s = find(wg_start, 2, w, s_base);
+            s = find(wg_start, 2, wt, s_base);
           }
           const SeqInfo si = seq_info<C::TT>(a, s, G);
           const int n_qt = (si.rows + PC::WGROWS - 1) / PC::WGROWS;
@@ -474,7 +490,7 @@ void rpa_tile_kernel(TileArgs a) {
           // causal tiles) of every kv head before the next shorter ones.  Head by head instead, the longest tiles of
           // the last head would start when most of the prompt is done and finish alone (a tenth of the time of two
           // 8192-token prompts).
-          const int local = w - s_base;
+          const int local = wt - s_base;
           const int full = n_qt / kQueueRun, per_round = kQueueRun * p.num_kv_heads;
           int j, member;
           if (local < full * per_round) {
@@ -486,7 +502,7 @@ void rpa_tile_kernel(TileArgs a) {
             j = rem / sz;
             member = full * kQueueRun + (rem - j * sz);
           }
-          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, n_qt - 1 - member);
+          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, n_qt - 1 - member, part, key_split, wt);
         }
         // The last workgroup out clears the counters for the next launch; the exit counts are kept per XCD and
         // then over the XCDs, so that the workgroups of a small batch, which all leave at once, do not queue up on one word.
@@ -659,6 +675,7 @@ struct Tune {
   int no_logit_stash;      // RPA_TUNE_NO_LOGIT_STASH: two-launch calls read K in both launches (experiments)
   int device_select;       // RPA_TUNE_DEVICE_SELECT: 0 = never enqueue both tile kernels and let the device pick
   int wg_item_tiles;       // RPA_TUNE_WG_ITEM_TILES: longest (sequence, kv head), in tiles, of a batch that runs one per workgroup
+  int tile_split;          // RPA_TUNE_TILE_SPLIT: most runs a prefill tile's key range is cut into when tiles are few
   int wg_unit_parts;       // RPA_TUNE_WG_UNIT_PARTS: parts per (sequence, kv head) from which few sequences are cut by workgroup
 };
 static const Tune& tune() {
@@ -685,6 +702,7 @@ static const Tune& tune() {
     x.device_select = env_int("RPA_TUNE_DEVICE_SELECT", 1);
     x.wg_item_tiles = max(0, env_int("RPA_TUNE_WG_ITEM_TILES", 32));
     x.wg_unit_parts = max(0, env_int("RPA_TUNE_WG_UNIT_PARTS", 32));
+    x.tile_split = max(0, env_int("RPA_TUNE_TILE_SPLIT", 4));
     return x;
   }();
   return t;
@@ -827,6 +845,16 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   a.select = 0;
   a.wg_item_tiles = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_item_tiles;  // a caller that names the split gets the split
   a.wg_unit_parts = p.num_kv_pages_per_block > 0 ? 0 : tune().wg_unit_parts;
+  {
+    // parts of split prefill tiles in the workspace: 64 KiB of accumulators each (128 rows x 128 elements, 256 x 64,
+    // 64 x 256) and 8 bytes per row
+    WorkspaceLayout wl;
+    tiled_workspace_layout(p, &wl);
+    const uint64_t rows = p.head_dim <= 64 ? 256 : p.head_dim <= 128 ? 128 : 64;
+    a.tile_split = tune().tile_split;
+    a.tile_parts_cap = static_cast<int>(std::min<uint64_t>(wl.partial_o_bytes >> 16, wl.partial_ml_bytes / (8 * rows)));
+    a.tile_ticket_base = p.max_num_seqs * p.num_kv_heads;
+  }
   // The wavefronts on odd XCDs stream about a tenth slower when all eight compete for memory; per-XCD exit times put the
   // balance at 54.0 % of the stream on the even ones with 256-byte rows and at 54.7 % with 512-byte rows (head_dim 256:
   // even XCDs left at 329 us, odd ones at 338 with 54.0 %; 0.3571 -> 0.3532 ms with 54.7 %).
@@ -875,7 +903,17 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     return p.head_dim <= 128 ? launch_two_pass<128, 2, 2, true>(kv_elem, a, grid, stream)
                              : launch_two_pass<256, 1, 1, true>(kv_elem, a, grid, stream);
   }
-  const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side || (small_batch && tune().no_wave_only == 0);
+  // A few long chunks and little else -- by the static shapes: 256 tokens or more per max_num_seqs and about as many
+  // rows as 256 tiles of 128 at most -- do not fill the device with tiles that each walk their keys alone, and as
+  // wave-level items they read K and V once per 16 rows (one chunk of 512 tokens after 2048: 95 us).  They take the
+  // 128-row tiles, whose key ranges the device cuts into up to four runs when tiles are few (TileArgs::tile_split):
+  // 57 us, 107 against 287 us after 8192 tokens; a chunk with no context at all loses a tenth (32 against 29 us).
+  const bool few_long_chunks = p.query_start_loc != nullptr && !tiles_flagged(p) && p.num_queries_per_block <= 0 &&
+                               a.tile_split > 1 && tune().no_wave_only == 0 &&
+                               static_cast<int64_t>(p.total_tokens) >= 256ll * p.max_num_seqs &&
+                               static_cast<int64_t>(p.total_tokens) * p.num_q_heads <= 32768 + 2048;
+  const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side ||
+                         (small_batch && !few_long_chunks && tune().no_wave_only == 0);
   if (wave_only) {
     // head_dim 64: two kv heads per item where that keeps a decode token's rows in one 16-row tile
     a.pair = p.head_dim == 64 && p.num_kv_heads % 2 == 0 && 2 * (p.num_q_heads / p.num_kv_heads) <= 16 && pre.ml == nullptr &&
@@ -904,6 +942,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // so it goes by the average number of query tokens per sequence.
     const bool pipe_ok = p.head_dim == 128 && p.page_size >= 16 && p.logits_soft_cap == 0.f &&
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
+    if (few_long_chunks) return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
     const int pipe_choice = pipe_choice_of(p);
     const bool pipe_wanted = pipe_choice > 0 ||
                              (pipe_choice == 0 && tune().pipe != 0 &&

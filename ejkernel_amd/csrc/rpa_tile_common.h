@@ -56,6 +56,11 @@ struct TileArgs {
   // stream is cut by workgroup: a workgroup's share of a (sequence, kv head) is walked by its four wavefronts, a quarter
   // each, and merged in LDS, so a (sequence, kv head) has a quarter of the parts that go through memory (0 = never).
   int wg_unit_parts;
+  // A launch of few prefill tiles and nothing else: into how many runs of key tiles a tile's key range may be cut, a
+  // workgroup each, so that the tiles of one long chunk fill the device (0 or 1 = never; 128-row tiles only).  The
+  // parts' states lie in partial_o / partial_ml (tile_parts_cap of them fit) and a tile's ticket is the word
+  // counters[tile_ticket_base + tile].
+  int tile_split, tile_parts_cap, tile_ticket_base;
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the

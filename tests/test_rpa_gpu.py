@@ -226,6 +226,35 @@ def test_bf16_small_decode_batches_one_workgroup_per_kv_head(hq, hkv, D, window,
         assert (out[:rows].float() - split[:rows].float()).abs().max().item() <= 2e-2
 
 
+@pytest.mark.parametrize("hq,hkv,D", [(32, 8, 128), (8, 2, 128), (16, 2, 256), (16, 2, 64), (12, 4, 96)])
+@pytest.mark.parametrize("window,cap,sinks", [(None, None, False), (1500, 30.0, True)])
+def test_bf16_few_long_chunks_have_their_key_ranges_cut(hq, hkv, D, window, cap, sinks):
+    """One or two long chunks after a long context are few 128-row tiles for the grid's 512 workgroups: the library
+    takes the 128-row tile kernel for such shapes and the device cuts every tile's key range into up to four runs, a
+    workgroup each, whose states (reference point, sum, unnormalised output) meet in the workspace where the last one
+    to arrive adds them up in run order.  Parity with the oracle, the same bits on every call, agreement with the
+    wave-level loop (`num_queries_per_block=16`, which never cuts), zeros past the batch; chunks whose tiles differ
+    in length (the first one sees 1 key tile or 30), a chunk that ends inside a tile, an empty run (the cut leaves
+    the last runs of a short range without keys)."""
+    aux = (torch.randn(hq, 2, generator=torch.Generator().manual_seed(5)) * 2).numpy() if sinks else None
+    cases = [([300], [2300]), ([257, 40], [1900, 700]), ([512], [512]), ([64], [3000])]
+    for ql, kl in cases:
+        b = small(ql, kl, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, pages_per_seq=192, sliding_window=window,
+                  logits_soft_cap=cap, seed=29)
+        ref = run_strict(b, softmax_aux=aux)
+        rows = b.total_valid_tokens
+        nan_rows = np.isnan(ref[:rows]).any(axis=(1, 2))   # the reference program's window defect: float64 stands in
+        if nan_rows.any():
+            ref[:rows][nan_rows] = run_exact(b, softmax_aux=aux)[:rows][nan_rows]
+        for flags in (0, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES):
+            out = run_hip(b, flags, softmax_aux=aux)
+            assert_bf16_parity(to_np(out), ref, rows, f"{ql}/{kl} {hq}/{hkv} D={D} W={window} flags={flags}")
+            assert torch.equal(run_hip(b, flags, softmax_aux=aux), out)
+            assert not out[rows:].any()
+        by_wave = run_hip(b, softmax_aux=aux, cfg=RaggedPageAttentionConfig(num_queries_per_block=16))
+        assert (out[:rows].float() - by_wave[:rows].float()).abs().max().item() <= 2e-2 * max(1.0, by_wave[:rows].float().abs().max().item())
+
+
 @pytest.mark.parametrize("flags", PATHS)
 @pytest.mark.parametrize("hq,hkv,D", [(16, 2, 256), (8, 2, 256), (8, 2, 128), (32, 8, 128), (8, 2, 64), (4, 4, 64)])
 @pytest.mark.parametrize("window", [None, 48])

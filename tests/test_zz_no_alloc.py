@@ -40,7 +40,14 @@ def batches():
                        page_size=16, pages_per_seq=256, seed=33, device=DEV, sliding_window=1500)
     mixed_small = make_batch([70, 1], [300, 1200], num_q_heads=8, num_kv_heads=2, head_dim=64, page_size=16,
                              pages_per_seq=128, seed=34, device=DEV, logits_soft_cap=30.0)
-    return [(big, 0), (small, 0), (mixed, _native.RPA_FLAG_PREFILL_TILES), (mixed_small, _native.RPA_FLAG_PREFILL_TILES)]
+    # one long chunk alone: few prefill tiles, whose key ranges are cut and whose parts meet in the scratch; then a shorter one
+    chunk = make_batch([300], [2300], num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=160, seed=35,
+                       device=DEV)
+    chunk_small = make_batch([130], [900], num_q_heads=8, num_kv_heads=2, head_dim=128, page_size=16, pages_per_seq=64,
+                             seed=36, device=DEV)
+    tiles = _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES
+    return [(big, 0), (small, 0), (mixed, _native.RPA_FLAG_PREFILL_TILES), (mixed_small, _native.RPA_FLAG_PREFILL_TILES),
+            (chunk, tiles), (chunk_small, tiles)]
 
 
 def test_static_scratch_matches_the_workspace_entry_point_on_consecutive_calls():
