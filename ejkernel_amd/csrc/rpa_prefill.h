@@ -72,9 +72,13 @@ constexpr float kLazy = 6.f;  // logits may exceed the softmax reference point b
 // fetch is the 16-bit tile; kPass 1 walks K alone and leaves each row's softmax reference point and its sum of
 // exp(logit - point) in TileArgs::stats, kPass 2 forms P = round(exp(logit - point) / sum) in the cache dtype from
 // them and accumulates P V with no rescaling.
-template <int D, int MRT, bool kMimic, int kKv = 0, int kPass = 0>
+// kCut: the instantiation that can cut a tile's key range over several workgroups (split_info); it is compiled into
+// kernels of their own, for launches of few tiles, because the code that exchanges the runs' states, though it comes
+// after the key loop and is seldom run, changes the registers the compiler gives the loop (a third slower on
+// every batch in one build, not at all in the next).
+template <int D, int MRT, bool kMimic, int kKv = 0, int kPass = 0, bool kCut = false>
 __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
-                                             int qt, int part = 0, int parts = 1, int tile_id = 0) {
+                                             int qt, int split_info = 0) {
   using C = PCfg<D, MRT>;
   static_assert(kKv == 0 || C::NSTG == 2, "the register stage of an 8-bit cache stands in for one LDS stage ahead");
   static_assert((kKv == 0) == (kPass == 0), "an 8-bit cache runs as two passes, a 16-bit cache as one");
@@ -108,7 +112,11 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
   // A batch of few tiles (TileArgs::tile_split): the key range is cut into `parts` runs of whole key tiles, one
   // workgroup each, whose states meet in the workspace (below).  A run may be empty.
-  if (kPass == 0 && parts > 1) {
+  // split_info (one word, so that one scalar register is what stays alive across the key loop): bits 28..30 the number
+  // of runs (0: the range is not cut), 25..27 this workgroup's run, 24 whether the launch also holds a decode stream,
+  // 0..23 the tile's number in the launch.
+  if (kCut && kPass == 0 && split_info != 0) {
+    const int parts = (split_info >> 28) & 7, part = (split_info >> 25) & 7;
     const int n_kt = (max(range_hi - range_lo, 0) + C::TK - 1) / C::TK, per = (n_kt + parts - 1) / parts;
     range_lo = min(range_lo + part * per * C::TK, range_hi);
     range_hi = min(range_hi, range_lo + per * C::TK);
@@ -654,20 +662,34 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
   // part order (its own included, so the result does not depend on who comes last) and goes on to normalise and
   // store.  Written and read at agent scope like the partial states of the decode stream.
   float m_merged[MRT], l_merged[MRT];
-  if constexpr (kPass == 0) {
-    if (parts > 1) {
-      // (fresh names for the accumulators: what this seldom-run block does with them must not shape the registers
-      // they have in the key loop)
+  if constexpr (kCut && kPass == 0) {
+    if (split_info != 0) {
+      const int parts = (split_info >> 28) & 7, part = (split_info >> 25) & 7;
+      int tile_id = split_info & 0xffffff;
+      const bool upper = ((split_info >> 24) & 1) != 0;
+      // (fresh names for the rows' state: what this seldom-run block does with it should not shape the registers it
+      // has in the key loop -- it still does, from one build to the next, which is why the block has instantiations
+      // of its own)
 #pragma unroll
       for (int m = 0; m < MRT; ++m)
 #pragma unroll
         for (int sN = 0; sN < C::NS; ++sN)
 #pragma unroll
           for (int c = 0; c < C::CB; ++c) asm volatile("" : "+v"(o_acc[m][sN][c]));
+#pragma unroll
+      for (int m = 0; m < MRT; ++m) {
+        asm volatile("" : "+v"(l_acc[m]));
+        asm volatile("" : "+v"(m_thr[m]), "+v"(m_neg[m]));
+      }
       constexpr int kAgentScope = 16;
       constexpr uint32_t kWaveState = MRT * C::NS * C::CB * 1024, kPartState = kWgWaves * kWaveState;  // bytes
-      const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(a.partial_o, 0, 0x7fffffff, 0x00020000);
-      float2* ml = reinterpret_cast<float2*>(a.partial_ml);
+      // (a launch that also holds a decode stream keeps that stream's partial states in the lower half of both
+      // regions; the tiles' parts then take the upper half)
+      const TileArgs* ap = &a;
+      const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          reinterpret_cast<char*>(ap->partial_o) + (upper ? ap->tile_state_o_half : 0u), 0, 0x7fffffff, 0x00020000);
+      float2* ml = reinterpret_cast<float2*>(reinterpret_cast<char*>(ap->partial_ml) + (upper ? ap->tile_state_ml_half : 0u));
+      uint32_t* const ticket_words = ap->counters + ap->tile_ticket_base;
       const uint32_t my_part = static_cast<uint32_t>(tile_id * parts + part);
       auto state_off = [&](uint32_t pt, int m, int sN, int c) {
         return static_cast<int>(pt * kPartState + wave * kWaveState + ((m * C::NS + sN) * C::CB + c) * 1024 + lane * 16);
@@ -689,7 +711,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();  // every wavefront's state has left (and every wavefront is out of the key loop's LDS)
-      uint32_t* ctr = a.counters + a.tile_ticket_base + tile_id;
+      uint32_t* ctr = ticket_words + tile_id;
       int* flag = reinterpret_cast<int*>(lds);
       if (threadIdx.x == 0)
         *flag = static_cast<int>(__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
@@ -742,7 +764,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
     row_of(m, opaque0, valid, head, q_off);
     const float l_row1 = kPass == 1 ? row_groups_sum(l32[m]) : 0.f;  // the four lanes of a row, every lane taking part
     if (!valid) continue;
-    const float m_row = kPass == 0 && parts > 1 ? m_merged[m] : m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
+    const float m_row = kCut && kPass == 0 && split_info != 0 ? m_merged[m] : m_thr[m] == -INFINITY ? -INFINITY : -m_neg[m] * (1.f / kLog2e);
     if constexpr (kPass == 1) {
       if (g == 0) {
         float* st = a.stats + 2 * (q_off / hd);  // q_off = ((q0 + qi) * num_q_heads + head) * head_dim
@@ -751,7 +773,7 @@ __device__ __forceinline__ void prefill_tile(const TileArgs& a, char* __restrict
       }
       continue;
     }
-    const float l_run = kPass == 0 && parts > 1 ? l_merged[m] : l_acc[m][0];
+    const float l_run = kCut && kPass == 0 && split_info != 0 ? l_merged[m] : l_acc[m][0];
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;

@@ -66,14 +66,14 @@ constexpr bool kWideDecode = D == 256 && kWaveOnly && kKv == 0;
 template <int D, int MRT, bool kWaveOnly, int kKv>
 constexpr int kWavesPerSimd = kPipeTile<D, MRT> || kWideDecode<D, MRT, kWaveOnly, kKv> ? 1 : 2;
 
-template <int D, int MRT, bool kMimic, int kKv, int kPass>
+template <int D, int MRT, bool kMimic, int kKv, int kPass, bool kCut>
 __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, const SeqInfo& si, int s, int j, int qt,
-                                                 int part = 0, int parts = 1, int tile_id = 0) {
+                                                 int split_info = 0) {
   if constexpr (kPipeTile<D, MRT>) {
     static_assert(kKv == 0, "the pipelined tile reads a 16-bit cache");
     prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
   } else {
-    prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds, si, s, j, qt, part, parts, tile_id);
+    prefill_tile<D, MRT, kMimic, kKv, kPass, kCut>(a, lds, si, s, j, qt, split_info);
   }
 }
 
@@ -86,8 +86,9 @@ __device__ __forceinline__ int kept_in_place(int x) {
   return x;
 }
 
-// kFew (with kWaveOnly): the instantiation for batches of a few dozen (sequence, kv head)s at most, where the host can
-// tell from max_num_seqs; its decode stream is cut by workgroup or by wavefront.
+// kFew with kWaveOnly: the instantiation for batches of a few dozen (sequence, kv head)s at most, where the host can
+// tell from max_num_seqs; its decode stream is cut by workgroup or by wavefront.  kFew without: the instantiation for
+// launches of few prefill tiles (by the static shapes), whose key ranges can be cut over the idle workgroups.
 template <int D, int NT, int MRT, bool kMimic, bool kWaveOnly = false, int kKv = 0, int kPass = 0, bool kFew = false>
 __global__ __launch_bounds__(kWgThreads) __attribute__((amdgpu_waves_per_eu(kWavesPerSimd<D, MRT, kWaveOnly, kKv>, kWavesPerSimd<D, MRT, kWaveOnly, kKv>)))
 void rpa_tile_kernel(TileArgs a) {
@@ -143,7 +144,7 @@ void rpa_tile_kernel(TileArgs a) {
     my_items += it;
     my_wg += wg;
     if constexpr (!kWaveOnly && kKv == 0) {
-      if ((a.select != 0 || a.tile_split > 1) && wg > 0) {
+      if ((a.select != 0 || (kFew && a.tile_split > 1)) && wg > 0) {
         const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
         my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
       }
@@ -202,16 +203,25 @@ void rpa_tile_kernel(TileArgs a) {
     }
   }
 
-  // ---- a launch of few prefill tiles and nothing to stream -- one chunk of 512 tokens after 2048 is 128 tiles for 512
+  // ---- a launch of few prefill tiles -- one chunk of 512 tokens after 2048 is 128 tiles for 512
   // workgroups, each walking 40 key tiles alone: every tile's key range is cut into `key_split` runs, a workgroup each
   // (TileArgs::tile_split), as many as leaves every part a workgroup of its own and four key tiles by the batch's
   // average (total_cost counts 1024 (query row, key) pairs).
   int key_split = 1;
-  if constexpr (!kWaveOnly && kKv == 0 && kPass == 0 && !kPipeTile<D, MRT>) {
-    if (a.tile_split > 1 && total_wg > 0 && total_tiles == 0 && a.phase_mode == 4 && shift == 0 &&
-        a.tile_ticket_base + total_wg <= static_cast<int>(kQueueCounterIndex)) {
+  bool tiles_beside_stream = false;  // the parts' states then lie in the upper half of the workspace regions
+  if constexpr (kFew && !kWaveOnly && kKv == 0 && kPass == 0 && !kPipeTile<D, MRT>) {
+    if (a.tile_split > 1 && total_wg > 0 && a.phase_mode == 4 && shift == 0 &&
+        a.tile_ticket_base + total_wg <= static_cast<int>(kQueueCounterIndex) && total_wg < (1 << 24) && a.tile_split <= 7) {
+      // With a decode stream in the launch the workgroups from decode_grid on stream first and keep their partial
+      // states in the lower half of the workspace (two slots per wavefront): the tiles have decode_grid workgroups to
+      // begin with and the upper half for their parts.  That needs the stream on half of the grid at most.
+      const int grid = static_cast<int>(gridDim.x);
+      tiles_beside_stream = total_tiles > 0;
+      const bool room = !tiles_beside_stream || (grid > a.decode_grid && 2 * (grid - a.decode_grid) <= grid);
+      const int begin = tiles_beside_stream || total_items > 0 ? min(grid, a.decode_grid) : grid;
+      const int cap = tiles_beside_stream ? a.tile_parts_cap / 2 : a.tile_parts_cap;
       const long long key_tiles = (static_cast<long long>(total_cost) << 10) / (static_cast<long long>(total_wg) * PC::WGROWS * PC::TK);
-      key_split = min(min(a.tile_split, static_cast<int>(gridDim.x) / total_wg), min(static_cast<int>(key_tiles / 4), a.tile_parts_cap / total_wg));
+      if (room) key_split = min(min(a.tile_split, begin / total_wg), min(static_cast<int>(key_tiles / 4), cap / total_wg));
       key_split = __builtin_amdgcn_readfirstlane(max(key_split, 1));
     }
   }
@@ -502,7 +512,8 @@ void rpa_tile_kernel(TileArgs a) {
             j = rem / sz;
             member = full * kQueueRun + (rem - j * sz);
           }
-          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, n_qt - 1 - member, part, key_split, wt);
+          run_prefill_tile<D, MRT, kMimic, kKv, kPass, kFew && !kWaveOnly>(a, lds_data, si, s, j, n_qt - 1 - member,
+                                                       key_split > 1 ? (key_split << 28) | (part << 25) | (tiles_beside_stream ? 1 << 24 : 0) | wt : 0);
         }
         // The last workgroup out clears the counters for the next launch; the exit counts are kept per XCD and
         // then over the XCDs, so that the workgroups of a small batch, which all leave at once, do not queue up on one word.
@@ -536,7 +547,7 @@ void rpa_tile_kernel(TileArgs a) {
           const int j = local / n_qt, member = local - j * n_qt;
           const int round0 = (base + j * n_qt) / static_cast<int>(gridDim.x);
           const int qt = (member + 5 * round0) % n_qt;
-          run_prefill_tile<D, MRT, kMimic, kKv, kPass>(a, lds_data, si, s, j, qt);
+          run_prefill_tile<D, MRT, kMimic, kKv, kPass, kFew && !kWaveOnly>(a, lds_data, si, s, j, qt);
         }
       }
       // The wave-private K tiles used from here on overlay the prefill stages: wait until every wavefront of the
@@ -854,6 +865,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     a.tile_split = tune().tile_split;
     a.tile_parts_cap = static_cast<int>(std::min<uint64_t>(wl.partial_o_bytes >> 16, wl.partial_ml_bytes / (8 * rows)));
     a.tile_ticket_base = p.max_num_seqs * p.num_kv_heads;
+    a.tile_state_o_half = static_cast<uint32_t>((wl.partial_o_bytes / 2) & ~0xffffull);
+    a.tile_state_ml_half = static_cast<uint32_t>((wl.partial_ml_bytes / 2) & ~0xffull);
   }
   // The wavefronts on odd XCDs stream about a tenth slower when all eight compete for memory; per-XCD exit times put the
   // balance at 54.0 % of the stream on the even ones with 256-byte rows and at 54.7 % with 512-byte rows (head_dim 256:
@@ -908,10 +921,17 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   // wave-level items they read K and V once per 16 rows (one chunk of 512 tokens after 2048: 95 us).  They take the
   // 128-row tiles, whose key ranges the device cuts into up to four runs when tiles are few (TileArgs::tile_split):
   // 57 us, 107 against 287 us after 8192 tokens; a chunk with no context at all loses a tenth (32 against 29 us).
+  // The same holds for a chunk beside a few decode steps (512 tokens after 8192 with 64 decode steps: 392 us on the
+  // wave-level loop, 244 on the tiles): where the rows are few, the token count says that some sequence has hundreds of
+  // tokens (224 more tokens than sequences) and the block tables are laid out for long contexts (4096 keys or more --
+  // with short ones the wave-level loop is the faster by a tenth or two), the tiles are taken as well.
+  const int64_t rows_static = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
+  const bool long_chunks_by_shape = static_cast<int64_t>(p.total_tokens) >= 256ll * p.max_num_seqs ||
+                                    (static_cast<int64_t>(p.total_tokens) - p.max_num_seqs >= 224 &&
+                                     static_cast<int64_t>(p.pages_per_seq) * p.page_size >= 4096);
   const bool few_long_chunks = p.query_start_loc != nullptr && !tiles_flagged(p) && p.num_queries_per_block <= 0 &&
-                               a.tile_split > 1 && tune().no_wave_only == 0 &&
-                               static_cast<int64_t>(p.total_tokens) >= 256ll * p.max_num_seqs &&
-                               static_cast<int64_t>(p.total_tokens) * p.num_q_heads <= 32768 + 2048;
+                               a.tile_split > 1 && tune().no_wave_only == 0 && long_chunks_by_shape &&
+                               rows_static <= 32768 + 2048;
   const bool wave_only = pre.ml != nullptr || pre.sink_aux != nullptr || !side_by_side ||
                          (small_batch && !few_long_chunks && tune().no_wave_only == 0);
   if (wave_only) {
@@ -932,8 +952,14 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     a.stream_grid = device_cu_count();
     return mimic ? launch_cfg<256, 1, 1, true, true>(a, a.stream_grid, stream) : launch_cfg<256, 1, 1, false, true>(a, a.stream_grid, stream);
   }
-  if (p.head_dim == 64)
+  // Few rows by the static shapes (about 256 tiles of 128 at most): the instantiations whose tiles' key ranges the device
+  // can cut over the idle workgroups (kFew; 128-row tiles).
+  const bool cut_kernel = a.tile_split > 1 && static_cast<int64_t>(p.total_tokens) * p.num_q_heads <= 32768 + 2048;
+  if (p.head_dim == 64) {
+    if (cut_kernel)
+      return mimic ? launch_cfg<64, 2, 4, true, false, 0, 0, true>(a, grid, stream) : launch_cfg<64, 2, 4, false, false, 0, 0, true>(a, grid, stream);
     return mimic ? launch_cfg<64, 2, 4, true>(a, grid, stream) : launch_cfg<64, 2, 4, false>(a, grid, stream);
+  }
   if (p.head_dim <= 128) {
     // The software-pipelined tile (one workgroup per compute unit) fetches 16 keys per page look-up, has no soft cap
     // and folds a positive logit scale into the exp2 argument.  It pays for batches of long chunks; a batch that mixes
@@ -942,7 +968,8 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // so it goes by the average number of query tokens per sequence.
     const bool pipe_ok = p.head_dim == 128 && p.page_size >= 16 && p.logits_soft_cap == 0.f &&
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
-    if (few_long_chunks) return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
+    if (few_long_chunks)
+      return mimic ? launch_cfg<128, 2, 2, true, false, 0, 0, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, false, 0, 0, true>(a, grid, stream);
     const int pipe_choice = pipe_choice_of(p);
     const bool pipe_wanted = pipe_choice > 0 ||
                              (pipe_choice == 0 && tune().pipe != 0 &&
@@ -969,8 +996,12 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
       a.decode_grid = max(0, g1 - tune().pipe_stream_wgs);
       return mimic ? launch_cfg<128, 2, 4, true>(a, g1, stream) : launch_cfg<128, 2, 4, false>(a, g1, stream);
     }
+    if (cut_kernel)
+      return mimic ? launch_cfg<128, 2, 2, true, false, 0, 0, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, false, 0, 0, true>(a, grid, stream);
     return mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
   }
+  if (cut_kernel)
+    return mimic ? launch_cfg<256, 1, 1, true, false, 0, 0, true>(a, grid, stream) : launch_cfg<256, 1, 1, false, false, 0, 0, true>(a, grid, stream);
   return mimic ? launch_cfg<256, 1, 1, true>(a, grid, stream) : launch_cfg<256, 1, 1, false>(a, grid, stream);
 }
 

@@ -61,6 +61,7 @@ struct TileArgs {
   // parts' states lie in partial_o / partial_ml (tile_parts_cap of them fit) and a tile's ticket is the word
   // counters[tile_ticket_base + tile].
   int tile_split, tile_parts_cap, tile_ticket_base;
+  uint32_t tile_state_o_half, tile_state_ml_half;  // bytes: half of partial_o and of partial_ml (a launch with a decode stream)
 };
 
 // How the softmax scale enters.  Reference arithmetic of ragged_page_attention (kMimic): q is multiplied by the

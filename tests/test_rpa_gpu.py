@@ -237,7 +237,9 @@ def test_bf16_few_long_chunks_have_their_key_ranges_cut(hq, hkv, D, window, cap,
     in length (the first one sees 1 key tile or 30), a chunk that ends inside a tile, an empty run (the cut leaves
     the last runs of a short range without keys)."""
     aux = (torch.randn(hq, 2, generator=torch.Generator().manual_seed(5)) * 2).numpy() if sinks else None
-    cases = [([300], [2300]), ([257, 40], [1900, 700]), ([512], [512]), ([64], [3000])]
+    # (the last one: a chunk beside decode steps -- the tiles' parts then share the workspace with the decode stream's
+    # partial states, which the long decode sequence makes sure there are)
+    cases = [([300], [2300]), ([257, 40], [1900, 700]), ([512], [512]), ([64], [3000]), ([280, 1, 1, 1], [2000, 3000, 17, 900])]
     for ql, kl in cases:
         b = small(ql, kl, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, pages_per_seq=192, sliding_window=window,
                   logits_soft_cap=cap, seed=29)
