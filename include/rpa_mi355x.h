@@ -109,6 +109,8 @@ typedef struct RpaParams {
                                   /* software-pipelined tiles where they exist (head_dim 128, no soft cap, pages of   */
                                   /* 16 tokens or more; by default at least 128 tokens per max_num_seqs), 128-row     */
                                   /* tiles otherwise.  RPA_FLAG_PREFILL_TILES / PIPE_TILES / PLAIN_TILES come first.  */
+                                  /* With few rows (total_tokens x num_q_heads up to 34816) the 128-row tiles' key     */
+                                  /* ranges are cut over idle workgroups when tiles are few: one long chunk alone.     */
   int32_t num_kv_pages_per_block; /* the least stretch of a sequence, in pages, that one streaming wavefront takes     */
                                   /* before a small batch is spread over more wavefronts (split-K granularity;        */
                                   /* default: 2 tiles of 32 keys, more for long sequences -- and one workgroup per     */
