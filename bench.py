@@ -40,6 +40,8 @@ def measured_traffic_bytes(workload: str):
 # second workload of a process, 0.392-0.398 ms as the fifth; 0.380 ms alone).
 EXTRA_CONFIGS = ["gemma2_local", "decode_long_context", "decode_small", "mixed_prefill_decode", "mixed_prefill_only",
                  "prefill_single_16k",
+                 # one request's chunked prefill, alone and beside 64 decode steps: latency, like decode_small
+                 "prefill_chunk_after_8k", "chunk_beside_decodes",
                  # What a serving caller with padded static shapes gets (max_num_seqs 512, query rows rounded up to
                  # 8192 / 16384, num_seqs as is): the library's own choice of kernel instantiation, made from those
                  # shapes, and the choice the caller names through RaggedPageAttentionConfig.num_queries_per_block.
@@ -669,8 +671,8 @@ def measure_config(name, steps, warmup, want_parity, queries_per_block=None):
         entry["static_shapes"] = {"total_tokens": int(batch.queries.shape[0]), "max_num_seqs": int(m["max_num_seqs"]),
                                   "num_seqs": len(batch.q_lens)}
         entry["num_queries_per_block"] = queries_per_block
-    if name == "decode_small":
-        # the launch-bound configuration: the same call replayed from a HIP graph, where no host code runs per step
+    if name in ("decode_small", "prefill_chunk_after_8k", "chunk_beside_decodes"):
+        # the launch-bound configurations: the same call replayed from a HIP graph, where no host code runs per step
         entry["graph_replay_ms"] = graph_replay_ms(step, max(steps, 50))
     if want_parity:
         if name in LONG_PROMPT_CONFIGS:

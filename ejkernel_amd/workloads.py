@@ -358,6 +358,9 @@ WORKLOADS = {
     # decode_llama3_8b and a mixed batch, 16 chunks x 256 tokens beside 112 decode sequences
     "decode_head_dim_96": "256 seqs x 1 token, kv 512..8192, 32q/8kv heads, D=96, page 16",
     "mixed_head_dim_96": "16 chunks x 256 tokens (prior 0..2048) + 112 decode seqs (kv 256..4096), 32q/8kv heads, D=96, page 32",
+    # one request's chunked prefill, alone and beside a few decode steps: few tiles, each with a long key range
+    "prefill_chunk_after_8k": "1 chunk x 512 tokens after 8192, 32q/8kv heads, D=128, page 16",
+    "chunk_beside_decodes": "1 chunk x 512 tokens after 8192 + 64 decode seqs (kv 256..4096), 32q/8kv heads, D=128, page 16",
     # one long prompt: 512 prefill tiles of 256 rows that walk up to 16384 keys each (per-tile costs vanish)
     "prefill_single_16k": "1 prompt x 16384 tokens from scratch, 32q/8kv heads, D=128, page 32",
     # the static shapes of a serving caller: the same sequences, pages and queries as the unpadded workloads inside
@@ -432,6 +435,13 @@ def make_workload(name: str, *, device="cpu", scale: float = 1.0, dtype=torch.bf
         return make_batch(q[order], kv[order], num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
                           pages_per_seq=pps, seed=seed, device=device, dtype=dtype,
                           name=(only or name) + ("_padded" if padded else ""), **pad)
+    if name in ("prefill_chunk_after_8k", "chunk_beside_decodes"):
+        chunk, prior = n(512), n(8192)
+        n_dec = n(64) if name == "chunk_beside_decodes" else 0
+        q = np.concatenate([[chunk], np.ones(n_dec, np.int64)])
+        kv = np.concatenate([[prior + chunk], rng.integers(n(256), n(4096) + 1, size=n_dec)])
+        return make_batch(q, kv, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=16,
+                          pages_per_seq=pages(prior + chunk, 16), seed=seed, device=device, dtype=dtype, name=name)
     if name == "prefill_long":
         L = n(8192)
         return make_batch(np.full(2, L), np.full(2, L), num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,

@@ -41,6 +41,9 @@ def check_sample(b, out, n_seqs, seed=0):
         short = [s for s in order if b.kv_lens[s] < b.sliding_window + 64 * b.meta["page_size"]]
         head = short[: n_seqs // 2]
         order = head + [s for s in order if s not in head]
+    longest = int(np.argmax(b.q_lens))   # a workload's one long chunk, if it has one, is always in the sample
+    if b.q_lens[longest] > 1:
+        order = [longest] + [s for s in order if s != longest]
     ids = sorted(order[:n_seqs])
     sub = compact_for_host(b, ids)
     ref = rpa_oracle_c.rpa_strict_c(*oracle_args(sub), softmax_scale=sub.softmax_scale,
@@ -72,7 +75,8 @@ def permuted(b, seed=9):
                                                    ("mixed_prefill_decode", 14, True), ("mixed_prefill_only", 3, True),
                                                    ("gemma2_local", 8, False), ("decode_long_context", 5, False),
                                                    ("decode_head_dim_96", 12, True), ("mixed_head_dim_96", 10, True),
-                                                   ("prefill_head_dim_256", 1, True), ("decode_head_dim_64", 12, True)])
+                                                   ("prefill_head_dim_256", 1, True), ("decode_head_dim_64", 12, True),
+                                                   ("prefill_chunk_after_8k", 1, True), ("chunk_beside_decodes", 6, True)])
 def test_full_size_workload(name, n_sample, permute):
     b = make_workload(name, device=DEV)
     out = run(b)
