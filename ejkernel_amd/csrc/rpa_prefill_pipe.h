@@ -132,7 +132,7 @@ __device__ __forceinline__ void pipe_key_loop(PipeIo& R) {
 
 template <bool kMimic>
 __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __restrict__ lds, const SeqInfo& si, int s, int j,
-                                                  int qt) {
+                                                  int qt, int split_info = 0) {
   using C = PipeCfg;
   constexpr int NRG = C::NRG;
   const RpaParams& p = a.p;
@@ -154,8 +154,17 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
   // ---- key range of the workgroup's rows
   const int wg_row_lo = qt * C::WGROWS, wg_row_hi = min(wg_row_lo + C::WGROWS, si.rows);
   const int wg_pos_min = pos0 + wg_row_lo / G, wg_pos_max = pos0 + (wg_row_hi - 1) / G;
-  const int range_hi = min(si.kv_len, wg_pos_max + 1);
-  const int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
+  int range_hi = min(si.kv_len, wg_pos_max + 1);
+  int range_lo = max(W > 0 ? max(0, wg_pos_min - W + 1) : 0, si.start) & ~(C::TK - 1);
+  // A launch of few tiles: the key range is cut into runs of whole key tiles, a workgroup each, whose states meet in the
+  // workspace (split_info and the exchange as in rpa_prefill.h; here the key loop is a fixed instruction stream, which
+  // what comes after it cannot disturb).  A run may be empty.
+  if (split_info != 0) {
+    const int parts = (split_info >> 28) & 7, part = (split_info >> 25) & 7;
+    const int n_kt = (max(range_hi - range_lo, 0) + C::TK - 1) / C::TK, per = (n_kt + parts - 1) / parts;
+    range_lo = min(range_lo + part * per * C::TK, range_hi);
+    range_hi = min(range_hi, range_lo + per * C::TK);
+  }
   const int t_last = range_hi - 1;
 
   // ---- this wavefront's rows: row group rg holds rows w_row_lo + 32 rg + i
@@ -365,6 +374,83 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     }
   }
 
+  // ---- a run of a cut key range: state to the workspace, a ticket of the tile, and the workgroup that draws the last
+  // one adds the runs up in run order (its own included) and goes on.  Per lane 32 pieces of 16 bytes (row group,
+  // block, four accumulators), 1 KiB per piece and wavefront in lane order; per row its reference point and sum.
+  float m_merged[NRG], l_merged[NRG];
+  if (split_info != 0) {
+    const int parts = (split_info >> 28) & 7, part = (split_info >> 25) & 7, tile_id = split_info & 0xffffff;
+    const bool upper = ((split_info >> 24) & 1) != 0;
+    constexpr int kAgentScope = 16;
+    constexpr uint32_t kWaveState = NRG * C::NBLK * 4 * 1024, kPartState = kWgWaves * kWaveState;  // bytes
+    const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        reinterpret_cast<char*>(a.partial_o) + (upper ? a.tile_state_o_half : 0u), 0, 0x7fffffff, 0x00020000);
+    uint64_t* ml = reinterpret_cast<uint64_t*>(reinterpret_cast<char*>(a.partial_ml) + (upper ? a.tile_state_ml_half : 0u));
+    const uint32_t my_part = static_cast<uint32_t>(tile_id * parts + part);
+    auto state_off = [&](uint32_t pt, int rg, int blk, int q4) {
+      return static_cast<int>(pt * kPartState + wave * kWaveState + ((rg * C::NBLK + blk) * 4 + q4) * 1024 + lane * 16);
+    };
+    auto ml_index = [&](uint32_t pt, int rg) { return (pt * kWgWaves + wave) * (32 * NRG) + 32 * rg + i; };
+#pragma unroll
+    for (int rg = 0; rg < NRG; ++rg) {
+#pragma unroll
+      for (int blk = 0; blk < C::NBLK; ++blk)
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) {
+          const f32x4_t v = {o_acc[rg][blk][4 * q4], o_acc[rg][blk][4 * q4 + 1], o_acc[rg][blk][4 * q4 + 2], o_acc[rg][blk][4 * q4 + 3]};
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v), o_rsrc, state_off(my_part, rg, blk, q4), 0, kAgentScope);
+        }
+      const float l_row = l_part[rg] + __shfl_xor(l_part[rg], 32, kWave);  // the two lanes of a row hold half its keys each
+      if (g == 0) {
+        const float m_row = m_thr[rg] == -INFINITY ? -INFINITY : -m_neg[rg] * (1.f / kLog2e);
+        const uint64_t v = static_cast<uint64_t>(__float_as_uint(m_row)) | (static_cast<uint64_t>(__float_as_uint(l_row)) << 32);
+        __hip_atomic_store(ml + ml_index(my_part, rg), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // every wavefront's state has left (and every wavefront is out of the key loop's LDS)
+    uint32_t* ctr = a.counters + a.tile_ticket_base + tile_id;
+    int* flag = reinterpret_cast<int*>(lds);
+    if (threadIdx.x == 0)
+      *flag = static_cast<int>(__hip_atomic_fetch_add(ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    __syncthreads();
+    const int ticket = *flag;
+    __syncthreads();  // (the flag's word belongs to the next tile's stage from here on)
+    if (ticket != parts - 1) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+#pragma unroll
+    for (int rg = 0; rg < NRG; ++rg) {
+      float M = -INFINITY, L = 0.f;
+#pragma unroll
+      for (int blk = 0; blk < C::NBLK; ++blk)
+#pragma unroll
+        for (int k = 0; k < 16; ++k) o_acc[rg][blk][k] = 0.f;
+      for (int pt = 0; pt < parts; ++pt) {
+        const uint32_t src = static_cast<uint32_t>(tile_id * parts + pt);
+        const uint64_t v = __hip_atomic_load(ml + ml_index(src, rg), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const float mk = __uint_as_float(static_cast<uint32_t>(v)), lk = __uint_as_float(static_cast<uint32_t>(v >> 32));
+        const float m_new = fmaxf(M, mk);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        const float keep = __builtin_amdgcn_exp2f((M - m_use) * kLog2e);
+        const float w = __builtin_amdgcn_exp2f((mk - m_use) * kLog2e);
+        L = L * keep + w * lk;
+        M = m_new;
+#pragma unroll
+        for (int blk = 0; blk < C::NBLK; ++blk)
+#pragma unroll
+          for (int q4 = 0; q4 < 4; ++q4) {
+            const f32x4_t ov = __builtin_bit_cast(f32x4_t, __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, state_off(src, rg, blk, q4), 0, kAgentScope));
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o_acc[rg][blk][4 * q4 + e] = o_acc[rg][blk][4 * q4 + e] * keep + w * ov[e];
+          }
+      }
+      m_merged[rg] = M;
+      l_merged[rg] = L;
+    }
+    if (threadIdx.x == 0) __hip_atomic_store(ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+
   // ---- normalise (with optional sinks) and store
 #pragma unroll
   for (int rg = 0; rg < NRG; ++rg) {
@@ -374,9 +460,13 @@ __device__ __forceinline__ void prefill_tile_pipe(const TileArgs& a, char* __res
     int opaque0 = 0;
     asm volatile("" : "+v"(opaque0));
     row_of(rg, opaque0, valid, head, q_off);
-    const float l_run = l_part[rg] + __shfl_xor(l_part[rg], 32, kWave);  // the two lanes of a row hold half its keys each
+    float l_run = l_part[rg] + __shfl_xor(l_part[rg], 32, kWave);  // the two lanes of a row hold half its keys each
     if (!valid) continue;
-    const float m_row = m_thr[rg] == -INFINITY ? -INFINITY : -m_neg[rg] * (1.f / kLog2e);
+    float m_row = m_thr[rg] == -INFINITY ? -INFINITY : -m_neg[rg] * (1.f / kLog2e);
+    if (split_info != 0) {
+      l_run = l_merged[rg];
+      m_row = m_merged[rg];
+    }
     float num_scale = 1.f, denom = l_run;
     if (p.sinks != nullptr && p.num_sinks > 0) {
       const float* __restrict__ sk = p.sinks + static_cast<size_t>(head) * p.num_sinks;

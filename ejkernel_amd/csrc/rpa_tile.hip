@@ -71,7 +71,7 @@ __device__ __forceinline__ void run_prefill_tile(const TileArgs& a, char* lds, c
                                                  int split_info = 0) {
   if constexpr (kPipeTile<D, MRT>) {
     static_assert(kKv == 0, "the pipelined tile reads a 16-bit cache");
-    prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt);
+    prefill_tile_pipe<kMimic>(a, lds, si, s, j, qt, split_info);
   } else {
     prefill_tile<D, MRT, kMimic, kKv, kPass, kCut>(a, lds, si, s, j, qt, split_info);
   }
@@ -144,7 +144,7 @@ void rpa_tile_kernel(TileArgs a) {
     my_items += it;
     my_wg += wg;
     if constexpr (!kWaveOnly && kKv == 0) {
-      if ((a.select != 0 || (kFew && a.tile_split > 1)) && wg > 0) {
+      if ((a.select != 0 || ((kFew || kPipeTile<D, MRT>) && a.tile_split > 1)) && wg > 0) {
         const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
         my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
       }
@@ -209,7 +209,7 @@ void rpa_tile_kernel(TileArgs a) {
   // average (total_cost counts 1024 (query row, key) pairs).
   int key_split = 1;
   bool tiles_beside_stream = false;  // the parts' states then lie in the upper half of the workspace regions
-  if constexpr (kFew && !kWaveOnly && kKv == 0 && kPass == 0 && !kPipeTile<D, MRT>) {
+  if constexpr ((kFew || kPipeTile<D, MRT>) && !kWaveOnly && kKv == 0 && kPass == 0) {
     if (a.tile_split > 1 && total_wg > 0 && a.phase_mode == 4 && shift == 0 &&
         a.tile_ticket_base + total_wg <= static_cast<int>(kQueueCounterIndex) && total_wg < (1 << 24) && a.tile_split <= 7) {
       // With a decode stream in the launch the workgroups from decode_grid on stream first and keep their partial
@@ -970,6 +970,10 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
                          (mimic || p.softmax_scale * (p.k_scale > 0.f ? p.k_scale : 1.f) * (p.q_scale > 0.f ? p.q_scale : 1.f) > 0.f);
     if (few_long_chunks)
       return mimic ? launch_cfg<128, 2, 2, true, false, 0, 0, true>(a, grid, stream) : launch_cfg<128, 2, 2, false, false, 0, 0, true>(a, grid, stream);
+    // (parts of cut 256-row tiles: 128 KiB of accumulators and 2 KiB of row statistics each)
+    WorkspaceLayout wl_pipe;
+    tiled_workspace_layout(p, &wl_pipe);
+    const int pipe_parts_cap = static_cast<int>(std::min<uint64_t>(wl_pipe.partial_o_bytes >> 17, wl_pipe.partial_ml_bytes >> 11));
     const int pipe_choice = pipe_choice_of(p);
     const bool pipe_wanted = pipe_choice > 0 ||
                              (pipe_choice == 0 && tune().pipe != 0 &&
@@ -984,6 +988,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
       if (rc != RPA_OK) return rc;
       const int g1 = device_cu_count();
       b.select = 2;
+      b.tile_parts_cap = pipe_parts_cap;
       b.stream_grid = g1;
       b.decode_grid = max(0, g1 - tune().pipe_stream_wgs);
       return mimic ? launch_cfg<128, 2, 4, true>(b, g1, stream) : launch_cfg<128, 2, 4, false>(b, g1, stream);
@@ -992,6 +997,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
       // one workgroup per compute unit; in a mixed batch the last pipe_stream_wgs of them (a multiple of 8: the same
       // number on every XCD) take the decode stream first and join the prefill queues when it is done
       const int g1 = device_cu_count();
+      a.tile_parts_cap = pipe_parts_cap;
       a.stream_grid = g1;
       a.decode_grid = max(0, g1 - tune().pipe_stream_wgs);
       return mimic ? launch_cfg<128, 2, 4, true>(a, g1, stream) : launch_cfg<128, 2, 4, false>(a, g1, stream);
