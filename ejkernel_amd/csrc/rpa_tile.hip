@@ -217,8 +217,12 @@ void rpa_tile_kernel(TileArgs a) {
       // begin with and the upper half for their parts.  That needs the stream on half of the grid at most.
       const int grid = static_cast<int>(gridDim.x);
       tiles_beside_stream = total_tiles > 0;
-      const bool room = !tiles_beside_stream || (grid > a.decode_grid && 2 * (grid - a.decode_grid) <= grid);
-      const int begin = tiles_beside_stream || total_items > 0 ? min(grid, a.decode_grid) : grid;
+      const bool room = !tiles_beside_stream ||
+                        (grid > a.decode_grid && 2 * kWgWaves * (grid - a.decode_grid) <= a.tile_stream_slots_half);
+      // (a stream shorter than the tiles' time, by the weights of the two kernels' pick above: the streaming workgroups
+      // come to the queues while parts are left, and every workgroup counts)
+      const bool short_stream = 10ll * total_cost >= 35ll * total_tiles;
+      const int begin = (tiles_beside_stream && !short_stream) || total_items > 0 ? min(grid, a.decode_grid) : grid;
       const int cap = tiles_beside_stream ? a.tile_parts_cap / 2 : a.tile_parts_cap;
       const long long key_tiles = (static_cast<long long>(total_cost) << 10) / (static_cast<long long>(total_wg) * PC::WGROWS * PC::TK);
       if (room) key_split = min(min(a.tile_split, begin / total_wg), min(static_cast<int>(key_tiles / 4), cap / total_wg));
@@ -867,6 +871,7 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     a.tile_ticket_base = p.max_num_seqs * p.num_kv_heads;
     a.tile_state_o_half = static_cast<uint32_t>((wl.partial_o_bytes / 2) & ~0xffffull);
     a.tile_state_ml_half = static_cast<uint32_t>((wl.partial_ml_bytes / 2) & ~0xffull);
+    a.tile_stream_slots_half = kWgWaves * tiled_grid();  // half of the slots of the decode stream's partial states
   }
   // The wavefronts on odd XCDs stream about a tenth slower when all eight compete for memory; per-XCD exit times put the
   // balance at 54.0 % of the stream on the even ones with 256-byte rows and at 54.7 % with 512-byte rows (head_dim 256:

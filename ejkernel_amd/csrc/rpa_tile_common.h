@@ -61,6 +61,7 @@ struct TileArgs {
   // parts' states lie in partial_o / partial_ml (tile_parts_cap of them fit) and a tile's ticket is the word
   // counters[tile_ticket_base + tile].
   int tile_split, tile_parts_cap, tile_ticket_base;
+  int tile_stream_slots_half;  // slots of the decode stream's partial states that fit in the lower half
   uint32_t tile_state_o_half, tile_state_ml_half;  // bytes: half of partial_o and of partial_ml (a launch with a decode stream)
 };
 
