@@ -123,6 +123,49 @@ def random_rpa_batch(seed, device, head_dims=(64, 128, 256)):
     return b, f"seed {seed}: {hq}/{hkv} D={D} page={page} q={q_lens} kv={kv_lens} W={window} cap={cap}"
 
 
+def random_serving_batch(seed, device):
+    """A seeded draw over the shapes of a serving step: one to three long chunks after contexts of up to 8000 tokens
+    with up to 70 decode steps beside them, small batches of decode steps, or a few decode sequences of up to 70000 keys;
+    sometimes inside padded static shapes, sometimes with the tile shape named.  Returns the batch, the sinks (or
+    None), the config hint (or 0) and a description."""
+    rng = np.random.default_rng(seed)
+    regime = ["chunks", "chunks", "small_decode", "long_decode"][rng.integers(4)]
+    hq, hkv = [(32, 8), (16, 4), (8, 2), (16, 2), (8, 8)][rng.integers(5)]
+    D = int(rng.choice([128, 128, 128, 64, 256]))
+    page = int(rng.choice([16, 32, 64]))
+    window = None if rng.random() < 0.7 else int(rng.integers(16, 3000))
+    cap = None if rng.random() < 0.8 else 30.0
+    aux = None if rng.random() < 0.8 else rng.standard_normal((hq, 1)).astype(np.float32)
+    if regime == "chunks":
+        n_ch = int(rng.integers(1, 4))
+        q = [int(rng.integers(60, 1100 // n_ch + 60)) for _ in range(n_ch)]
+        kv = [qq + int(rng.choice([0, rng.integers(0, 600), rng.integers(0, 8000)])) for qq in q]
+        n_dec = int(rng.choice([0, 0, rng.integers(1, 8), rng.integers(8, 72)]))
+        q += [1] * n_dec
+        kv += [int(rng.integers(1, 4000)) for _ in range(n_dec)]
+    elif regime == "small_decode":
+        n = int(rng.integers(1, 72))
+        q = [int(rng.choice([1, 1, 1, rng.integers(1, 5)])) for _ in range(n)]
+        kv = [max(qq, int(rng.integers(1, rng.choice([64, 600, 3000])))) for qq in q]
+    else:
+        q = [1] * int(rng.integers(1, 5))
+        kv = [int(rng.integers(1, rng.choice([9000, 70000]))) for _ in q]
+    order = rng.permutation(len(q))
+    q, kv = [q[i] for i in order], [kv[i] for i in order]
+    pps = -(-max(kv) // page)
+    pps = pps if pps < 64 else -(-pps // 64) * 64
+    kw = {}
+    if rng.random() < 0.4:   # a caller's padded static shapes
+        kw = dict(max_num_seqs=int(rng.choice([len(q) + 3, 256, 512])), pool_seqs=len(q),
+                  total_tokens=int(max(((sum(q) + 7) // 8) * 8 + 8, rng.choice([2048, 8192]))))
+    hint = int(rng.choice([0, 0, 128, 256])) if regime == "chunks" else 0
+    b = make_batch(q, kv, num_q_heads=hq, num_kv_heads=hkv, head_dim=D, page_size=page, pages_per_seq=pps, seed=seed,
+                   device=device, sliding_window=window, logits_soft_cap=cap, **kw)
+    what = (f"seed {seed} {regime}: {hq}/{hkv} D={D} page={page} q={q} kv={kv} W={window} cap={cap} "
+            f"sinks={aux is not None} pad={kw} hint={hint}")
+    return b, aux, hint, what
+
+
 def two_key_cap_batch(device="cpu", head_dim=16, dtype=torch.bfloat16):
     """One query row over two keys with the soft cap 23.7, which bf16 does not hold (the weakly typed scalar becomes
     23.75 before it divides and multiplies, _xla_impl_fwd.py:125-126).  q . k is 20 for key 0 and 16 for key 1

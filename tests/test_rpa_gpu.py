@@ -12,7 +12,7 @@ import torch
 from ejkernel_amd import _native
 from ejkernel_amd.modules import RaggedPageAttention, RaggedPageAttentionConfig, ragged_page_attention
 from ejkernel_amd.workloads import Batch, compact_for_host, make_batch, make_workload
-from tests.helpers import (F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, random_rpa_batch,
+from tests.helpers import (F32_MAX_ABS, assert_bf16_parity, assert_bf16_parity_stepwise, err_stats, random_rpa_batch, random_serving_batch,
                            run_exact, run_strict, to_np, two_key_cap_batch)
 
 pytestmark = pytest.mark.gpu
@@ -429,6 +429,29 @@ def test_bf16_random_batches(seed):
         mx, mean = err_stats(out, exact, rows)
         assert mx <= 4e-2 and mean <= 2e-3, f"{what} flags={flags}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
         assert not out[rows:].any()
+
+
+@pytest.mark.parametrize("seed", range(60000, 60048))
+def test_bf16_random_serving_batches(seed):
+    """Seeded random serving steps -- long chunks whose few tiles have their key ranges cut, with and without decode
+    steps beside them; small decode batches (one workgroup per (sequence, kv head)); a few very long decode sequences
+    (the stream cut by workgroup) -- on the library's own choice of kernel: against the float64 evaluation where that
+    takes a second or two (4e-2 / 2e-3, as for the other random batches: bf16 logits alone put 2.5e-2 between the
+    reference's arithmetic and float64), against the wave-level loop with a caller-named split (which cuts no tile
+    and merges no parts in LDS) to the parity bound, the same bits on a second call, zeros past the batch."""
+    b, aux, hint, what = random_serving_batch(seed, DEV)
+    rows = b.total_valid_tokens
+    cfg = RaggedPageAttentionConfig(num_queries_per_block=hint) if hint else None
+    out = run_hip(b, softmax_aux=aux, cfg=cfg)
+    assert torch.equal(run_hip(b, softmax_aux=aux, cfg=cfg), out), what
+    assert not out[rows:].any(), what
+    page, pps = b.kv_pages.shape[1], b.block_tables.shape[1]
+    by_wave = run_hip(b, softmax_aux=aux, cfg=RaggedPageAttentionConfig(num_queries_per_block=16,
+                                                                         num_kv_pages_per_block=min(pps, max(1, 256 // page))))
+    assert_bf16_parity_stepwise(to_np(out)[:rows], to_np(by_wave)[:rows], what + " (against the wave-level loop)")
+    if sum(int(q) * int(k) for q, k in zip(b.q_lens, b.kv_lens)) * b.queries.shape[1] * b.queries.shape[2] <= 6e9:
+        mx, mean = err_stats(to_np(out), run_exact(b, softmax_aux=aux), rows)
+        assert mx <= 4e-2 and mean <= 2e-3, f"{what}: vs float64 max-abs {mx:.4g} mean-abs {mean:.4g}"
 
 
 @pytest.mark.parametrize("seed", [8028, 8038, 9067])
