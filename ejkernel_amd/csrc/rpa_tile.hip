@@ -207,6 +207,17 @@ void rpa_tile_kernel(TileArgs a) {
   // workgroups, each walking 40 key tiles alone: every tile's key range is cut into `key_split` runs, a workgroup each
   // (TileArgs::tile_split), as many as leaves every part a workgroup of its own and four key tiles by the batch's
   // average (total_cost counts 1024 (query row, key) pairs).
+  // Workgroups from `dgrid` on begin with the wave-level work (TileArgs::decode_grid).  A launch whose decode stream
+  // is a few tiles -- a decode step or two and a handful of short sequences beside the chunks -- keeps no more
+  // workgroups from the prefill tiles than that work has wavefronts for: the stream's wavefronts of min_share_tiles
+  // tiles each (they are numbered over the even XCDs first, hence twice as many workgroups) and the wave-level items'.
+  // A multiple of 8, the same on every XCD.
+  int dgrid = a.decode_grid;
+  if constexpr (!kWaveOnly) {
+    const int stream_waves = total_tiles > 0 ? total_tiles / max(a.min_share_tiles, 1) + 1 : 0;
+    const int wave_wgs = (2 * ((stream_waves + kWgWaves - 1) / kWgWaves) + (total_items + kWgWaves - 1) / kWgWaves + 7) & ~7;
+    dgrid = __builtin_amdgcn_readfirstlane(max(dgrid, static_cast<int>(gridDim.x) - wave_wgs));
+  }
   int key_split = 1;
   bool tiles_beside_stream = false;  // the parts' states then lie in the upper half of the workspace regions
   if constexpr ((kFew || kPipeTile<D, MRT>) && !kWaveOnly && kKv == 0 && kPass == 0) {
@@ -218,11 +229,11 @@ void rpa_tile_kernel(TileArgs a) {
       const int grid = static_cast<int>(gridDim.x);
       tiles_beside_stream = total_tiles > 0;
       const bool room = !tiles_beside_stream ||
-                        (grid > a.decode_grid && 2 * kWgWaves * (grid - a.decode_grid) <= a.tile_stream_slots_half);
+                        (grid > dgrid && 2 * kWgWaves * (grid - dgrid) <= a.tile_stream_slots_half);
       // (a stream shorter than the tiles' time, by the weights of the two kernels' pick above: the streaming workgroups
       // come to the queues while parts are left, and every workgroup counts)
       const bool short_stream = 10ll * total_cost >= 35ll * total_tiles;
-      const int begin = (tiles_beside_stream && !short_stream) || total_items > 0 ? min(grid, a.decode_grid) : grid;
+      const int begin = (tiles_beside_stream && !short_stream) || total_items > 0 ? min(grid, dgrid) : grid;
       const int cap = tiles_beside_stream ? a.tile_parts_cap / 2 : a.tile_parts_cap;
       const long long key_tiles = (static_cast<long long>(total_cost) << 10) / (static_cast<long long>(total_wg) * PC::WGROWS * PC::TK);
       if (room) key_split = min(min(a.tile_split, begin / total_wg), min(static_cast<int>(key_tiles / 4), cap / total_wg));
@@ -238,8 +249,8 @@ void rpa_tile_kernel(TileArgs a) {
   if constexpr (!kWaveOnly) {
     // (With no more tiles than workgroups that begin with tiles every tile starts at once and the order is of no
     // consequence: the sort, two microseconds of a launch that takes thirty, is left out.)
-    const int begin_with_tiles = static_cast<int>(gridDim.x) > a.decode_grid && (total_tiles > 0 || total_items > 0)
-                                     ? a.decode_grid : static_cast<int>(gridDim.x);
+    const int begin_with_tiles = static_cast<int>(gridDim.x) > dgrid && (total_tiles > 0 || total_items > 0)
+                                     ? dgrid : static_cast<int>(gridDim.x);
     if (total_wg > begin_with_tiles && shift == 0 && a.phase_mode == 4) {
       int mine = 0;
       for (int s = s_begin; s < s_end; ++s) {
@@ -391,9 +402,9 @@ void rpa_tile_kernel(TileArgs a) {
   // prefill tiles are handed out from queues, so the streaming workgroups join in when the stream is done, and
   // whichever kind of work is longer sets the time.  phase_mode 0..3 keep the static split for experiments.
   const bool queued = total_wg > 0 && a.phase_mode == 4;
-  const bool split = queued && grid_all > a.decode_grid;
-  const bool do_stream = !split || static_cast<int>(blockIdx.x) >= a.decode_grid;
-  const int stream_wg0 = split ? a.decode_grid : 0;
+  const bool split = queued && grid_all > dgrid;
+  const bool do_stream = !split || static_cast<int>(blockIdx.x) >= dgrid;
+  const int stream_wg0 = split ? dgrid : 0;
   const int stream_wgs = grid_wgs - stream_wg0;
   const int n_workers = stream_wgs * kWgWaves;
   // Workgroup b runs on XCD b % 8.  The XCDs do not stream from memory at the same rate (on MI355X the odd ones
@@ -405,7 +416,7 @@ void rpa_tile_kernel(TileArgs a) {
     const int rel = static_cast<int>(blockIdx.x) - stream_wg0, xcd = rel & 7;
     worker = (xcd & 1) * (n_workers / 2) + (((rel >> 3) * 4 + (xcd >> 1)) * kWgWaves + wave);
   }
-  const bool stream_first = total_wg > 0 && (a.phase_mode == 1 ? static_cast<int>(blockIdx.x) >= a.decode_grid
+  const bool stream_first = total_wg > 0 && (a.phase_mode == 1 ? static_cast<int>(blockIdx.x) >= dgrid
                                             : a.phase_mode == 2 ? (blockIdx.x & 1) != 0
                                             : a.phase_mode == 3 ? ((blockIdx.x >> 3) & 1) != 0
                                             : a.phase_mode == 4);
@@ -434,16 +445,21 @@ void rpa_tile_kernel(TileArgs a) {
         // the count says items are left.
         uint32_t* qctr = a.counters + kQueueCounterIndex;
         const int home = blockIdx.x & 7;
-        const int n_first = split && (total_tiles > 0 || total_items > 0) ? a.decode_grid : grid_all;  // begin with tiles
+        const int n_first = split && (total_tiles > 0 || total_items > 0) ? dgrid : grid_all;  // begin with tiles
         auto owned = [&](int x) { return n_first > x ? (n_first - x + 7) >> 3 : 0; };    // ... and have home queue x
         // items of queue x: its full runs (run r belongs to queue r % 8) and the partial last run if it is x's
         auto items_of = [&](int x) {
           const int runs = total_wg_here / kQueueRun, rem = total_wg_here - runs * kQueueRun;
           return (runs > x ? (runs - x + 7) >> 3 : 0) * kQueueRun + ((runs & 7) == x ? rem : 0);
         };
+        // Few items -- every one the first ticket of a workgroup that begins with the tiles: nobody asks a counter,
+        // nothing is left to clear, and a workgroup leaves after its tile (three microseconds of a launch of thirty).
+        bool every_item_owned = true;
+        for (int x = 0; x < 8; ++x) every_item_owned = every_item_owned && owned(x) >= items_of(x);
         int probe = 0;
         bool first = static_cast<int>(blockIdx.x) < n_first;
         while (true) {
+          if (every_item_owned && !first) break;
           // counters of the queues in this workgroup's order, read when the home queue is known to be empty
           uint32_t left = 0;  // bit k: the k-th queue in this workgroup's order has items left by its counter
           if (probe > 0 && wave == 0) {
@@ -521,7 +537,7 @@ void rpa_tile_kernel(TileArgs a) {
         }
         // The last workgroup out clears the counters for the next launch; the exit counts are kept per XCD and
         // then over the XCDs, so that the workgroups of a small batch, which all leave at once, do not queue up on one word.
-        if (tid == 0) {
+        if (tid == 0 && !every_item_owned) {
           const uint32_t n_home = (static_cast<uint32_t>(grid_all) - home + 7) >> 3;  // workgroups b with b % 8 == home
           const uint32_t gone = __hip_atomic_fetch_add(&qctr[kQueueXcdExitIndex + kQueueStride * home], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (gone == n_home - 1) {
