@@ -1001,8 +1001,11 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
                               static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs);
     // Neither flag nor hint, and the static shapes do not say "long chunks": the batch may still be one (a serving
     // caller pads total_tokens and max_num_seqs), so both kernels are enqueued and the device picks (TileArgs::select).
-    // The launch that is not picked builds the schedule and ends: a few microseconds.
-    if (pipe_choice == 0 && !pipe_wanted && pipe_ok && canonical && tune().pipe != 0 && tune().device_select != 0) {
+    // The launch that is not picked builds the schedule and ends: five microseconds, which a launch of few rows
+    // (cut_kernel: every tile starts at once on either kernel) does not get back -- it takes the 128-row tiles
+    // (the reference's benchmark shapes of 16 x 16, 16 x 32 and 32 x 16: 32.3 / 39.6 / 32.8 us picked on the device,
+    // 29.7 / 36.7 / 26.2 us on the 128-row tiles, 27.3 / 34.7 / 27.9 us on the pipelined ones).
+    if (pipe_choice == 0 && !pipe_wanted && !cut_kernel && pipe_ok && canonical && tune().pipe != 0 && tune().device_select != 0) {
       TileArgs b = a;
       a.select = 1;
       int rc = mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);
