@@ -41,12 +41,12 @@ constexpr int kQueueRun = 16;            // consecutive prefill tiles that go to
 constexpr int kSortMax = kWgThreads;      // sequences with prefill tiles that are put in order of length (one per thread)
 constexpr int kWaveOnlyMaxRows = 20480;   // (token, query head) rows up to which a batch runs without prefill tiles
 
-// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 16 ints of scratch and the sequences with prefill
+// Dynamic LDS: three schedule arrays of max_num_seqs + 1 ints, 24 ints of scratch and the sequences with prefill
 // tiles in order of length (up to kSortMax ints), then the data region
 // shared by the prefill tiles (workgroup) and the decode K tiles (one per wavefront).
 __host__ __device__ constexpr int sort_entries(int max_num_seqs) { return max_num_seqs < kSortMax ? max_num_seqs : kSortMax; }
 __host__ __device__ constexpr size_t sched_bytes(int max_num_seqs) {
-  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 16 + sort_entries(max_num_seqs)) * sizeof(int) + 15) &
+  return ((static_cast<size_t>(3) * (max_num_seqs + 1) + 24 + sort_entries(max_num_seqs)) * sizeof(int) + 15) &
          ~static_cast<size_t>(15);
 }
 
@@ -110,7 +110,7 @@ void rpa_tile_kernel(TileArgs a) {
   int* tile_start = item_start + (sched_n + 1);     // decode stream tiles
   int* wg_start = tile_start + (sched_n + 1);       // workgroup-level prefill tiles
   int* scratch = wg_start + (sched_n + 1);
-  int* wg_seq = scratch + 16;                       // sequence of the r-th entry of wg_start, when those are sorted
+  int* wg_seq = scratch + 24;                       // sequence of the r-th entry of wg_start, when those are sorted
   char* lds_data = smem + sched_bytes(sched_n);
   char* lds_k = lds_data + wave * C::LDS_PER_WAVE;
 
@@ -136,6 +136,7 @@ void rpa_tile_kernel(TileArgs a) {
   const int s_begin = min(tid * per, nseq), s_end = min(s_begin + per, nseq);
   int my_items = 0, my_tiles = 0, my_wg = 0;
   int my_cost = 0;  // TileArgs::select: prefill work in units of 1024 (query row, key) pairs, see below
+  int my_rows = 0;  // ... and its (query row, kv head)s
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
     const SeqInfo si = seq_info<C::TT>(a, s, G);
@@ -147,16 +148,25 @@ void rpa_tile_kernel(TileArgs a) {
       if ((a.select != 0 || ((kFew || kPipeTile<D, MRT>) && a.tile_split > 1)) && wg > 0) {
         const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
         my_cost += static_cast<int>(min(pairs >> 10, 1ll << 24));
+        my_rows += si.rows * p.num_kv_heads;
       }
     }
   }
   // (all four sums behind one pair of barriers: a small launch is a chain of such waits)
-  int total_items, total_tiles, total_wg, total_cost;
+  int total_items, total_tiles, total_wg, total_cost, total_rows = 0;
   int item_base, tile_base, wg_base;
-  {
+  if constexpr (!kWaveOnly && kKv == 0) {
+    const int mine[5] = {my_items, my_tiles, my_wg, my_cost, my_rows};
+    int base[5], total[5];
+    block_excl_scan_n<5>(mine, scratch, base, total);
+    item_base = base[0], tile_base = base[1], wg_base = base[2];
+    total_items = total[0], total_tiles = total[1], total_wg = total[2];
+    total_cost = __builtin_amdgcn_readfirstlane(total[3]);
+    total_rows = __builtin_amdgcn_readfirstlane(total[4]);
+  } else {
     const int mine[4] = {my_items, my_tiles, my_wg, my_cost};
     int base[4], total[4];
-    block_excl_scan4(mine, scratch, base, total);
+    block_excl_scan_n<4>(mine, scratch, base, total);
     item_base = base[0], tile_base = base[1], wg_base = base[2];
     total_items = total[0], total_tiles = total[1], total_wg = total[2];
     total_cost = __builtin_amdgcn_readfirstlane(total[3]);
@@ -195,10 +205,14 @@ void rpa_tile_kernel(TileArgs a) {
   // 1.08 against 0.92 ms).  The host sees padded shapes only, so where it cannot tell it enqueues both kernels and
   // every workgroup of both decides here, from the same sums: prefill work in units of 1024 (query row, key) pairs
   // against the stream's tiles of 32 keys -- 0.6 ns against 3 ns apiece at the rates the two kernels reach, and the
-  // pipelined tiles are worth it from seven tenths of the stream's time on.
+  // pipelined tiles are worth it from seven tenths of the stream's time on.  And from 512 keys per query row on, by the
+  // batch's average: a pipelined tile has its compute unit to itself, and what a tile costs besides its keys -- query
+  // rows, first fetches, normalising, storing, the next ticket -- is hidden by nothing, where the 128-row tiles have a
+  // second workgroup on the unit (32 to 256 chunks of 128 or 256 tokens: the 128-row tiles are 7-20 % faster with up to
+  // 450 keys per row on average, the pipelined ones 5-12 % with 770 to 900).
   if constexpr (!kWaveOnly && kKv == 0) {
     if (a.select != 0) {
-      const bool pick_pipe = 10ll * total_cost >= 35ll * total_tiles;
+      const bool pick_pipe = 10ll * total_cost >= 35ll * total_tiles && 2ll * total_cost >= total_rows;
       if ((a.select == 2) != pick_pipe) return;
     }
   }
@@ -996,8 +1010,11 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     tiled_workspace_layout(p, &wl_pipe);
     const int pipe_parts_cap = static_cast<int>(std::min<uint64_t>(wl_pipe.partial_o_bytes >> 17, wl_pipe.partial_ml_bytes >> 11));
     const int pipe_choice = pipe_choice_of(p);
+    // (block tables for fewer than 1024 keys: no batch in them averages the 512 keys per query row from which the
+    // pipelined tiles pay, see the device's pick)
+    const bool short_tables = static_cast<int64_t>(p.pages_per_seq) * p.page_size < 1024;
     const bool pipe_wanted = pipe_choice > 0 ||
-                             (pipe_choice == 0 && tune().pipe != 0 &&
+                             (pipe_choice == 0 && tune().pipe != 0 && !short_tables &&
                               static_cast<int64_t>(p.total_tokens) >= static_cast<int64_t>(tune().pipe_min_tokens_per_seq) * p.max_num_seqs);
     // Neither flag nor hint, and the static shapes do not say "long chunks": the batch may still be one (a serving
     // caller pads total_tokens and max_num_seqs), so both kernels are enqueued and the device picks (TileArgs::select).
@@ -1005,7 +1022,10 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
     // (cut_kernel: every tile starts at once on either kernel) does not get back -- it takes the 128-row tiles
     // (the reference's benchmark shapes of 16 x 16, 16 x 32 and 32 x 16: 32.3 / 39.6 / 32.8 us picked on the device,
     // 29.7 / 36.7 / 26.2 us on the 128-row tiles, 27.3 / 34.7 / 27.9 us on the pipelined ones).
-    if (pipe_choice == 0 && !pipe_wanted && !cut_kernel && pipe_ok && canonical && tune().pipe != 0 && tune().device_select != 0) {
+    // (So is a batch of a million rows and more whose shapes say "long chunks": whether they come after long contexts only the
+    // device sees, and the unpicked launch is two percent of such a batch at most.)
+    if (pipe_choice == 0 && (!pipe_wanted || rows_static >= (1ll << 20)) && !cut_kernel && !short_tables && pipe_ok && canonical &&
+        tune().pipe != 0 && tune().device_select != 0) {
       TileArgs b = a;
       a.select = 1;
       int rc = mimic ? launch_cfg<128, 2, 2, true>(a, grid, stream) : launch_cfg<128, 2, 2, false>(a, grid, stream);

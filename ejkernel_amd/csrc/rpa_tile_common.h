@@ -176,15 +176,18 @@ __device__ __forceinline__ int block_excl_scan(int v, int* wave_tot, int& total)
   return base + inc - v;
 }
 
-// Four such sums at once behind one pair of barriers (wave_tot: 4 * kWgWaves ints): v and total are arrays of four,
+// N such sums at once behind one pair of barriers (wave_tot: N * kWgWaves ints): v and total are arrays of N,
 // base receives the exclusive prefix sums.
-__device__ __forceinline__ void block_excl_scan4(const int (&v)[4], int* wave_tot, int (&base)[4], int (&total)[4]) {
+template <int N>
+__device__ __forceinline__ void block_excl_scan_n(const int (&v)[N], int* wave_tot, int (&base)[N], int (&total)[N]) {
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  int inc[4] = {v[0], v[1], v[2], v[3]};
+  int inc[N];
+#pragma unroll
+  for (int k = 0; k < N; ++k) inc[k] = v[k];
 #pragma unroll
   for (int o = 1; o < kWave; o <<= 1) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) {
+    for (int k = 0; k < N; ++k) {
       const int t = __shfl_up(inc[k], o, kWave);
       if (lane >= o) inc[k] += t;
     }
@@ -192,15 +195,15 @@ __device__ __forceinline__ void block_excl_scan4(const int (&v)[4], int* wave_to
   __syncthreads();
   if (lane == kWave - 1) {
 #pragma unroll
-    for (int k = 0; k < 4; ++k) wave_tot[4 * wave + k] = inc[k];
+    for (int k = 0; k < N; ++k) wave_tot[N * wave + k] = inc[k];
   }
   __syncthreads();
 #pragma unroll
-  for (int k = 0; k < 4; ++k) {
+  for (int k = 0; k < N; ++k) {
     int b = 0, tot = 0;
 #pragma unroll
     for (int w = 0; w < kWgWaves; ++w) {
-      const int t = wave_tot[4 * w + k];
+      const int t = wave_tot[N * w + k];
       if (w < wave) b += t;
       tot += t;
     }

@@ -12,7 +12,9 @@ mean:
                             for long chunks; above 128 = 256-row software-pipelined tiles where they exist
                             (head_dim 128, no soft cap, pages of 16 tokens or more).  None = library default
                             (wave-level loop up to 20480 (token, query head) rows, pipelined tiles from 128
-                            tokens per ``max_num_seqs``).  Results stay within the same tolerance either way.
+                            tokens per ``max_num_seqs`` with block tables for 1024 keys or more, otherwise the
+                            device picks them from 512 keys per query row on).  Results stay within the same
+                            tolerance either way.
 ``num_kv_pages_per_block``  the least stretch of a sequence, in pages, one streaming wavefront takes before a small
                             batch is spread over more wavefronts (None = 2 tiles of 32 keys, more for long sequences;
                             and a decode batch of at most 512 (sequence, kv head)s of up to 1024 keys runs one

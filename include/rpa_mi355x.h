@@ -107,7 +107,9 @@ typedef struct RpaParams {
                                   /* steps and short chunks; by default batches of up to 20480 (token, query head)   */
                                   /* rows); 17..128 = 128-row workgroup tiles for long chunks; above 128 = 256-row    */
                                   /* software-pipelined tiles where they exist (head_dim 128, no soft cap, pages of   */
-                                  /* 16 tokens or more; by default at least 128 tokens per max_num_seqs), 128-row     */
+                                  /* 16 tokens or more; by default at least 128 tokens per max_num_seqs and block     */
+                                  /* tables for 1024 keys or more; where the shapes do not say, the device picks      */
+                                  /* them from 512 keys per query row on, by the batch's average), 128-row            */
                                   /* tiles otherwise.  RPA_FLAG_PREFILL_TILES / PIPE_TILES / PLAIN_TILES come first.  */
                                   /* With few rows (total_tokens x num_q_heads up to 34816) the 128-row tiles' key     */
                                   /* ranges are cut over idle workgroups when tiles are few: one long chunk alone.     */

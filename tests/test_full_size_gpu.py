@@ -151,7 +151,8 @@ def test_tile_kernel_is_picked_on_the_device_where_the_host_cannot_tell():
     """Static shapes that say nothing about the batch (many rows, few tokens per max_num_seqs, no flag, no hint): both
     tile kernels are enqueued and the device picks one from the lengths.  A batch whose prefill work outweighs its
     decode stream must come out bit for bit as the pipelined tiles give it, one whose stream outweighs the chunks as
-    the 128-row tiles do; and the pair of launches replays from a HIP graph on new queries."""
+    the 128-row tiles do, and so must one of short chunks (fewer than 512 keys per query row on average: a pipelined
+    tile's fixed costs are hidden by nothing); and the pair of launches replays from a HIP graph on new queries."""
     from ejkernel_amd import _native
     from ejkernel_amd.modules.operations import RaggedPageAttention, RaggedPageAttentionConfig
     from ejkernel_amd.workloads import make_batch
@@ -167,8 +168,10 @@ def test_tile_kernel_is_picked_on_the_device_where_the_host_cannot_tell():
                         num_kv_heads=8, head_dim=128, page_size=32, pages_per_seq=128, seed=51, device=DEV, max_num_seqs=64)
     stream = make_batch([600] + [1] * 60, [900] + list(rng.integers(3000, 4096, size=60)), num_q_heads=32, num_kv_heads=8,
                         head_dim=128, page_size=32, pages_per_seq=128, seed=52, device=DEV, max_num_seqs=64)
+    short = make_batch([200] * 16, [200] * 12 + [500] * 4, num_q_heads=32, num_kv_heads=8, head_dim=128, page_size=32,
+                       pages_per_seq=128, seed=53, device=DEV, max_num_seqs=64)
     pipe, plain = _native.RPA_FLAG_PIPE_TILES, _native.RPA_FLAG_PREFILL_TILES | _native.RPA_FLAG_PLAIN_TILES
-    for b, picked, other in ((chunks, pipe, plain), (stream, plain, pipe)):
+    for b, picked, other in ((chunks, pipe, plain), (stream, plain, pipe), (short, plain, pipe)):
         assert b.queries.shape[0] * 32 > 20480 and b.queries.shape[0] < 128 * 64   # no rule of the host's applies
         out = run_flags(b, 0)
         assert torch.equal(out, run_flags(b, picked))
