@@ -958,12 +958,14 @@ static int launch_tiled_impl(const RpaParams& p, const KvLayout& kv, hipStream_t
   // 57 us, 107 against 287 us after 8192 tokens; a chunk with no context at all loses a tenth (32 against 29 us).
   // The same holds for a chunk beside a few decode steps (512 tokens after 8192 with 64 decode steps: 392 us on the
   // wave-level loop, 244 on the tiles): where the rows are few, the token count says that some sequence has hundreds of
-  // tokens (224 more tokens than sequences) and the block tables are laid out for long contexts (4096 keys or more --
-  // with short ones the wave-level loop is the faster by a tenth or two), the tiles are taken as well.
+  // tokens (224 more tokens than sequences) and the block tables are laid out for long contexts (2048 keys or more --
+  // with short ones the wave-level loop is the faster by a tenth or two), the tiles are taken as well.  (Small batches
+  // of chunks over heads, lengths and contexts: after up to 1024 keys the two are within a tenth of each other, 16.6
+  // against 19.0 us from scratch; after 2048 to 3000 the tiles take 56 us where the wave-level loop takes 73 to 96.)
   const int64_t rows_static = static_cast<int64_t>(p.total_tokens) * p.num_q_heads;
   const bool long_chunks_by_shape = static_cast<int64_t>(p.total_tokens) >= 256ll * p.max_num_seqs ||
                                     (static_cast<int64_t>(p.total_tokens) - p.max_num_seqs >= 224 &&
-                                     static_cast<int64_t>(p.pages_per_seq) * p.page_size >= 4096);
+                                     static_cast<int64_t>(p.pages_per_seq) * p.page_size >= 2048);
   const bool few_long_chunks = p.query_start_loc != nullptr && !tiles_flagged(p) && p.num_queries_per_block <= 0 &&
                                a.tile_split > 1 && tune().no_wave_only == 0 && long_chunks_by_shape &&
                                rows_static <= 32768 + 2048;
