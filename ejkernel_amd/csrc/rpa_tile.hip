@@ -137,6 +137,7 @@ void rpa_tile_kernel(TileArgs a) {
   int my_items = 0, my_tiles = 0, my_wg = 0;
   int my_cost = 0;  // TileArgs::select: prefill work in units of 1024 (query row, key) pairs, see below
   int my_rows = 0;  // ... and its (query row, kv head)s
+  int my_kv_len = 0;  // length of this thread's last sequence (the sort below: a thread with one sequence need not read it again)
   for (int s = s_begin; s < s_end; ++s) {
     int t, it, wg;
     const SeqInfo si = seq_info<C::TT>(a, s, G);
@@ -144,6 +145,7 @@ void rpa_tile_kernel(TileArgs a) {
     my_tiles += t;
     my_items += it;
     my_wg += wg;
+    my_kv_len = si.kv_len;
     if constexpr (!kWaveOnly && kKv == 0) {
       if ((a.select != 0 || ((kFew || kPipeTile<D, MRT>) && a.tile_split > 1)) && wg > 0) {
         const long long pairs = static_cast<long long>(si.rows) * p.num_kv_heads * max(si.kv_len - si.q_len / 2, 1);
@@ -266,8 +268,11 @@ void rpa_tile_kernel(TileArgs a) {
     const int begin_with_tiles = static_cast<int>(gridDim.x) > dgrid && (total_tiles > 0 || total_items > 0)
                                      ? dgrid : static_cast<int>(gridDim.x);
     if (total_wg > begin_with_tiles && shift == 0 && a.phase_mode == 4) {
-      int mine = 0;
-      for (int s = s_begin; s < s_end; ++s) {
+      // (a thread with one sequence -- every thread of a batch of up to 256 -- has its numbers from the first pass:
+      // reading the lengths again is two round trips to memory, two microseconds of a launch of a hundred)
+      const bool one = s_end - s_begin <= 1;
+      int mine = one ? (my_wg > 0) : 0;
+      for (int s = s_begin; s < s_end && !one; ++s) {
         int t, it, wg;
         classify(seq_info<C::TT>(a, s, G), t, it, wg);
         mine += wg > 0;
@@ -280,7 +285,12 @@ void rpa_tile_kernel(TileArgs a) {
         int* t_key = t_seq + kSortMax;
         int* t_cnt = t_key + kSortMax;
         int* o_cnt = t_cnt + kSortMax;
-        for (int s = s_begin; s < s_end; ++s) {
+        if (one && my_wg > 0) {
+          t_seq[at] = s_begin;
+          t_key[at] = my_kv_len;
+          t_cnt[at] = my_wg;
+        }
+        for (int s = s_begin; s < s_end && !one; ++s) {
           int t, it, wg;
           const SeqInfo si = seq_info<C::TT>(a, s, G);
           classify(si, t, it, wg);
